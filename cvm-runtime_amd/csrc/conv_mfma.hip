@@ -1,0 +1,496 @@
+// conv2d / dense on gfx950 as an exact int8 x int8 -> int32 implicit GEMM.
+//
+//   D[oc][px] = sum_k Wp[oc][k] * Xcol[px][k],   k = (kh, kw, c),  px = (n, oh, ow)
+//
+// Data layout
+//   Xp : int8 NHWC activations, channels padded to Cp (4, 8 or a multiple of 16)
+//   Wp : int8 [OCp][Kp] filter rows, k ordered (kh, kw, c) with c padded to Cp,
+//        Kp = K rounded up to 64, OCp = OC rounded up to 128; padding is zero
+//   D  : int32 NCHW (the operator contract) or int8 NHWC (fused requantised output)
+//
+// One workgroup = 4 wavefronts (2 x 2) and computes a (64*WM) x (64*WN) tile of
+// D with v_mfma_i32_32x32x32_i8.  Each K step stages a 64-byte slab of both
+// operands in LDS (row pitch 80 B so the 16-byte MFMA operand reads of 8
+// consecutive lanes hit disjoint banks); the im2col addressing happens while
+// the slab is fetched, so no column buffer ever exists in HBM.  Global fetches
+// for step t+1 are issued before the MFMAs of step t and land in the other LDS
+// buffer (one barrier per step).
+#include "conv_mfma.h"
+
+namespace cvmhip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int KSTEP = 64;   // bytes of K per LDS slab
+constexpr int LDK = 80;     // LDS row pitch in bytes
+
+__device__ __forceinline__ int4 zero4() { return make_int4(0, 0, 0, 0); }
+
+// Fetch the 16 consecutive k-bytes [kk, kk+16) of one im2col row.
+// G = bytes that are contiguous in memory for one filter tap (16 when Cp % 16 == 0,
+// else Cp itself, which is then 4 or 8).
+template <int G>
+__device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const ConvGeom& g, bool row_ok,
+                                          int64_t img_base, int ih0, int iw0, int tap, int r, int s, int c0) {
+  if (G == 16) {
+    const int ih = ih0 + r * g.DH, iw = iw0 + s * g.DW;
+    if (row_ok && tap < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+      return *reinterpret_cast<const int4*>(xp + img_base + ((int64_t)ih * g.W + iw) * g.Cp + c0);
+    return zero4();
+  } else {
+    // Cp == G: each granule is a whole tap
+    int v[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16 / G; ++j) {
+      const int t = tap + j;
+      const int rr = t / g.KW, ss = t - rr * g.KW;
+      const int ih = ih0 + rr * g.DH, iw = iw0 + ss * g.DW;
+      if (row_ok && t < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W) {
+        const int8_t* p = xp + img_base + ((int64_t)ih * g.W + iw) * g.Cp;
+        if (G == 4) {
+          v[j] = *reinterpret_cast<const int*>(p);
+        } else {
+          const int2 u = *reinterpret_cast<const int2*>(p);
+          v[2 * j] = u.x;
+          v[2 * j + 1] = u.y;
+        }
+      }
+    }
+    return make_int4(v[0], v[1], v[2], v[3]);
+  }
+}
+
+__device__ __forceinline__ int32_t requant(const Epilogue& ep, int32_t v, int oc) {
+  if (ep.bias) v = wadd(v, ep.bias[oc]);
+  if (ep.relu) v = v < 0 ? 0 : v;
+  if (ep.has_shift) v = apply_rshift(ep.rs, v);
+  if (ep.has_clip) v = v > ep.chi ? ep.chi : (v < ep.clo ? ep.clo : v);
+  return v;
+}
+
+template <int WM, int WN, int G>
+__global__ void __launch_bounds__(256)
+k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void* __restrict__ out,
+             const ConvGeom g, const Epilogue ep) {
+  constexpr int BM = 64 * WM;  // output channels per workgroup
+  constexpr int BN = 64 * WN;  // output pixels per workgroup
+  __shared__ __attribute__((aligned(16))) int8_t sA[2][BM * LDK];
+  __shared__ __attribute__((aligned(16))) int8_t sB[2][BN * LDK];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so
+  // give each XCD a contiguous run of tiles (neighbouring tiles share the
+  // activation slab in that XCD's L2).
+  int pid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);
+  const int oc_tiles = (g.OC + BM - 1) / BM;
+  const int oc0 = (pid % oc_tiles) * BM;
+  const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
+
+  // ---- per-thread fetch assignment: chunk column kc (16 B of the 64 B slab),
+  // rows tid/4 + 64*i
+  const int kc = tid & 3;
+  const int frow = tid >> 2;
+  const int OHW = g.OH * g.OW;
+  bool row_ok[WN];
+  int64_t img_base[WN];
+  int ih0[WN], iw0[WN];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) {
+    const int64_t p = px0 + frow + 64 * i;
+    row_ok[i] = p < g.P;
+    const int64_t pp = row_ok[i] ? p : 0;
+    const int n = (int)(pp / OHW);
+    const int rem = (int)(pp - (int64_t)n * OHW);
+    const int oh = rem / g.OW, ow = rem - oh * g.OW;
+    img_base[i] = (int64_t)n * g.H * g.W * g.Cp;
+    ih0[i] = oh * g.SH - g.PH;
+    iw0[i] = ow * g.SW - g.PW;
+  }
+  const int8_t* wrow[WM];
+#pragma unroll
+  for (int i = 0; i < WM; ++i) wrow[i] = wp + (int64_t)(oc0 + frow + 64 * i) * g.Kp + kc * 16;
+
+  // position of this thread's chunk inside the (tap, channel) space
+  int kk = kc * 16;
+  int tap = kk / g.Cp, c0 = kk - tap * g.Cp;
+  int r = tap / g.KW, s = tap - r * g.KW;
+
+  v16i acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  int4 ra[WM], rb[WN];
+  const int nk = g.Kp / KSTEP;
+
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) ra[i] = *reinterpret_cast<const int4*>(wrow[i] + (int64_t)kt * KSTEP);
+#pragma unroll
+    for (int i = 0; i < WN; ++i) rb[i] = fetch_act<G>(xp, g, row_ok[i], img_base[i], ih0[i], iw0[i], tap, r, s, c0);
+    // advance (tap, c0) by one K step
+    if (G == 16) {
+      c0 += KSTEP;
+      while (c0 >= g.Cp) {
+        c0 -= g.Cp;
+        ++tap;
+        if (++s == g.KW) { s = 0; ++r; }
+      }
+    } else {
+      tap += KSTEP / G;
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) *reinterpret_cast<int4*>(&sA[buf][(frow + 64 * i) * LDK + kc * 16]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < WN; ++i) *reinterpret_cast<int4*>(&sB[buf][(frow + 64 * i) * LDK + kc * 16]) = rb[i];
+  };
+
+  fetch(0);
+  stage(0);
+  __syncthreads();
+
+  const int lrow = lane & 31;
+  const int lgrp = lane >> 5;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) fetch(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      v4i a[WM], b[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        a[i] = *reinterpret_cast<const v4i*>(&sA[cur][((wm * WM + i) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        b[j] = *reinterpret_cast<const v4i*>(&sB[cur][((wn * WN + j) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) stage(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue.  Accumulator element e of lane l in a 32x32 tile is
+  // row (e/4)*8 + (l/32)*4 + e%4 (output channel), column l%32 (pixel).
+#pragma unroll
+  for (int j = 0; j < WN; ++j) {
+    const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
+    if (p >= g.P) continue;
+    const int n = (int)(p / OHW);
+    const int rem = (int)(p - (int64_t)n * OHW);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int ocb = oc0 + (wm * WM + i) * 32 + lgrp * 4;
+      if (ep.out_mode == OUT_I32_NCHW) {
+        int32_t* y = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int oc = ocb + (e >> 2) * 8 + (e & 3);
+          if (oc < g.OC) y[(int64_t)oc * OHW] = requant(ep, acc[i][j][e], oc);
+        }
+      } else {  // OUT_I8_NHWC: 4 consecutive channels -> one 32-bit store
+        int8_t* y = reinterpret_cast<int8_t*>(out) + p * ep.out_cp;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int oc = ocb + q * 8;
+          if (oc >= ep.out_cp) continue;
+          uint32_t pack = 0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int32_t v = (oc + e < g.OC) ? requant(ep, acc[i][j][q * 4 + e], oc + e) : 0;
+            pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * e);
+          }
+          *reinterpret_cast<uint32_t*>(y + oc) = pack;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- packing
+// int32 NCHW -> int8 NHWC (channels padded to cp with zeros); narrowing is
+// static_cast<int8_t>, the reference's own (ops.cc:234).
+__global__ void __launch_bounds__(256) k_pack_nhwc(const int32_t* __restrict__ x, int8_t* __restrict__ xp, int64_t total,
+                                                   int c, int hw, int cp) {
+  const int c4n = cp / 4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int pix = (int)(i % hw);
+    const int64_t t = i / hw;
+    const int c4 = (int)(t % c4n);
+    const int64_t n = t / c4n;
+    uint32_t pack = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int ch = c4 * 4 + j;
+      const int32_t v = ch < c ? x[((int64_t)n * c + ch) * hw + pix] : 0;
+      pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
+    }
+    *reinterpret_cast<uint32_t*>(xp + ((int64_t)n * hw + pix) * cp + c4 * 4) = pack;
+  }
+}
+
+// int32 OIHW -> int8 [OCp][Kp], k = (r*KW + s)*Cp + c, zero padded
+__global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict__ w, int8_t* __restrict__ wp, int64_t total,
+                                                      int oc, int ic, int taps, int cp, int kp) {
+  const int k4n = kp / 4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int k4 = (int)(i % k4n);
+    const int64_t o = i / k4n;
+    const int k = k4 * 4;
+    const int tap = k / cp, c = k - tap * cp;
+    uint32_t pack = 0;
+    if (o < oc && tap < taps) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int32_t v = (c + j < ic) ? w[((int64_t)o * ic + c + j) * taps + tap] : 0;
+        pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
+      }
+    }
+    *reinterpret_cast<uint32_t*>(wp + o * kp + k) = pack;
+  }
+}
+
+// int8 NHWC (padded to cp) -> int32 NCHW
+__global__ void __launch_bounds__(256) k_unpack_nchw(const int8_t* __restrict__ xp, int32_t* __restrict__ x, int64_t total,
+                                                     int c, int hw, int cp) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int pix = (int)(i % hw);
+    const int64_t t = i / hw;
+    const int ch = (int)(t % c);
+    const int64_t n = t / c;
+    x[i] = xp[((int64_t)n * hw + pix) * cp + ch];
+  }
+}
+
+// ---------------------------------------------------------------- exact int32 paths
+// groups > 1 (incl. depthwise): direct convolution on the int32 values, no
+// narrowing -- what the reference does for grouped filters (ops.cc:333-366).
+__global__ void __launch_bounds__(256)
+k_conv_grouped(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const int32_t* __restrict__ bias,
+               int32_t* __restrict__ y, int64_t total, int ic, int h, int wd, int oc, int oh, int ow, int kh, int kw,
+               int sh, int sw, int ph, int pw, int dh, int dw, int icg, int ocg) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int q = (int)(i % ow);
+    const int p = (int)((i / ow) % oh);
+    const int o = (int)((i / ((int64_t)ow * oh)) % oc);
+    const int64_t b = i / ((int64_t)ow * oh * oc);
+    const int cbase = (o / ocg) * icg;
+    int32_t acc = 0;
+    for (int c = 0; c < icg; ++c) {
+      const int32_t* xc = x + ((int64_t)b * ic + cbase + c) * h * wd;
+      const int32_t* wc = w + ((int64_t)o * icg + c) * kh * kw;
+      for (int r = 0; r < kh; ++r) {
+        const int ih = p * sh + r * dh - ph;
+        if (ih < 0 || ih >= h) continue;
+        for (int t = 0; t < kw; ++t) {
+          const int iw = q * sw + t * dw - pw;
+          if (iw < 0 || iw >= wd) continue;
+          acc = wadd(acc, wmul(xc[(int64_t)ih * wd + iw], wc[r * kw + t]));
+        }
+      }
+    }
+    y[i] = wadd(acc, bias ? bias[o] : 0);
+  }
+}
+
+// dense on int32 operands without narrowing: one wavefront per output element.
+__global__ void __launch_bounds__(256)
+k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const int32_t* __restrict__ bias,
+            int32_t* __restrict__ y, int64_t total, int k, int n) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  for (int64_t o = wave; o < total; o += nwaves) {
+    const int64_t m = o / n;
+    const int j = (int)(o - m * n);
+    const int32_t* xr = x + m * k;
+    const int32_t* wr = w + (int64_t)j * k;
+    int32_t acc = 0;
+    for (int t = lane; t < k; t += 64) acc = wadd(acc, wmul(xr[t], wr[t]));
+    for (int d = 32; d >= 1; d >>= 1) acc = wadd(acc, __shfl_xor(acc, d, 64));
+    if (lane == 0) y[o] = wadd(acc, bias ? bias[j] : 0);
+  }
+}
+
+// ---------------------------------------------------------------- host side
+int pad_channels(int c) {
+  if (c <= 4) return 4;
+  if (c <= 8) return 8;
+  return (c + 15) / 16 * 16;
+}
+
+size_t packed_act_bytes(int64_t npix, int c) { return ((size_t)npix * pad_channels(c) + 255) / 256 * 256; }
+
+void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp) {
+  const int cp = pad_channels(ic);
+  *kp = (kh * kw * cp + KSTEP - 1) / KSTEP * KSTEP;
+  *ocp = (oc + 127) / 128 * 128;
+}
+
+size_t packed_weight_bytes(int oc, int ic, int kh, int kw) {
+  int ocp, kp;
+  weight_dims(oc, ic, kh, kw, &ocp, &kp);
+  return ((size_t)ocp * kp + 255) / 256 * 256;
+}
+
+int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStream_t s) {
+  const int cp = pad_channels(c);
+  const int64_t total = (int64_t)n * (cp / 4) * hw;
+  if (total == 0) return CVMHIP_OK;
+  k_pack_nhwc<<<grid_for(total, 256), 256, 0, s>>>(x, xp, total, c, hw, cp);
+  return check_launch("pack_nhwc");
+}
+
+int unpack_activations(const int8_t* xp, int32_t* x, int n, int c, int hw, hipStream_t s) {
+  const int64_t total = (int64_t)n * c * hw;
+  if (total == 0) return CVMHIP_OK;
+  k_unpack_nchw<<<grid_for(total, 256), 256, 0, s>>>(xp, x, total, c, hw, pad_channels(c));
+  return check_launch("unpack_nchw");
+}
+
+int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, hipStream_t s) {
+  int ocp, kp;
+  weight_dims(oc, ic, kh, kw, &ocp, &kp);
+  const int64_t total = (int64_t)ocp * (kp / 4);
+  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, ic, kh * kw, pad_channels(ic), kp);
+  return check_launch("pack_weights");
+}
+
+template <int WM, int WN>
+static void launch_tile(int gran, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+                        const ConvGeom& g, const Epilogue& ep) {
+  if (gran == 16) k_conv_igemm<WM, WN, 16><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  else if (gran == 8) k_conv_igemm<WM, WN, 8><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  else k_conv_igemm<WM, WN, 4><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+}
+
+int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, hipStream_t s) {
+  if (g.N < 1 || g.H < 1 || g.W < 1 || g.OC < 1 || g.OH < 1 || g.OW < 1 || g.KH < 1 || g.KW < 1 || g.SH < 1 ||
+      g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
+    return arg_error("conv geometry");
+  if (g.Cp != 4 && g.Cp != 8 && (g.Cp % 16) != 0) return arg_error("conv channel padding");
+  if (((uintptr_t)xp | (uintptr_t)wp) & 15) return arg_error("conv operand alignment");
+  if (ep.out_mode == OUT_I8_NHWC && (ep.out_cp % 4 != 0 || ep.out_cp < g.OC || ((uintptr_t)out & 3)))
+    return arg_error("conv int8 output layout");
+  g.taps = g.KH * g.KW;
+  g.K = g.taps * g.Cp;
+  g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
+  g.P = (int64_t)g.N * g.OH * g.OW;
+  const int gran = g.Cp >= 16 ? 16 : g.Cp;
+  // Tile choice: the largest tile that still yields >= 2 workgroups per CU;
+  // small layers fall back to smaller tiles to keep all 256 CUs busy.
+  auto blocks = [&](int bm, int bn) { return (int64_t)((g.OC + bm - 1) / bm) * ((g.P + bn - 1) / bn); };
+  int wm = g.OC > 64 ? 2 : 1, wn = 2;
+  if (blocks(64 * wm, 64 * wn) < 512 && wn == 2) wn = 1;
+  if (blocks(64 * wm, 64 * wn) < 512 && wm == 2) wm = 1;
+  const int64_t nb = blocks(64 * wm, 64 * wn);
+  if (nb > 0x7fffffff) return arg_error("conv grid too large");
+  const unsigned grid = (unsigned)nb;
+  if (wm == 2 && wn == 2) launch_tile<2, 2>(gran, grid, s, xp, wp, out, g, ep);
+  else if (wm == 1 && wn == 2) launch_tile<1, 2>(gran, grid, s, xp, wp, out, g, ep);
+  else if (wm == 2 && wn == 1) launch_tile<2, 1>(gran, grid, s, xp, wp, out, g, ep);
+  else launch_tile<1, 1>(gran, grid, s, xp, wp, out, g, ep);
+  return check_launch("conv_igemm");
+}
+
+}  // namespace cvmhip
+
+using namespace cvmhip;
+
+extern "C" {
+
+size_t cvmhip_conv2d_workspace_bytes(int n, int ic, int h, int w, int oc, int kh, int kw, int groups) {
+  if (groups != 1) return 0;
+  return packed_act_bytes((int64_t)n * h * w, ic) + packed_weight_bytes(oc, ic, kh, kw);
+}
+
+int cvmhip_conv2d(const int32_t* x, const int32_t* w, const int32_t* bias, int32_t* y,
+                  int n, int ic, int h, int wd, int oc, int kh, int kw,
+                  int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                  int groups, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !w || !y) return arg_error("conv2d null tensor");
+  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1 || groups < 1 || ic % groups || oc % groups)
+    return arg_error("conv2d attributes");
+  const int oh = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  const int ow = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1) return arg_error("conv2d kernel exceeds input");
+  hipStream_t s = as_stream(stream);
+  if (groups > 1) {
+    const int64_t total = (int64_t)n * oc * oh * ow;
+    k_conv_grouped<<<grid_for(total, 256, 1 << 20), 256, 0, s>>>(x, w, bias, y, total, ic, h, wd, oc, oh, ow, kh, kw,
+                                                               stride_h, stride_w, pad_h, pad_w, dil_h, dil_w,
+                                                               ic / groups, oc / groups);
+    return check_launch("conv_grouped");
+  }
+  const size_t need = cvmhip_conv2d_workspace_bytes(n, ic, h, wd, oc, kh, kw, 1);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return arg_error("conv2d workspace");
+  int8_t* xp = reinterpret_cast<int8_t*>(workspace);
+  int8_t* wp = xp + packed_act_bytes((int64_t)n * h * wd, ic);
+  int rc = pack_activations(x, xp, n, ic, h * wd, s);
+  if (rc) return rc;
+  rc = pack_weights(w, wp, oc, ic, kh, kw, s);
+  if (rc) return rc;
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic);
+  g.OC = oc; g.OH = oh; g.OW = ow;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  Epilogue ep = {};
+  ep.bias = bias;
+  ep.out_mode = OUT_I32_NCHW;
+  return conv_igemm(xp, wp, y, g, ep, s);
+}
+
+size_t cvmhip_dense_workspace_bytes(int m, int k, int n) {
+  return packed_act_bytes(m, k) + packed_weight_bytes(n, k, 1, 1);
+}
+
+int cvmhip_dense(const int32_t* x, const int32_t* w, const int32_t* bias, int32_t* y,
+                 int m, int k, int n, int operand_bits,
+                 void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !w || !y || m < 1 || k < 1 || n < 1) return arg_error("dense");
+  hipStream_t s = as_stream(stream);
+  if (operand_bits > 8) {
+    const int64_t total = (int64_t)m * n;
+    k_dense_i32<<<grid_for(total * 64, 256, 1 << 20), 256, 0, s>>>(x, w, bias, y, total, k, n);
+    return check_launch("dense_i32");
+  }
+  const size_t need = cvmhip_dense_workspace_bytes(m, k, n);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return arg_error("dense workspace");
+  // x[m][k] is already "NHWC" with one pixel per row; the filter is OC x K x 1 x 1
+  int8_t* xp = reinterpret_cast<int8_t*>(workspace);
+  int8_t* wp = xp + packed_act_bytes(m, k);
+  int rc = pack_activations(x, xp, m, k, 1, s);
+  if (rc) return rc;
+  rc = pack_weights(w, wp, n, k, 1, 1, s);
+  if (rc) return rc;
+  ConvGeom g = {};
+  g.N = m; g.H = 1; g.W = 1; g.Cp = pad_channels(k);
+  g.OC = n; g.OH = 1; g.OW = 1;
+  g.KH = g.KW = g.SH = g.SW = g.DH = g.DW = 1;
+  Epilogue ep = {};
+  ep.bias = bias;
+  ep.out_mode = OUT_I32_NCHW;
+  return conv_igemm(xp, wp, y, g, ep, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,275 @@
+// get_valid_counts and non_max_suppression for gfx950.
+//
+// Both are order-sensitive on the CPU; here the order is reproduced with
+// wavefront ballots / prefix sums (stream compaction) and a rank sort whose key
+// (score descending, original index ascending) is unique, so the result does
+// not depend on scheduling.  Nothing is copied back to the host: valid_count is
+// read on the device and every launch shape depends only on (batches, n, k).
+#include "hip_common.h"
+
+namespace cvmhip {
+
+constexpr int GVC_CHUNK = 256;
+
+// number of rows in this 256-row chunk whose score passes the threshold
+__global__ void __launch_bounds__(GVC_CHUNK)
+k_gvc_count(const int32_t* __restrict__ x, int32_t* __restrict__ counts, int n, int k, int32_t thr, int nchunks) {
+  __shared__ int wsum[GVC_CHUNK / 64];
+  const int b = blockIdx.y, chunk = blockIdx.x;
+  const int row = chunk * GVC_CHUNK + threadIdx.x;
+  const bool keep = row < n && x[((int64_t)b * n + row) * k + 1] > thr;
+  const unsigned long long m = __ballot(keep);
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = __popcll(m);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int t = 0;
+    for (int i = 0; i < GVC_CHUNK / 64; ++i) t += wsum[i];
+    counts[b * nchunks + chunk] = t;
+  }
+}
+
+// Each chunk derives its output offset from the counts of the chunks before it,
+// then places its surviving rows in their original order; rows at or past the
+// batch total are filled with -1.
+__global__ void __launch_bounds__(GVC_CHUNK)
+k_gvc_scatter(const int32_t* __restrict__ x, const int32_t* __restrict__ counts, int32_t* __restrict__ valid_count,
+              int32_t* __restrict__ y, int n, int k, int32_t thr, int nchunks) {
+  __shared__ int wsum[GVC_CHUNK / 64];
+  __shared__ int s_before, s_total;
+  const int b = blockIdx.y, chunk = blockIdx.x;
+  if (threadIdx.x == 0) {
+    int before = 0, total = 0;
+    for (int c = 0; c < nchunks; ++c) {
+      const int v = counts[b * nchunks + c];
+      if (c < chunk) before += v;
+      total += v;
+    }
+    s_before = before;
+    s_total = total;
+    if (chunk == 0) valid_count[b] = total;
+  }
+  const int row = chunk * GVC_CHUNK + threadIdx.x;
+  const int32_t* src = x + ((int64_t)b * n + row) * k;
+  const bool keep = row < n && src[1] > thr;
+  const unsigned long long m = __ballot(keep);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int in_wave = __popcll(m & ((1ull << lane) - 1ull));
+  if (lane == 0) wsum[wv] = __popcll(m);
+  __syncthreads();
+  int pos = s_before + in_wave;
+  for (int i = 0; i < wv; ++i) pos += wsum[i];
+  int32_t* yb = y + (int64_t)b * n * k;
+  if (keep)
+    for (int c = 0; c < k; ++c) yb[(int64_t)pos * k + c] = src[c];
+  if (row < n && row >= s_total)
+    for (int c = 0; c < k; ++c) yb[(int64_t)row * k + c] = -1;
+}
+
+// ------------------------------------------------------------------ NMS
+// int64 IoU*100 of two corner-format boxes, same arithmetic as the reference
+// (src/runtime/cpu/ops/nms.cc:4-40).
+__device__ __forceinline__ int64_t iou100(const int32_t* r1, const int32_t* r2) {
+  const int64_t a1 = (int64_t)wsub(r1[2], r1[0]) * wsub(r1[3], r1[1]);
+  const int64_t a2 = (int64_t)wsub(r2[2], r2[0]) * wsub(r2[3], r2[1]);
+  const int64_t sum_area = (int64_t)((uint64_t)a1 + (uint64_t)a2);
+  if (sum_area <= 0) return 0;
+  const int32_t xr = r1[2] < r2[2] ? r1[2] : r2[2], xl = r1[0] > r2[0] ? r1[0] : r2[0];
+  const int32_t yb = r1[3] < r2[3] ? r1[3] : r2[3], yt = r1[1] > r2[1] ? r1[1] : r2[1];
+  int32_t w = wsub(xr, xl), h = wsub(yb, yt);
+  if (w < 0) w = 0;
+  if (h < 0) h = 0;
+  int64_t overlap = (int64_t)h * w;
+  int64_t uni = sum_area - overlap;
+  if (uni <= 0) return 0;
+  if (INT64_MAX / 100 < overlap) uni /= 100; else overlap *= 100;
+  return overlap / uni;
+}
+
+__device__ __forceinline__ int clamp_vc(int vc, int n) { return vc > n ? n : (vc < 0 ? 0 : vc); }
+
+// The reference returns from the whole call at the first batch without valid
+// rows (nms.cc:76-79): that batch is filled with -1 and later batches are left
+// untouched.  0 = process normally, 1 = this is that batch, 2 = skipped.
+__device__ __forceinline__ int batch_state(const int32_t* valid_count, int b, int n) {
+  for (int i = 0; i < b; ++i)
+    if (clamp_vc(valid_count[i], n) <= 0) return 2;
+  return clamp_vc(valid_count[b], n) <= 0 ? 1 : 0;
+}
+
+// Rank of row i among the first vc rows under (score descending, index
+// ascending) -- the order std::stable_sort gives (nms.cc:89-91).
+// Also gathers the row into its sorted slot.
+__global__ void __launch_bounds__(256)
+k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ order,
+           int32_t* __restrict__ sorted, int n, int k, int score_index, int64_t ws_stride) {
+  __shared__ int32_t tile[256];
+  const int b = blockIdx.y;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (blockIdx.x * 256 >= vc) return;
+  const int32_t* xb = x + (int64_t)b * n * k;
+  const int32_t si = i < vc ? xb[(int64_t)i * k + score_index] : 0;
+  int rank = 0;
+  for (int base = 0; base < vc; base += 256) {
+    const int j = base + threadIdx.x;
+    __syncthreads();
+    tile[threadIdx.x] = j < vc ? xb[(int64_t)j * k + score_index] : INT32_MIN;
+    __syncthreads();
+    const int lim = vc - base < 256 ? vc - base : 256;
+    for (int t = 0; t < lim; ++t) {
+      const int32_t sj = tile[t];
+      rank += (sj > si) || (sj == si && base + t < i);
+    }
+  }
+  if (i < vc) {
+    order[b * ws_stride + rank] = i;
+    int32_t* dst = sorted + b * ws_stride * k + (int64_t)rank * k;
+    for (int c = 0; c < k; ++c) dst[c] = xb[(int64_t)i * k + c];
+  }
+}
+
+constexpr int NMS_THREADS = 1024;
+
+// One workgroup per batch walks the sorted rows in order.  Row i is emitted if
+// it survived and has id >= 0; a surviving row then suppresses, in parallel,
+// the rows after it up to (not including) the first row with a negative id.
+__global__ void __launch_bounds__(NMS_THREADS)
+k_nms_select(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ y,
+             const int32_t* __restrict__ order, const int32_t* __restrict__ sorted, int32_t* __restrict__ nextneg,
+             int32_t* __restrict__ removed, int n, int k, int max_output_size, int iou_threshold, int topk,
+             int coord_start, int id_index, int force_suppress, int64_t ws_stride) {
+  __shared__ int s_wmin[NMS_THREADS / 64];
+  __shared__ int s_carry;
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int state = batch_state(valid_count, b, n);
+  if (state == 2) return;
+  int32_t* yb = y + (int64_t)b * n * k;
+  if (state == 1) {
+    for (int64_t i = tid; i < (int64_t)n * k; i += NMS_THREADS) yb[i] = -1;
+    return;
+  }
+  const int vc = clamp_vc(valid_count[b], n);
+  int32_t* xb = x + (int64_t)b * n * k;
+  const int32_t* ord = order + b * ws_stride;
+  const int32_t* srt = sorted + b * ws_stride * k;
+  int32_t* nn = nextneg + b * (ws_stride + 1);
+  int32_t* rem = removed + b * ws_stride;
+  const int keep = (topk >= 0 && topk < vc) ? topk : vc;
+
+  // rows past top_k are overwritten with -1 in the input tensor (nms.cc:92-96)
+  if (topk > 0 && topk < vc)
+    for (int64_t i = tid; i < (int64_t)(vc - topk) * k; i += NMS_THREADS) {
+      const int r = topk + (int)(i / k);
+      xb[(int64_t)ord[r] * k + (i % k)] = -1;
+    }
+
+  // nn[j] = smallest j' >= j with a negative id (keep if none): suffix minimum,
+  // computed chunk by chunk from the back.
+  if (tid == 0) { s_carry = keep; nn[keep] = keep; }
+  for (int i = tid; i < keep; i += NMS_THREADS) rem[i] = 0;
+  __syncthreads();
+  for (int base = ((keep - 1) / NMS_THREADS) * NMS_THREADS; base >= 0 && keep > 0; base -= NMS_THREADS) {
+    const int j = base + tid;
+    int v = (j < keep && srt[(int64_t)j * k] < 0) ? j : keep;
+    // inclusive suffix-min inside the wavefront
+    const int lane = tid & 63, wv = tid >> 6;
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_down(v, d, 64);
+      if (lane + d < 64) v = o < v ? o : v;
+    }
+    if (lane == 0) s_wmin[wv] = v;
+    __syncthreads();
+    int later = s_carry;
+    for (int w = wv + 1; w < NMS_THREADS / 64; ++w) later = s_wmin[w] < later ? s_wmin[w] : later;
+    v = later < v ? later : v;
+    if (j < keep) nn[j] = v;
+    __syncthreads();
+    if (tid == 0) s_carry = v;  // thread 0 holds the minimum of the whole chunk and everything after it
+    __syncthreads();
+  }
+
+  int yi = 0;
+  for (int i = 0; i < keep; ++i) {
+    __syncthreads();  // removals from the previous row are visible
+    if (rem[i]) continue;
+    const int32_t* r1 = srt + (int64_t)i * k;
+    if (r1[0] >= 0) {
+      if (tid < k) yb[(int64_t)yi * k + tid] = r1[tid];
+      ++yi;
+    }
+    const int limit = nn[i + 1];
+    const int32_t id1 = id_index >= 0 ? r1[id_index] : 0;
+    for (int j = i + 1 + tid; j < limit; j += NMS_THREADS) {
+      if (rem[j]) continue;
+      const int32_t* r2 = srt + (int64_t)j * k;
+      if (force_suppress || id_index < 0 || id1 == r2[id_index])
+        if (iou100(r1 + coord_start, r2 + coord_start) >= iou_threshold) rem[j] = 1;
+    }
+  }
+  // max_output_size keeps the first `max_output_size` emitted rows (nms.cc:126-137)
+  if (max_output_size > 0 && yi > max_output_size) yi = max_output_size;
+  __syncthreads();
+  for (int64_t i = (int64_t)yi * k + tid; i < (int64_t)n * k; i += NMS_THREADS) yb[i] = -1;
+}
+
+}  // namespace cvmhip
+
+using namespace cvmhip;
+
+extern "C" {
+
+size_t cvmhip_get_valid_counts_workspace_bytes(int batches, int n) {
+  const int nchunks = (n + GVC_CHUNK - 1) / GVC_CHUNK;
+  return (size_t)batches * nchunks * sizeof(int32_t);
+}
+
+int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
+                            int batches, int n, int k, int32_t score_threshold,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !valid_count || !y || batches < 1 || n < 1 || k < 2 || batches > 65535) return arg_error("get_valid_counts");
+  if (!workspace || workspace_bytes < cvmhip_get_valid_counts_workspace_bytes(batches, n))
+    return arg_error("get_valid_counts workspace");
+  const int nchunks = (n + GVC_CHUNK - 1) / GVC_CHUNK;
+  int32_t* counts = reinterpret_cast<int32_t*>(workspace);
+  hipStream_t s = as_stream(stream);
+  dim3 grid(nchunks, batches);
+  k_gvc_count<<<grid, GVC_CHUNK, 0, s>>>(x, counts, n, k, score_threshold, nchunks);
+  int rc = check_launch("get_valid_counts.count");
+  if (rc) return rc;
+  k_gvc_scatter<<<grid, GVC_CHUNK, 0, s>>>(x, counts, valid_count, y, n, k, score_threshold, nchunks);
+  return check_launch("get_valid_counts.scatter");
+}
+
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k]
+size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
+  return (size_t)batches * ((size_t)n * (3 + (size_t)k) + 1) * sizeof(int32_t);
+}
+
+int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
+                               int batches, int n, int k, int max_output_size,
+                               int iou_threshold, int topk, int coord_start,
+                               int score_index, int id_index, int force_suppress,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !valid_count || !y || batches < 1 || n < 1 || k < 2 || batches > 65535) return arg_error("non_max_suppression");
+  if (iou_threshold <= 0) return arg_error("non_max_suppression.iou_threshold must be positive");
+  if (coord_start < 0 || coord_start + 4 > k || score_index < 0 || score_index >= k || id_index >= k)
+    return arg_error("non_max_suppression indices");
+  if (n > (1 << 18)) return arg_error("non_max_suppression: more than 2^18 anchors per batch is not supported");
+  if (!workspace || workspace_bytes < cvmhip_nms_workspace_bytes(batches, n, k)) return arg_error("non_max_suppression workspace");
+  hipStream_t s = as_stream(stream);
+  int32_t* order = reinterpret_cast<int32_t*>(workspace);
+  int32_t* nextneg = order + (size_t)batches * n;
+  int32_t* removed = nextneg + (size_t)batches * (n + 1);
+  int32_t* sorted = removed + (size_t)batches * n;
+  dim3 grid((n + 255) / 256, batches);
+  k_nms_rank<<<grid, 256, 0, s>>>(x, valid_count, order, sorted, n, k, score_index, (int64_t)n);
+  int rc = check_launch("nms.rank");
+  if (rc) return rc;
+  k_nms_select<<<batches, NMS_THREADS, 0, s>>>(x, valid_count, y, order, sorted, nextneg, removed, n, k,
+                                               max_output_size, iou_threshold, topk, coord_start, id_index,
+                                               force_suppress, (int64_t)n);
+  return check_launch("nms.select");
+}
+
+}  // extern "C"

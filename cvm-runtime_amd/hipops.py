@@ -1,0 +1,290 @@
+"""Thin ctypes wrappers over the operator-level C ABI (include/cvm_hip_ops.h).
+
+Arguments and results are int32 torch tensors on the GPU (torch only supplies
+the device memory and the stream).  The names and argument meaning follow the
+reference's operators (`cvm.runtime.<dev>.<op>`, src/runtime/cpu/ops), so a
+parity test reads like the reference's tests/test_op.cc cases.
+"""
+import ctypes
+
+import torch
+
+from . import check, lib
+
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_i64p = ctypes.POINTER(ctypes.c_int64)
+
+BCAST = {"broadcast_add": 0, "broadcast_sub": 1, "broadcast_mul": 2,
+         "broadcast_max": 3, "broadcast_div": 4, "broadcast_greater": 5}
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.dtype == torch.int32 and t.is_contiguous(), "int32 contiguous CUDA tensor required"
+    return ctypes.cast(t.data_ptr(), _i32p)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _shape(s):
+    return (ctypes.c_int64 * max(len(s), 1))(*[int(v) for v in s])
+
+
+def _new(shape, like):
+    return torch.empty(tuple(int(v) for v in shape), dtype=torch.int32, device=like.device)
+
+
+def _workspace(nbytes, dev):
+    # 256-byte aligned scratch (torch's caching allocator aligns to 512)
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=dev)
+
+
+def conv_out_hw(h, w, kh, kw, sh, sw, ph, pw, dh, dw):
+    return ((h + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1,
+            (w + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
+
+
+def conv2d(x, w, b=None, strides=(1, 1), padding=(0, 0), dilation=(1, 1), groups=1):
+    n, ic, h, wd = x.shape
+    oc, _, kh, kw = w.shape
+    oh, ow = conv_out_hw(h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    y = _new((n, oc, oh, ow), x)
+    L = lib()
+    nbytes = L.cvmhip_conv2d_workspace_bytes(n, ic, h, wd, oc, kh, kw, groups)
+    ws = _workspace(nbytes, x.device)
+    check(L.cvmhip_conv2d(_ptr(x), _ptr(w), _ptr(b), _ptr(y), n, ic, h, wd, oc, kh, kw,
+                          strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1],
+                          groups, ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()), _stream()))
+    return y
+
+
+def dense(x, w, b=None, operand_bits=8):
+    m, k = x.shape
+    n = w.shape[0]
+    y = _new((m, n), x)
+    L = lib()
+    ws = _workspace(L.cvmhip_dense_workspace_bytes(m, k, n), x.device)
+    check(L.cvmhip_dense(_ptr(x), _ptr(w), _ptr(b), _ptr(y), m, k, n, operand_bits,
+                         ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()), _stream()))
+    return y
+
+
+def _unary(fn, x, *args, out=None):
+    y = torch.empty_like(x) if out is None else out
+    check(fn(_ptr(x), _ptr(y), ctypes.c_int64(x.numel()), *args, _stream()))
+    return y
+
+
+def relu(x, out=None):
+    return _unary(lib().cvmhip_relu, x, out=out)
+
+
+def cvm_clip(x, precision, out=None):
+    return _unary(lib().cvmhip_cvm_clip, x, int(precision), out=out)
+
+
+def cvm_right_shift(x, precision, shift_bit, out=None):
+    return _unary(lib().cvmhip_cvm_right_shift, x, int(precision), int(shift_bit), out=out)
+
+
+def cvm_left_shift(x, precision, shift_bit, out=None):
+    return _unary(lib().cvmhip_cvm_left_shift, x, int(precision), int(shift_bit), out=out)
+
+
+def clip(x, a_min, a_max, out=None):
+    return _unary(lib().cvmhip_clip, x, ctypes.c_int32(a_min), ctypes.c_int32(a_max), out=out)
+
+
+def abs_(x, out=None):
+    return _unary(lib().cvmhip_abs, x, out=out)
+
+
+def negative(x, out=None):
+    return _unary(lib().cvmhip_negative, x, out=out)
+
+
+def cvm_precision(x, out=None):
+    return _unary(lib().cvmhip_cvm_precision, x, out=out)
+
+
+def elemwise(op, a, b, out=None):
+    c = torch.empty_like(a) if out is None else out
+    check(lib().cvmhip_elemwise(0 if op == "elemwise_add" else 1, _ptr(a), _ptr(b), _ptr(c),
+                                ctypes.c_int64(a.numel()), _stream()))
+    return c
+
+
+def broadcast_shape(sa, sb):
+    nd = max(len(sa), len(sb))
+    pa = (1,) * (nd - len(sa)) + tuple(sa)
+    pb = (1,) * (nd - len(sb)) + tuple(sb)
+    return tuple(max(u, v) for u, v in zip(pa, pb))
+
+
+def broadcast(op, a, b):
+    cs = broadcast_shape(a.shape, b.shape)
+    c = _new(cs, a)
+    check(lib().cvmhip_broadcast(BCAST[op], _ptr(a), _shape(a.shape), a.dim(), _ptr(b), _shape(b.shape),
+                                 b.dim(), _ptr(c), _shape(cs), len(cs), _stream()))
+    return c
+
+
+def pool_out(h, k, s, p, ceil_mode):
+    if ceil_mode:
+        return (h + 2 * p - k + s - 1) // s + 1
+    return (h + 2 * p - k) // s + 1
+
+
+def max_pool2d(x, pool_size, strides=(1, 1), padding=(0, 0), ceil_mode=False):
+    n, c, h, w = x.shape
+    pad = list(padding)
+    if len(pad) == 1:
+        pad = [pad[0], pad[0]]
+    oh = pool_out(h, pool_size[0], strides[0], pad[0], ceil_mode)
+    ow = pool_out(w, pool_size[1], strides[1], pad[1], ceil_mode)
+    y = _new((n, c, oh, ow), x)
+    check(lib().cvmhip_max_pool2d(_ptr(x), _ptr(y), n, c, h, w, oh, ow, pool_size[0], pool_size[1],
+                                  strides[0], strides[1], pad[0], pad[1], _stream()))
+    return y
+
+
+def reduce_shape(shape, axes, keepdims, exclude):
+    nd = len(shape)
+    ax = sorted(a + nd if a < 0 else a for a in axes)
+    if not ax:
+        r = list(range(nd))
+    elif exclude:
+        r = [i for i in range(nd) if i not in ax]
+    else:
+        r = ax
+    if not r:
+        return tuple(shape)
+    if len(r) == nd:
+        return (1,) * nd if keepdims else (1,)
+    if keepdims:
+        return tuple(1 if i in r else s for i, s in enumerate(shape))
+    return tuple(s for i, s in enumerate(shape) if i not in r)
+
+
+def reduce(op, x, axes=(), keepdims=False, exclude=False):
+    ys = reduce_shape(x.shape, list(axes), keepdims, exclude)
+    y = _new(ys, x)
+    ax = _shape(list(axes)) if len(axes) else None
+    check(lib().cvmhip_reduce(0 if op == "sum" else 1, _ptr(x), _shape(x.shape), x.dim(), _ptr(y),
+                              ctypes.c_int64(y.numel()), ax, len(axes), int(bool(exclude)), _stream()))
+    return y
+
+
+def copy(x, shape):
+    y = _new(shape, x)
+    check(lib().cvmhip_copy(_ptr(x), _ptr(y), ctypes.c_int64(x.numel()), _stream()))
+    return y
+
+
+def concatenate(xs, axis):
+    nd = xs[0].dim()
+    ax = axis + nd if axis < 0 else axis
+    ys = list(xs[0].shape)
+    ys[ax] = sum(v.shape[ax] for v in xs)
+    y = _new(ys, xs[0])
+    n = len(xs)
+    ptrs = (_i32p * n)(*[_ptr(v) for v in xs])
+    shp = [_shape(v.shape) for v in xs]
+    shps = (_i64p * n)(*[ctypes.cast(s, _i64p) for s in shp])
+    check(lib().cvmhip_concatenate(ptrs, shps, n, nd, axis, _ptr(y), _shape(ys), _stream()))
+    return y
+
+
+def transpose(x, axes=()):
+    nd = x.dim()
+    perm = [a + nd if a < 0 else a for a in axes] if len(axes) else list(range(nd))[::-1]
+    y = _new([x.shape[p] for p in perm], x)
+    check(lib().cvmhip_transpose(_ptr(x), _shape(x.shape), nd, _shape(list(axes)) if len(axes) else None,
+                                 len(axes), _ptr(y), _stream()))
+    return y
+
+
+def strided_slice(x, begin, end, stride, out_shape):
+    y = _new(out_shape, x)
+    check(lib().cvmhip_strided_slice(_ptr(x), _shape(x.shape), x.dim(), _shape(begin), len(begin),
+                                     _shape(stride) if len(stride) else None, len(stride),
+                                     _ptr(y), _shape(out_shape), _stream()))
+    return y
+
+
+def slice_like(x, out_shape):
+    y = _new(out_shape, x)
+    check(lib().cvmhip_slice_like(_ptr(x), _shape(x.shape), x.dim(), _ptr(y), _shape(out_shape), _stream()))
+    return y
+
+
+def take(x, indices, axis=None):
+    if axis is None:
+        ys = tuple(indices.shape)
+    else:
+        a = axis + x.dim() if axis < 0 else axis
+        ys = tuple(x.shape[:a]) + tuple(indices.shape) + tuple(x.shape[a + 1:])
+    y = _new(ys, x)
+    check(lib().cvmhip_take(_ptr(x), _shape(x.shape), x.dim(), _ptr(indices), _shape(indices.shape),
+                            indices.dim(), _ptr(y), _shape(ys), len(ys), int(axis is not None),
+                            int(axis or 0), _stream()))
+    return y
+
+
+def repeat(x, repeats, axis=0):
+    a = axis + x.dim() if axis < 0 else axis
+    ys = list(x.shape)
+    ys[a] *= repeats
+    y = _new(ys, x)
+    check(lib().cvmhip_repeat(_ptr(x), _shape(x.shape), _ptr(y), _shape(ys), x.dim(), axis, repeats, _stream()))
+    return y
+
+
+def tile(x, reps):
+    nd = max(x.dim(), len(reps))
+    xs = (1,) * (nd - x.dim()) + tuple(x.shape)
+    rp = (1,) * (nd - len(reps)) + tuple(reps)
+    ys = [a * b for a, b in zip(xs, rp)]
+    y = _new(ys, x)
+    check(lib().cvmhip_tile(_ptr(x), _shape(x.shape), x.dim(), _ptr(y), _shape(ys), nd, _stream()))
+    return y
+
+
+def upsampling(x, scale):
+    n, c, h, w = x.shape
+    y = _new((n, c, h * scale, w * scale), x)
+    check(lib().cvmhip_upsampling(_ptr(x), _ptr(y), n, c, h, w, scale, _stream()))
+    return y
+
+
+def where(cond, x, y, out):
+    check(lib().cvmhip_where(_ptr(cond), _ptr(x), _ptr(y), _ptr(out), _shape(x.shape), x.dim(),
+                             int(cond.dim() == x.dim()), _stream()))
+    return out
+
+
+def get_valid_counts(x, score_threshold):
+    b, n, k = x.shape
+    vc = _new((b,), x)
+    y = torch.empty_like(x)
+    L = lib()
+    ws = _workspace(L.cvmhip_get_valid_counts_workspace_bytes(b, n), x.device)
+    check(L.cvmhip_get_valid_counts(_ptr(x), _ptr(vc), _ptr(y), b, n, k, ctypes.c_int32(score_threshold),
+                                    ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel()), _stream()))
+    return vc, y
+
+
+def non_max_suppression(x, valid_count, y, iou_threshold=50, force_suppress=False, top_k=-1,
+                        id_index=0, coord_start=2, score_index=1, max_output_size=-1):
+    """In place on y; x is mutated exactly as the reference mutates it."""
+    b, n, k = x.shape
+    L = lib()
+    ws = _workspace(L.cvmhip_nms_workspace_bytes(b, n, k), x.device)
+    check(L.cvmhip_non_max_suppression(_ptr(x), _ptr(valid_count), _ptr(y), b, n, k, max_output_size,
+                                       iou_threshold, top_k, coord_start, score_index, id_index,
+                                       int(bool(force_suppress)), ctypes.c_void_p(ws.data_ptr()),
+                                       ctypes.c_size_t(ws.numel()), _stream()))
+    return y

@@ -1,0 +1,154 @@
+/*
+ * Operator-level C ABI of the MI355X (gfx950) CVM backend.
+ *
+ * One entry point per reference operator kernel.  These are what a
+ * `CVM_REGISTER_GLOBAL("cvm.runtime.hip.<op>")` wrapper calls after unpacking
+ * its DLTensor arguments -- the role the `cuda_*` wrappers declared in the
+ * reference's src/runtime/cuda/ops/cuda_ops.h:111-235 play for the CUDA
+ * device.  Plain pointers and sizes only; no HIP or torch types.
+ *
+ * Conventions
+ *  - every tensor pointer is DEVICE memory holding contiguous row-major int32
+ *    (the reference's storage contract, src/runtime/graph_runtime.cc:505-506);
+ *  - shape arrays are HOST memory, int64, length ndim (ndim <= 6);
+ *  - `stream` is a hipStream_t passed as void* (NULL = default stream); calls
+ *    only enqueue work, they never synchronise the device;
+ *  - return value: CVMHIP_OK, or an error code.  Codes 10..19 are argument /
+ *    logic errors (map to VERIFY -> std::logic_error -> ERROR_LOGIC), codes
+ *    >= 20 are runtime failures (map to CHECK -> ERROR_RUNTIME), the same
+ *    split the reference uses in src/runtime/cuda/ops/ops_cuda.cc:33-43.
+ *    cvmhip_last_error() returns a message for the calling thread.
+ *  - results are bit-identical to the reference CPU operators
+ *    (src/runtime/cpu/ops) on the same inputs, including int32 wrap-around.
+ */
+#ifndef CVM_HIP_OPS_H_
+#define CVM_HIP_OPS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+#define CVMHIP_OK 0
+#define CVMHIP_ERR_ARG 10
+#define CVMHIP_ERR_RUNTIME 20
+
+enum { CVMHIP_ADD = 0, CVMHIP_SUB = 1, CVMHIP_MUL = 2, CVMHIP_MAX = 3, CVMHIP_DIV = 4, CVMHIP_GREATER = 5 };
+enum { CVMHIP_SUM = 0, CVMHIP_RMAX = 1 };
+
+const char* cvmhip_last_error(void);
+
+/* ---- conv2d: replaces cuda_conv2d / cuda_depthwise_conv2d / cuda_groupwise_conv2d
+ * (cuda_ops.h:113-142, conv.cu:394-700); semantics of cvm.runtime.cpu.conv2d
+ * (src/runtime/cpu/ops/ops.cc:368-456).  NCHW data, OIHW filter, bias[oc] or NULL.
+ * groups == 1: data and filter are narrowed to int8 (ops.cc:234,431) and the
+ * product runs on i8 MFMA as an implicit GEMM; groups > 1: exact int32 direct
+ * convolution, no narrowing (ops.cc:333-366).
+ * `workspace` is device scratch of at least cvmhip_conv2d_workspace_bytes()
+ * bytes -- the role args.ext_space plays for the CUDA backend
+ * (src/top/nn/convolution.cc:237-272). */
+size_t cvmhip_conv2d_workspace_bytes(int n, int ic, int h, int w, int oc, int kh, int kw, int groups);
+int cvmhip_conv2d(const int32_t* x, const int32_t* w, const int32_t* bias, int32_t* y,
+                  int n, int ic, int h, int wd, int oc, int kh, int kw,
+                  int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                  int groups, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- dense: replaces cuda_dense (cuda_ops.h:149, cuda_ops.cu:9-66); semantics of
+ * cvm.runtime.cpu.dense (ops.cc:34-75): y[m][n] = sum_k x[m][k]*w[n][k] (+ bias[n]).
+ * operand_bits <= 8 promises |x|,|w| <= 127 (what DenseInferPrecision,
+ * src/top/nn/nn.cc:22-44, guarantees inside a verified graph) and selects the
+ * i8 MFMA path; larger values select the exact int32 path. */
+size_t cvmhip_dense_workspace_bytes(int m, int k, int n);
+int cvmhip_dense(const int32_t* x, const int32_t* w, const int32_t* bias, int32_t* y,
+                 int m, int k, int n, int operand_bits,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- unary elementwise (y may alias x): cuda_relu / cuda_cvm_clip /
+ * cuda_cvm_right_shift / cuda_cvm_left_shift / cuda_clip / cuda_abs /
+ * cuda_negative / cuda_log (cuda_ops.h:154-211); CPU semantics in
+ * src/runtime/cpu/ops/ops.cc:12-26,525-553,632-642 and elemwise.cc:47-193. */
+int cvmhip_relu(const int32_t* x, int32_t* y, int64_t size, void* stream);
+int cvmhip_cvm_clip(const int32_t* x, int32_t* y, int64_t size, int precision, void* stream);
+int cvmhip_cvm_right_shift(const int32_t* x, int32_t* y, int64_t size, int precision, int shift_bit, void* stream);
+int cvmhip_cvm_left_shift(const int32_t* x, int32_t* y, int64_t size, int precision, int shift_bit, void* stream);
+int cvmhip_clip(const int32_t* x, int32_t* y, int64_t size, int32_t a_min, int32_t a_max, void* stream);
+int cvmhip_abs(const int32_t* x, int32_t* y, int64_t size, void* stream);
+int cvmhip_negative(const int32_t* x, int32_t* y, int64_t size, void* stream);
+int cvmhip_cvm_precision(const int32_t* x, int32_t* y, int64_t size, void* stream);
+
+/* ---- elemwise_add / elemwise_sub (c may alias a or b): cuda_elemwise_add/sub
+ * (cuda_ops.h:111-112); CPU elemwise.cc:8-45.  op is CVMHIP_ADD or CVMHIP_SUB. */
+int cvmhip_elemwise(int op, const int32_t* a, const int32_t* b, int32_t* c, int64_t size, void* stream);
+
+/* ---- broadcast_{add,sub,mul,max,div,greater}: cuda_broadcast_* (cuda_ops.h:157-188);
+ * CPU broadcast.cc:6-125 (right-aligned numpy broadcasting, div by 0 -> 0). */
+int cvmhip_broadcast(int op, const int32_t* a, const int64_t* ashape, int andim,
+                     const int32_t* b, const int64_t* bshape, int bndim,
+                     int32_t* c, const int64_t* cshape, int cndim, void* stream);
+
+/* ---- max_pool2d: cuda_max_pool (cuda_ops.h:143, conv.cu:704-760); CPU ops.cc:466-523
+ * (padding counts as INT32_MIN; output extent given by the caller). */
+int cvmhip_max_pool2d(const int32_t* x, int32_t* y, int n, int c, int h, int w,
+                      int oh, int ow, int kh, int kw, int stride_h, int stride_w,
+                      int pad_h, int pad_w, void* stream);
+
+/* ---- sum / max over an axis set: cuda_sum / cuda_max (cuda_ops.h:189-201);
+ * CPU reduce.cc:6-140.  `axes` as written in the attribute (negatives allowed). */
+int cvmhip_reduce(int op, const int32_t* x, const int64_t* xshape, int ndim,
+                  int32_t* y, int64_t ysize, const int64_t* axes, int naxes, int exclude,
+                  void* stream);
+
+/* ---- index-remap copies: cuda_concatenate, cuda_transpose, cuda_stride_slice,
+ * cuda_slice_like, cuda_take, cuda_repeat, cuda_tile, cuda_upsampling_nearest,
+ * cuda_where, cuda_flatten/reshape/expand_dims/squeeze (cuda_ops.h:156-235);
+ * CPU ops.cc:567-989,1049-1075 and elemwise.cc:64-86. */
+int cvmhip_copy(const int32_t* x, int32_t* y, int64_t size, void* stream); /* flatten/reshape/expand_dims/squeeze */
+int cvmhip_concatenate(const int32_t* const* inputs, const int64_t* const* ishapes, int ninputs,
+                       int ndim, int axis, int32_t* y, const int64_t* yshape, void* stream);
+int cvmhip_transpose(const int32_t* x, const int64_t* xshape, int ndim,
+                     const int64_t* axes, int naxes, int32_t* y, void* stream);
+int cvmhip_strided_slice(const int32_t* x, const int64_t* xshape, int ndim,
+                         const int64_t* begin, int nbegin, const int64_t* stride, int nstride,
+                         int32_t* y, const int64_t* yshape, void* stream);
+int cvmhip_slice_like(const int32_t* x, const int64_t* xshape, int ndim,
+                      int32_t* y, const int64_t* yshape, void* stream);
+int cvmhip_take(const int32_t* x, const int64_t* xshape, int xndim,
+                const int32_t* indices, const int64_t* ishape, int indim,
+                int32_t* y, const int64_t* yshape, int yndim, int has_axis, int axis, void* stream);
+int cvmhip_repeat(const int32_t* x, const int64_t* xshape, int32_t* y, const int64_t* yshape,
+                  int ndim, int axis, int repeats, void* stream);
+int cvmhip_tile(const int32_t* x, const int64_t* xshape, int xndim,
+                int32_t* y, const int64_t* yshape, int yndim, void* stream);
+int cvmhip_upsampling(const int32_t* x, int32_t* y, int n, int c, int h, int w, int scale, void* stream);
+int cvmhip_where(const int32_t* cond, const int32_t* x, const int32_t* y, int32_t* out,
+                 const int64_t* oshape, int ndim, int same_shape, void* stream);
+
+/* ---- get_valid_counts: cuda_get_valid_counts (cuda_ops.h:225, nms.cu:11-127);
+ * CPU nms.cc:42-63.  Rows with row[1] > score_threshold are compacted in their
+ * original order, the rest of y is -1, valid_count[b] is the count.
+ * `workspace`: cvmhip_get_valid_counts_workspace_bytes() bytes of device scratch. */
+size_t cvmhip_get_valid_counts_workspace_bytes(int batches, int n);
+int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
+                            int batches, int n, int k, int32_t score_threshold,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- non_max_suppression: cuda_non_max_suppression (cuda_ops.h:228, nms.cu:310-430);
+ * semantics of the CPU operator (nms.cc:65-140), including its early exit on a
+ * batch with no valid rows, its stop at the first negative id and its in-place
+ * overwrite of x rows past top_k.  No host synchronisation: valid_count is read
+ * on the device.  `workspace`: cvmhip_nms_workspace_bytes() bytes of scratch. */
+size_t cvmhip_nms_workspace_bytes(int batches, int n, int k);
+int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
+                               int batches, int n, int k, int max_output_size,
+                               int iou_threshold, int topk, int coord_start,
+                               int score_index, int id_index, int force_suppress,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* CVM_HIP_OPS_H_ */
