@@ -493,4 +493,41 @@ int cvmhip_dense(const int32_t* x, const int32_t* w, const int32_t* bias, int32_
   return conv_igemm(xp, wp, y, g, ep, s);
 }
 
+size_t cvmhip_packed_weight_bytes(int oc, int ic, int kh, int kw) { return packed_weight_bytes(oc, ic, kh, kw); }
+
+size_t cvmhip_packed_act_bytes(int64_t npix, int channels) { return packed_act_bytes(npix, channels); }
+
+int cvmhip_pack_weights(const int32_t* w, void* wp, int oc, int ic, int kh, int kw, void* stream) {
+  if (!w || !wp || oc < 1 || ic < 1 || kh < 1 || kw < 1 || ((uintptr_t)wp & 15)) return arg_error("pack_weights");
+  return pack_weights(w, reinterpret_cast<int8_t*>(wp), oc, ic, kh, kw, as_stream(stream));
+}
+
+int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, int32_t* y,
+                         int n, int ic, int h, int wd, int oc, int kh, int kw,
+                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !wp || !y) return arg_error("conv2d_packed null tensor");
+  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+    return arg_error("conv2d_packed attributes");
+  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("conv2d_packed kernel exceeds input");
+  const size_t need = packed_act_bytes((int64_t)n * h * wd, ic);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return arg_error("conv2d_packed workspace");
+  hipStream_t s = as_stream(stream);
+  int8_t* xp = reinterpret_cast<int8_t*>(workspace);
+  int rc = pack_activations(x, xp, n, ic, h * wd, s);
+  if (rc) return rc;
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic);
+  g.OC = oc;
+  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  Epilogue ep = {};
+  ep.bias = bias;
+  ep.out_mode = OUT_I32_NCHW;
+  return conv_igemm(xp, reinterpret_cast<const int8_t*>(wp), y, g, ep, s);
+}
+
 }  // extern "C"

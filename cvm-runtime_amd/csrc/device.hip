@@ -1,0 +1,115 @@
+// Device memory, streams and events behind plain C entry points, so the host
+// runtime (plain C++) never sees a HIP type.
+#include "hip_common.h"
+
+using namespace cvmhip;
+
+#define HIP_TRY(expr, what)                                         \
+  do {                                                              \
+    hipError_t e_ = (expr);                                         \
+    if (e_ != hipSuccess) {                                         \
+      set_error("%s: %s", what, hipGetErrorString(e_));             \
+      return CVMHIP_ERR_RUNTIME;                                    \
+    }                                                               \
+  } while (0)
+
+namespace cvmhip {
+__global__ void __launch_bounds__(256) k_fill32(int32_t* p, int32_t v, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+}  // namespace cvmhip
+
+extern "C" {
+
+int cvmhip_device_count(int* count) {
+  if (!count) return arg_error("device_count");
+  HIP_TRY(hipGetDeviceCount(count), "hipGetDeviceCount");
+  return CVMHIP_OK;
+}
+
+int cvmhip_set_device(int device_id) {
+  HIP_TRY(hipSetDevice(device_id), "hipSetDevice");
+  return CVMHIP_OK;
+}
+
+int cvmhip_alloc(void** ptr, size_t bytes) {
+  if (!ptr) return arg_error("alloc");
+  HIP_TRY(hipMalloc(ptr, bytes ? bytes : 256), "hipMalloc");
+  return CVMHIP_OK;
+}
+
+int cvmhip_free(void* ptr) {
+  if (ptr) HIP_TRY(hipFree(ptr), "hipFree");
+  return CVMHIP_OK;
+}
+
+// A fill kernel rather than hipMemsetAsync so the call stays valid inside a captured graph.
+int cvmhip_memset32(void* ptr, int32_t value, size_t count, void* stream) {
+  if (count == 0) return CVMHIP_OK;
+  if (!ptr) return arg_error("memset32");
+  k_fill32<<<grid_for((int64_t)count, 256), 256, 0, as_stream(stream)>>>((int32_t*)ptr, value, count);
+  return check_launch("memset32");
+}
+
+int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return CVMHIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)), "copy_h2d");
+  return CVMHIP_OK;
+}
+
+int cvmhip_copy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return CVMHIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)), "copy_d2h");
+  return CVMHIP_OK;
+}
+
+int cvmhip_copy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0 || dst == src) return CVMHIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)), "copy_d2d");
+  return CVMHIP_OK;
+}
+
+int cvmhip_stream_create(void** stream) {
+  if (!stream) return arg_error("stream_create");
+  hipStream_t s;
+  HIP_TRY(hipStreamCreate(&s), "hipStreamCreate");  // default priority
+  *stream = s;
+  return CVMHIP_OK;
+}
+
+int cvmhip_stream_destroy(void* stream) {
+  if (stream) HIP_TRY(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy");
+  return CVMHIP_OK;
+}
+
+int cvmhip_stream_sync(void* stream) {
+  HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+  return CVMHIP_OK;
+}
+
+int cvmhip_event_create(void** event) {
+  if (!event) return arg_error("event_create");
+  hipEvent_t e;
+  HIP_TRY(hipEventCreate(&e), "hipEventCreate");
+  *event = e;
+  return CVMHIP_OK;
+}
+
+int cvmhip_event_destroy(void* event) {
+  if (event) HIP_TRY(hipEventDestroy((hipEvent_t)event), "hipEventDestroy");
+  return CVMHIP_OK;
+}
+
+int cvmhip_event_record(void* event, void* stream) {
+  HIP_TRY(hipEventRecord((hipEvent_t)event, as_stream(stream)), "hipEventRecord");
+  return CVMHIP_OK;
+}
+
+int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms) {
+  HIP_TRY(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize");
+  HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+  return CVMHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,165 @@
+// Host-side graph runtime for the HIP device: loads a CVM graph (JSON) and its
+// parameter blob, verifies them with the reference's rules, plans device
+// storage and executes the nodes in topological order on one HIP stream.
+//
+// Mirrors the interface and behaviour of the reference's CvmRuntime
+// (src/runtime/graph_runtime.{h,cc}, src/runtime/infer_attr.cc) for a single
+// device type, "hip".  Operator kernels are looked up in a registry under
+// "cvm.runtime.hip.<op>" -- the naming scheme of graph_runtime.cc:660-664.
+#ifndef CVM_RT_GRAPH_RUNTIME_H_
+#define CVM_RT_GRAPH_RUNTIME_H_
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "base.h"
+#include "json.h"
+#include "op_schema.h"
+
+namespace cvmrt {
+
+// A device tensor as an operator sees it: int32, contiguous, row-major.
+struct DevTensor {
+  int32_t* data = nullptr;
+  Shape shape;
+  int precision = -1;
+  bool is_param = false;  // produced by a variable node other than `data` (constant after load_params)
+  int64_t size() const { return shape_size(shape); }
+};
+
+struct OpCall;
+
+// What the registry stores for one operator of the device.
+struct OpKernel {
+  // bytes of device scratch the operator needs for these tensors (the role of
+  // FOpExtraSpace, include/cvm/op_attr_types.h:86-90)
+  std::function<size_t(const OpCall&)> workspace_bytes;
+  // once, after the parameters are on the device (e.g. pre-pack constant filters)
+  std::function<void(OpCall&)> prepare;
+  // enqueue the operator on call.stream
+  std::function<void(OpCall&)> run;
+};
+
+// Arguments of one node: inputs, outputs, parsed attributes, scratch, stream --
+// the same information CVMArgs carries ([in..., out..., NodeAttrs*] + ext_space).
+struct OpCall {
+  std::string op;
+  std::vector<DevTensor> in, out;
+  const OpAttrs* attrs = nullptr;
+  void* workspace = nullptr;
+  size_t workspace_bytes = 0;
+  void* stream = nullptr;
+  std::shared_ptr<void> state;  // per-node data owned by the kernel (packed filters ...)
+};
+
+class OpRegistry {
+ public:
+  static OpRegistry& Global();
+  void Register(const std::string& name, OpKernel k) { table_[name] = std::move(k); }
+  const OpKernel* Get(const std::string& name) const {
+    auto it = table_.find(name);
+    return it == table_.end() ? nullptr : &it->second;
+  }
+  std::vector<std::string> ListNames() const;
+
+ private:
+  std::map<std::string, OpKernel> table_;
+};
+
+void RegisterHipKernels();  // fills the registry with cvm.runtime.hip.* (hip_ops.cc)
+
+struct NodeEntry {
+  uint32_t node_id = 0, index = 0, version = 0;
+};
+
+struct Node {
+  std::string op_type;
+  std::string name;
+  std::string func_name;
+  std::vector<NodeEntry> inputs;
+  const OpSchema* schema = nullptr;
+  OpAttrs attrs;
+  uint32_t num_inputs = 1, num_outputs = 1;
+  bool is_variable() const { return op_type == "null"; }
+  bool is_data() const { return is_variable() && name == "data"; }
+};
+
+class HipGraphRuntime {
+ public:
+  // with_device == false parses and verifies only (gas estimation from a graph file)
+  HipGraphRuntime(const std::string& graph_json, int device_id, bool with_device);
+  ~HipGraphRuntime();
+  HipGraphRuntime(const HipGraphRuntime&) = delete;
+  HipGraphRuntime& operator=(const HipGraphRuntime&) = delete;
+
+  void LoadParams(const std::string& blob);
+  // `data` tensor from host memory: int32 values, already widened
+  void SetData(const int32_t* host, const Shape& shape);
+  void Run();
+  void CopyOutputTo(int index, int32_t* host);  // synchronises the stream
+
+  // device-resident variants used to time Run() alone
+  int32_t* DataDevicePtr();
+  void SyncStream();
+
+  int NumOutputs() const { return static_cast<int>(outputs_.size()); }
+  const Shape& InputShape() const;
+  const Shape& OutputShape(int index) const;
+  int GetInputPrecision() const;
+  int GetOutputPrecision() const;
+  int64_t GetOps() const;
+  int64_t GetStorageSize() const;
+  std::string version() const { return version_.substr(0, 32); }
+  std::string postprocess_method() const { return postprocess_.substr(0, 32); }
+
+  // per-operator device time of one Run(), in milliseconds, keyed by operator name
+  std::map<std::string, double> ProfileRun();
+  // elapsed device milliseconds of `iterations` back-to-back Run() calls
+  float TimeRuns(int iterations);
+  size_t NumNodes() const { return nodes_.size(); }
+
+ private:
+  uint32_t entry_id(uint32_t nid, uint32_t index) const { return node_row_ptr_[nid] + index; }
+  uint32_t entry_id(const NodeEntry& e) const { return entry_id(e.node_id, e.index); }
+  void Load(const Json& doc);
+  void PrepareGraph();
+  void SetupShape();
+  void SetupPrecision();
+  void PlanStorage();
+  void SetupStorage();
+  void SetupOpExecs();
+  void Release();
+  void SetInput(uint32_t input_index, const int32_t* data32, const Shape& shape);
+  int GetInputIndex(const std::string& name) const;
+
+  std::vector<Node> nodes_;
+  std::vector<uint32_t> input_nodes_, node_row_ptr_;
+  std::vector<NodeEntry> outputs_;
+  uint32_t num_node_entries_ = 0;
+  // graph attributes
+  std::vector<int> storage_id_, device_index_, precision_;
+  std::vector<std::string> dltype_, op_attrs_;
+  std::vector<Shape> shape_;
+  std::string version_ = "cvm_1.0.0";
+  std::string postprocess_;
+
+  struct PoolEntry { size_t bytes = 0; size_t offset = 0; };
+  std::vector<PoolEntry> pool_;
+  int device_id_ = 0;
+  bool with_device_ = false;
+  void* slab_ = nullptr;       // one allocation backing every pool entry
+  size_t slab_bytes_ = 0;
+  void* workspace_ = nullptr;  // shared operator scratch
+  size_t workspace_bytes_ = 0;
+  void* stream_ = nullptr;
+  std::vector<int32_t*> entry_ptr_;
+  struct Exec { uint32_t nid; const OpKernel* kernel; OpCall call; };
+  std::vector<Exec> execs_;
+  bool params_loaded_ = false;
+};
+
+}  // namespace cvmrt
+#endif

@@ -1,0 +1,43 @@
+/*
+ * Additions of the gfx950 backend that have no counterpart in the reference's
+ * C API.  They exist for measurement and for testing the host logic; a caller
+ * that only knows include/cvm_c_api.h never needs them.
+ */
+#ifndef CVM_HIP_EXT_H_
+#define CVM_HIP_EXT_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+/* CVMAPIInference split in its three stages (src/core/model.cc:154-291):
+ * stage the input on the device, run the graph, fetch and post-process the
+ * outputs.  Lets a harness time the device-resident part alone. */
+int CVMHIPSetInput(void* net, const char* input_data, int input_len);
+int CVMHIPRun(void* net);
+int CVMHIPGetOutput(void* net, char* output_data);
+/* Runs the graph `iterations` times on the input already on the device and
+ * returns the elapsed device time in milliseconds, measured with events
+ * recorded on the runtime's own stream. */
+int CVMHIPTimeRun(void* net, int iterations, float* elapsed_ms);
+/* Per-operator device time of one run as a JSON object {"op": ms, ...}
+ * (the table the reference prints under -DPROFILE, graph_runtime.cc:62-87). */
+int CVMHIPProfileOps(void* net, char* json_out, int capacity);
+
+/* Host-side inference for ONE node, no device needed: parses `attr_json`
+ * (string-valued dict) and applies the operator's shape and precision rules
+ * (src/top/**).  Shapes are rows of 6 int64.  Returns SUCCEED / ERROR_LOGIC /
+ * ERROR_RUNTIME with the message in err. */
+int CVMHIPInferNode(const char* op, const char* attr_json, int n_in,
+                    const long long* in_shapes, const int* in_ndims, const int* in_precs,
+                    int* n_out, long long* out_shapes, int* out_ndims, int* out_precs,
+                    char* err, int errlen);
+/* Newline-separated names registered for the device: cvm.runtime.hip.<op> */
+int CVMHIPListOps(char* out, int capacity);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* CVM_HIP_EXT_H_ */

@@ -147,6 +147,42 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
                                int score_index, int id_index, int force_suppress,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- device memory and streams: what a DeviceAPI subclass registered as
+ * "device_api.hip" needs (include/cvm/runtime/device_api.h:43-108: SetDevice,
+ * AllocDataSpace, FreeDataSpace, CopyDataFromTo, StreamSync).  Allocations are
+ * aligned to at least 256 bytes. */
+int cvmhip_device_count(int* count);
+int cvmhip_set_device(int device_id);
+int cvmhip_alloc(void** ptr, size_t bytes);
+int cvmhip_free(void* ptr);
+int cvmhip_memset32(void* ptr, int32_t value, size_t count, void* stream);
+int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream);
+int cvmhip_copy_d2h(void* dst, const void* src, size_t bytes, void* stream);
+int cvmhip_copy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int cvmhip_stream_create(void** stream);
+int cvmhip_stream_destroy(void* stream);
+int cvmhip_stream_sync(void* stream);
+/* elapsed-time probes for the per-operator time table (the reference's -DPROFILE
+ * table, src/runtime/graph_runtime.cc:62-87, measured with device events) */
+int cvmhip_event_create(void** event);
+int cvmhip_event_destroy(void* event);
+int cvmhip_event_record(void* event, void* stream);
+int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---- conv2d / dense with the filter packed once at model-load time.  The
+ * filter of a graph node is a constant parameter, so the int32 OIHW -> int8
+ * MFMA-row layout conversion that cuda_conv2d redoes on every call
+ * (conv.cu:430-438) is hoisted out of the inference path.
+ * `wp` is cvmhip_packed_weight_bytes() bytes; `workspace` holds the packed
+ * activations, cvmhip_packed_act_bytes(n*h*w, ic) bytes. */
+size_t cvmhip_packed_weight_bytes(int oc, int ic, int kh, int kw);
+size_t cvmhip_packed_act_bytes(int64_t npix, int channels);
+int cvmhip_pack_weights(const int32_t* w, void* wp, int oc, int ic, int kh, int kw, void* stream);
+int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, int32_t* y,
+                         int n, int ic, int h, int wd, int oc, int kh, int kw,
+                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

@@ -1,0 +1,117 @@
+"""GPU parity of whole graphs through the model-level C ABI (CVMAPILoadModel /
+CVMAPIInference, include/cvm_c_api.h) against the CPU oracle executing the same
+graph node by node -- the method of the reference's tests/test_model.cc:94-235,
+with the oracle in place of the absent /data fixtures.  Bit-exact."""
+import numpy as np
+import pytest
+
+import oracle
+import oracle.graph as og
+from cvm_runtime_amd import graphgen, runtime, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_both(g, heads, cid, postprocess=None):
+    js, pb = g.build(heads, postprocess=postprocess)
+    x = synth.tensor(cid, "data", g.shape((0, 0)), -127, 127)
+    m = runtime.HipModel(js, pb)
+    try:
+        assert m.input_length == x.size      # int8 input: 1 byte per element
+        out = m.inference(x.astype(np.int8).tobytes())
+        out2 = m.inference(x.astype(np.int8).tobytes())   # storage is reused across calls
+        assert out == out2
+        tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+    finally:
+        m.close()
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    return out, tsize, ref
+
+
+def _check(out, tsize, ref):
+    got = np.frombuffer(out, np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    want = np.concatenate([r.ravel() for r in ref])
+    assert got.shape == want.shape
+    if not np.array_equal(got, want):
+        bad = np.flatnonzero(got != want)
+        raise AssertionError("%d of %d outputs differ, first at %d: got %d want %d" % (
+            len(bad), want.size, bad[0], got[bad[0]], want[bad[0]]))
+
+
+def test_config1_conv_shift_clip(dev):
+    g, heads = graphgen.conv_op_graph()
+    out, tsize, ref = _run_both(g, heads, "cfg1")
+    assert tsize == 1                        # 8-bit output precision -> int8 bytes
+    _check(out, tsize, ref)
+
+
+@pytest.mark.parametrize("batch", [1, 64])
+def test_config2_resnet20(batch, dev):
+    g, heads = graphgen.resnet20_cifar(batch)
+    out, tsize, ref = _run_both(g, heads, "cfg2-b%d" % batch)
+    _check(out, tsize, ref)
+
+
+def test_config3_resnet50_batch1_full_size(dev):
+    g, heads = graphgen.resnet50(1)
+    out, tsize, ref = _run_both(g, heads, "cfg3-b1")
+    _check(out, tsize, ref)
+
+
+def test_config3_resnet50_batch16_matches_per_image_runs(dev):
+    # full-size batch 16: every image of the batch must equal the batch-1 result
+    # of the same image (images are independent), and image 0 equals the oracle
+    # through the batch-1 test above (same weights: same config id).
+    g16, h16 = graphgen.resnet50(16)
+    js16, pb = g16.build(h16)
+    x = synth.tensor("cfg3-b16", "data", (16, 3, 224, 224), -127, 127).astype(np.int8)
+    m16 = runtime.HipModel(js16, pb)
+    out16 = np.frombuffer(m16.inference(x.tobytes()), np.int32).reshape(16, 1000)
+    m16.close()
+    g1, h1 = graphgen.resnet50(1)
+    js1, pb1 = g1.build(h1)
+    assert pb1 == pb
+    m1 = runtime.HipModel(js1, pb1)
+    for i in (0, 7, 15):
+        o = np.frombuffer(m1.inference(x[i:i + 1].tobytes()), np.int32)
+        assert np.array_equal(o, out16[i]), "image %d differs between batch 16 and batch 1" % i
+    m1.close()
+    ref = og.run_graph(js1, graphgen.load_params(pb1), x[3:4].astype(np.int32))
+    assert np.array_equal(ref[0].ravel(), out16[3])
+
+
+def test_config4_vgg16_reduced_width(dev):
+    # same 13-conv / 5-pool / 3-dense structure at 1/4 width so the oracle finishes in seconds
+    g, heads = graphgen.vgg16(2, size=64, width=16, fc=256, classes=100, config_id="cfg4-small")
+    out, tsize, ref = _run_both(g, heads, "cfg4-small")
+    _check(out, tsize, ref)
+
+
+def test_config4_vgg16_full_size_batch1(dev):
+    g, heads = graphgen.vgg16(1)
+    out, tsize, ref = _run_both(g, heads, "cfg4-b1")
+    _check(out, tsize, ref)
+
+
+@pytest.mark.parametrize("neg_ids", [False, True])
+def test_config5_ssd_mobilenet_detector(neg_ids, dev):
+    g, heads = graphgen.ssd_mobilenet(neg_ids=neg_ids, config_id="cfg5-%d" % neg_ids)
+    assert g.shape(heads[0]) == (1, 24564, 6)
+    out, tsize, ref = _run_both(g, heads, "cfg5")
+    _check(out, tsize, ref)
+    kept = (ref[0][0, :, 0] >= 0).sum()
+    assert 0 < kept <= 400
+
+
+def test_argmax_and_detection_postprocess(dev):
+    g, heads = graphgen.resnet20_cifar(1)
+    js, pb = g.build(heads, postprocess="argmax")
+    x = synth.tensor("post", "data", (1, 3, 32, 32), -127, 127)
+    m = runtime.HipModel(js, pb)
+    assert runtime.CVMAPIGetPreprocessMethod(m.net) == "argmax"
+    assert m.output_length == 4
+    out = np.frombuffer(m.inference(x.astype(np.int8).tobytes()), np.int32)
+    m.close()
+    logits = og.run_graph(js, graphgen.load_params(pb), x)[0].ravel()
+    # the reference compares the logits as int8 (src/core/model.cc:193)
+    assert out[0] == int(np.argmax(logits.astype(np.int8)))
