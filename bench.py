@@ -1,0 +1,157 @@
+#!/usr/bin/env python3
+"""Headline benchmark: images/s of the int8 ResNet-50 v1 graph (224x224) on one MI355X.
+
+A step is one pass of the graph (`CvmRuntime::Run`) over one batch that already
+sits in HBM.  The line printed at the end carries the whole-job throughput, the
+roofline position of the dominant kernel (the i8 MFMA implicit GEMM, timed with
+HIP events on the runtime's own stream while the same steps run) and the
+reference CPU runtime timed on this machine's host cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 16]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
+
+
+def cpu_baseline(js1, pb1, budget_s=20.0):
+    """Reference CPU runtime (oracle/_ref, built from the reference sources) on
+    batch-1 inputs of the same model; falls back to the C restatement when the
+    reference build is absent.  Checker code is only timed here, never used to
+    produce the GPU result."""
+    import numpy as np
+    import oracle
+    import oracle.graph as og
+    from cvm_runtime_amd import graphgen, synth
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    x = synth.tensor("bench-cpu", "data", (1, 3, 224, 224), -127, 127)
+    n = 0
+    if oracle.have_ref():
+        L = og.ref_lib()
+        net = ctypes.c_void_p()
+        gj = js1.encode()
+        rc = L.CVMAPILoadModel(ctypes.c_char_p(gj), len(gj), ctypes.c_char_p(pb1), len(pb1), ctypes.byref(net), 0, 0)
+        assert rc == 0
+        out = ctypes.create_string_buffer(4000)
+        xb = x.astype(np.int8).tobytes()
+        L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out)   # warm-up
+        t0 = time.perf_counter()
+        while True:
+            L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s or n >= 64:
+                break
+        L.CVMAPIFreeModel(net)
+        kind = "reference"
+    else:
+        params = graphgen.load_params(pb1)
+        og.run_graph(js1, params, x)
+        t0 = time.perf_counter()
+        while True:
+            og.run_graph(js1, params, x)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s or n >= 64:
+                break
+        kind = "port"
+    return {"value": n / dt, "unit": "images/s", "cores": cores, "kind": kind,
+            "sample": "%d batch-1 CVMAPIInference calls of the same ResNet-50 graph, %.1f s" % (n, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on exactly one GPU (got --gpus %d); the path shards by batch "
+                 "with no exchange step, see DESIGN.md" % args.gpus)
+
+    import numpy as np
+    import torch
+    import __graft_entry__
+    pkg = __graft_entry__.load_package()
+    from cvm_runtime_amd import graphgen, runtime, synth
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    L = pkg.lib()
+
+    g, heads = graphgen.resnet50(args.batch)
+    js, pb = g.build(heads)
+    gmac = g.macs / 1e9
+    x = synth.tensor("bench", "data", (args.batch, 3, 224, 224), -127, 127).astype(np.int8)
+    model = runtime.HipModel(js, pb)
+    model.set_input(x.tobytes())            # input resident in HBM from here on
+    model.time_run(max(args.warmup, 1))
+    torch.cuda.synchronize()
+
+    # timed region: exactly `steps` graph runs, with per-kernel event pairs around the implicit-GEMM launches
+    L.cvmhip_kernel_timing_begin()
+    t0 = time.perf_counter()
+    dev_ms = model.time_run(args.steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    buf = ctypes.create_string_buffer(1 << 16)
+    pkg.check(L.cvmhip_kernel_timing_end(buf, len(buf)))
+    kt = json.loads(buf.value.decode())
+
+    # the same steps without the event pairs, to show what the instrumentation costs
+    t0 = time.perf_counter()
+    model.time_run(args.steps)
+    torch.cuda.synchronize()
+    wall_plain = time.perf_counter() - t0
+    out = np.frombuffer(model.get_output(), np.int32)
+    model.close()
+
+    conv = kt.get("k_conv_igemm", {"launches": 0, "ms": 0.0, "work": 0.0})
+    launches = max(conv["launches"], 1)
+    ops_per_launch = conv["work"] / launches
+    avg_s = conv["ms"] / 1e3 / launches
+    achieved = ops_per_launch / avg_s / 1e12 if avg_s > 0 else 0.0
+    step_s = min(wall, wall_plain) / args.steps
+    line = {
+        "metric": "images/sec int8 ResNet-50 (224x224), one MI355X, input resident in HBM",
+        "value": args.batch / step_s,
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {"workload": "cfg3 ResNet-50 v1 quantised graph, batch %d, 3x224x224 int8, random int8 weights" % args.batch,
+                   "batch": args.batch, "graph_nodes": len(g.nodes), "gmac_per_step": gmac,
+                   "device_ms_per_step": dev_ms / args.steps,
+                   "ms_per_step_with_kernel_events": wall / args.steps * 1e3,
+                   "ms_per_step_without_kernel_events": wall_plain / args.steps * 1e3,
+                   "output_checksum": int(np.bitwise_xor.reduce(out.view(np.uint32)))},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_I8_TOPS, "unit": "TOP/s",
+                     "frac": achieved / PEAK_I8_TOPS, "traffic": None,
+                     "kernel": "k_conv_igemm", "launches_per_step": conv["launches"] / args.steps,
+                     "avg_launch_us": avg_s * 1e6, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
+                     "kernel_ms_per_step": conv["ms"] / args.steps,
+                     "other_kernels_ms_per_step": {k: v["ms"] / args.steps for k, v in kt.items() if k != "k_conv_igemm"}},
+    }
+    if not args.no_cpu_baseline:
+        g1, h1 = graphgen.resnet50(1)
+        js1, pb1 = g1.build(h1)
+        line["cpu_baseline"] = cpu_baseline(js1, pb1)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -11,6 +11,7 @@ enum { OUT_I32_NCHW = 0, OUT_I8_NHWC = 1 };
 
 struct ConvGeom {
   int N, H, W, Cp;         // input: int8 NHWC, channels padded to Cp
+  int C;                   // true channel count (0 = unknown, only used to count algorithmic work)
   int OC, OH, OW;          // output extent
   int KH, KW, SH, SW, PH, PW, DH, DW;
   int taps, K, Kp;         // filled by conv_igemm: KH*KW, taps*Cp, K rounded up to 64

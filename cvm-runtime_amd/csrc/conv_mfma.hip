@@ -356,6 +356,7 @@ int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStre
   const int cp = pad_channels(c);
   const int64_t total = (int64_t)n * (cp / 4) * hw;
   if (total == 0) return CVMHIP_OK;
+  KernelTimer timer("k_pack_nhwc", (double)n * c * hw * 5.0, s);  // bytes: 4 read + 1 written per element
   k_pack_nhwc<<<grid_for(total, 256), 256, 0, s>>>(x, xp, total, c, hw, cp);
   return check_launch("pack_nhwc");
 }
@@ -405,6 +406,8 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   const int64_t nb = blocks(64 * wm, 64 * wn);
   if (nb > 0x7fffffff) return arg_error("conv grid too large");
   const unsigned grid = (unsigned)nb;
+  // algorithmic work of this launch: 2 * pixels * OC * (true channels * taps); padding not counted
+  KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
   if (wm == 2 && wn == 2) launch_tile<2, 2>(gran, grid, s, xp, wp, out, g, ep);
   else if (wm == 1 && wn == 2) launch_tile<1, 2>(gran, grid, s, xp, wp, out, g, ep);
   else if (wm == 2 && wn == 1) launch_tile<2, 1>(gran, grid, s, xp, wp, out, g, ep);
@@ -451,7 +454,7 @@ int cvmhip_conv2d(const int32_t* x, const int32_t* w, const int32_t* bias, int32
   rc = pack_weights(w, wp, oc, ic, kh, kw, s);
   if (rc) return rc;
   ConvGeom g = {};
-  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic);
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
   g.OC = oc; g.OH = oh; g.OW = ow;
   g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
   Epilogue ep = {};
@@ -484,7 +487,7 @@ int cvmhip_dense(const int32_t* x, const int32_t* w, const int32_t* bias, int32_
   rc = pack_weights(w, wp, n, k, 1, 1, s);
   if (rc) return rc;
   ConvGeom g = {};
-  g.N = m; g.H = 1; g.W = 1; g.Cp = pad_channels(k);
+  g.N = m; g.H = 1; g.W = 1; g.Cp = pad_channels(k); g.C = k;
   g.OC = n; g.OH = 1; g.OW = 1;
   g.KH = g.KW = g.SH = g.SW = g.DH = g.DW = 1;
   Epilogue ep = {};
@@ -519,7 +522,7 @@ int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, 
   int rc = pack_activations(x, xp, n, ic, h * wd, s);
   if (rc) return rc;
   ConvGeom g = {};
-  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic);
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
   g.OC = oc;
   g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
   g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;

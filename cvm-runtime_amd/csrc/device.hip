@@ -13,7 +13,34 @@ using namespace cvmhip;
     }                                                               \
   } while (0)
 
+#include <string.h>
+#include <map>
+#include <string>
+#include <vector>
+
 namespace cvmhip {
+
+namespace {
+struct TimedLaunch { std::string name; double work; hipEvent_t e0, e1; };
+bool g_timing = false;
+std::vector<TimedLaunch> g_launches;
+}  // namespace
+
+bool kernel_timing_enabled() { return g_timing; }
+
+void kernel_timing_mark(const char* name, double work, hipStream_t s, bool start) {
+  if (start) {
+    TimedLaunch t;
+    t.name = name;
+    t.work = work;
+    if (hipEventCreate(&t.e0) != hipSuccess || hipEventCreate(&t.e1) != hipSuccess) return;
+    hipEventRecord(t.e0, s);
+    g_launches.push_back(t);
+  } else if (!g_launches.empty()) {
+    hipEventRecord(g_launches.back().e1, s);
+  }
+}
+
 __global__ void __launch_bounds__(256) k_fill32(int32_t* p, int32_t v, size_t n) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
@@ -85,6 +112,46 @@ int cvmhip_stream_destroy(void* stream) {
 
 int cvmhip_stream_sync(void* stream) {
   HIP_TRY(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize");
+  return CVMHIP_OK;
+}
+
+// Timing is process-wide and meant for a single-threaded measurement harness.
+int cvmhip_kernel_timing_begin(void) {
+  g_launches.clear();
+  g_timing = true;
+  return CVMHIP_OK;
+}
+
+// Writes {"kernel": {"launches": n, "ms": total, "work": total}, ...}
+int cvmhip_kernel_timing_end(char* json_out, int capacity) {
+  g_timing = false;
+  HIP_TRY(hipDeviceSynchronize(), "kernel_timing_end");
+  struct Acc { long n = 0; double ms = 0, work = 0; };
+  std::map<std::string, Acc> acc;
+  for (TimedLaunch& t : g_launches) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, t.e0, t.e1) == hipSuccess) {
+      Acc& a = acc[t.name];
+      a.n += 1;
+      a.ms += ms;
+      a.work += t.work;
+    }
+    hipEventDestroy(t.e0);
+    hipEventDestroy(t.e1);
+  }
+  g_launches.clear();
+  std::string out = "{";
+  bool first = true;
+  for (const auto& kv : acc) {
+    char buf[256];
+    snprintf(buf, sizeof(buf), "%s\"%s\": {\"launches\": %ld, \"ms\": %.6f, \"work\": %.6e}", first ? "" : ", ",
+             kv.first.c_str(), kv.second.n, kv.second.ms, kv.second.work);
+    out += buf;
+    first = false;
+  }
+  out += "}";
+  if (!json_out || (int)out.size() >= capacity) return arg_error("kernel_timing_end buffer");
+  memcpy(json_out, out.c_str(), out.size() + 1);
   return CVMHIP_OK;
 }
 

@@ -31,6 +31,25 @@ inline int arg_error(const char* what) {
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Optional per-kernel timing (cvmhip_kernel_timing_begin/end): while enabled,
+// launches bracketed by KernelTimer record a HIP event pair on the launch
+// stream; totals per kernel name are read back when timing ends.
+bool kernel_timing_enabled();
+void kernel_timing_mark(const char* name, double work, hipStream_t s, bool start);
+
+struct KernelTimer {
+  const char* name;
+  hipStream_t s;
+  bool on;
+  // `work` = algorithmic operations (or bytes) of this launch
+  KernelTimer(const char* n, double work, hipStream_t st) : name(n), s(st), on(kernel_timing_enabled()) {
+    if (on) kernel_timing_mark(name, work, s, true);
+  }
+  ~KernelTimer() {
+    if (on) kernel_timing_mark(name, 0, s, false);
+  }
+};
+
 // Grid for a grid-stride loop over `work` items with `block` threads: enough
 // workgroups to put several waves on each of the 256 CUs, never more than needed.
 inline unsigned grid_for(int64_t work, int block, int64_t cap = 256 * 16) {

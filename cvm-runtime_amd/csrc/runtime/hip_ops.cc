@@ -36,6 +36,9 @@ ConvDims GetConvDims(const OpCall& c) {
   d.ph = (int)a.t("padding")[0]; d.pw = (int)a.t("padding")[1];
   d.dh = (int)a.t("dilation")[0]; d.dw = (int)a.t("dilation")[1];
   d.groups = (int)a.i("groups");
+  CVM_VERIFY(w.size() == 4 && w[0] == a.i("channels") && w[1] == x[1] / d.groups && w[2] == a.t("kernel_size")[0] &&
+             w[3] == a.t("kernel_size")[1])
+      << "conv2d " << a.node_name << ": filter shape " << shape_str(w) << " does not match the data and attributes";
   return d;
 }
 

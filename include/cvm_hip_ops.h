@@ -168,6 +168,12 @@ int cvmhip_event_create(void** event);
 int cvmhip_event_destroy(void* event);
 int cvmhip_event_record(void* event, void* stream);
 int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms);
+/* Per-kernel device time for a measurement harness: between begin and end the
+ * implicit-GEMM and packing launches are bracketed by event pairs on their own
+ * stream; end synchronises and writes {"kernel": {"launches", "ms", "work"}}
+ * where work is the algorithmic operation (or byte) count of the launches. */
+int cvmhip_kernel_timing_begin(void);
+int cvmhip_kernel_timing_end(char* json_out, int capacity);
 
 /* ---- conv2d / dense with the filter packed once at model-load time.  The
  * filter of a graph node is a constant parameter, so the int32 OIHW -> int8
