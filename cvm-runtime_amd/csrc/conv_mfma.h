@@ -16,19 +16,19 @@ struct ConvGeom {
   int KH, KW, SH, SW, PH, PW, DH, DW;
   int taps, K, Kp;         // filled by conv_igemm: KH*KW, taps*Cp, K rounded up to 64
   int64_t P;               // filled by conv_igemm: N*OH*OW
+  int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
 };
 
-// What happens to an accumulator before it is stored, in this order:
-// + bias[oc], relu, cvm_right_shift, cvm_clip.
+// What happens to an accumulator before it is stored:
+//   v = chain(acc + bias[oc]);  if (residual) v = chain2(v + residual[p][oc]);
 struct Epilogue {
   const int32_t* bias;     // device pointer or nullptr
-  int relu;
-  int has_shift;
-  RShift rs;
-  int has_clip;
-  int32_t clo, chi;
+  int bias_vec;            // set by conv_igemm: bias is 16-byte aligned
+  DevChain chain;
+  const int8_t* residual;  // int8 NHWC with pitch out_cp, or nullptr
+  DevChain chain2;
   int out_mode;            // OUT_I32_NCHW or OUT_I8_NHWC
-  int out_cp;              // channel pitch of an int8 NHWC output (multiple of 4, >= OC)
+  int out_cp;              // channel pitch of int8 NHWC output / residual (multiple of 4, >= OC)
 };
 
 int pad_channels(int c);

@@ -9,12 +9,18 @@
 //   D  : int32 NCHW (the operator contract) or int8 NHWC (fused requantised output)
 //
 // One workgroup = 4 wavefronts (2 x 2) and computes a (64*WM) x (64*WN) tile of
-// D with v_mfma_i32_32x32x32_i8.  Each K step stages a 64-byte slab of both
-// operands in LDS (row pitch 80 B so the 16-byte MFMA operand reads of 8
-// consecutive lanes hit disjoint banks); the im2col addressing happens while
-// the slab is fetched, so no column buffer ever exists in HBM.  Global fetches
-// for step t+1 are issued before the MFMAs of step t and land in the other LDS
-// buffer (one barrier per step).
+// D with v_mfma_i32_32x32x32_i8.  Each K step stages a KS-byte slab (64 or 128)
+// of both operands in LDS (row pitch KS+16 bytes, so the 16-byte MFMA operand
+// reads of 8 consecutive lanes hit disjoint banks); the im2col addressing
+// happens while the slab is fetched, so no column buffer ever exists in HBM.
+// Global fetches run two K steps ahead of the MFMAs (registers hold step t+1
+// and t+2 while LDS holds t and t+1), with one barrier per step.  The int8
+// epilogue transposes the tile through LDS so that every lane writes 16
+// contiguous output bytes.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "conv_mfma.h"
 
 namespace cvmhip {
@@ -22,61 +28,61 @@ namespace cvmhip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int KSTEP = 64;   // bytes of K per LDS slab
-constexpr int LDK = 80;     // LDS row pitch in bytes
-
 __device__ __forceinline__ int4 zero4() { return make_int4(0, 0, 0, 0); }
 
-// Fetch the 16 consecutive k-bytes [kk, kk+16) of one im2col row.
-// G = bytes that are contiguous in memory for one filter tap (16 when Cp % 16 == 0,
-// else Cp itself, which is then 4 or 8).
+// Source of every out-of-image (padding) granule: loads stay unconditional and
+// the data needs no fix-up before it goes to LDS, so nothing but the loads
+// themselves sits between a fetch and the matrix instructions of that K step.
+__device__ __attribute__((aligned(16))) int g_zero_granule[4] = {0, 0, 0, 0};  // never written
+
+// Fetch the 16 consecutive k-bytes of one im2col row that start at filter tap
+// (r, s), channel c0.  G = bytes that are contiguous in memory for one filter
+// tap: 16 when Cp % 16 == 0, else Cp itself (4 or 8) and the chunk spans 16/G taps.
 template <int G>
-__device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const ConvGeom& g, bool row_ok,
-                                          int64_t img_base, int ih0, int iw0, int tap, int r, int s, int c0) {
+__device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const ConvGeom& g, bool row_ok, int img_off,
+                                          int ih0, int iw0, int tap, int r, int s, int c0) {
+  const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   if (G == 16) {
     const int ih = ih0 + r * g.DH, iw = iw0 + s * g.DW;
-    if (row_ok && tap < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
-      return *reinterpret_cast<const int4*>(xp + img_base + ((int64_t)ih * g.W + iw) * g.Cp + c0);
-    return zero4();
+    const bool ok = row_ok && tap < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+    const int8_t* src = ok ? xp + (img_off + (ih * g.W + iw) * g.Cp + c0) : zero;
+    return *reinterpret_cast<const int4*>(src);
   } else {
-    // Cp == G: each granule is a whole tap
     int v[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < 16 / G; ++j) {
       const int t = tap + j;
       const int rr = t / g.KW, ss = t - rr * g.KW;
       const int ih = ih0 + rr * g.DH, iw = iw0 + ss * g.DW;
-      if (row_ok && t < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W) {
-        const int8_t* p = xp + img_base + ((int64_t)ih * g.W + iw) * g.Cp;
-        if (G == 4) {
-          v[j] = *reinterpret_cast<const int*>(p);
-        } else {
-          const int2 u = *reinterpret_cast<const int2*>(p);
-          v[2 * j] = u.x;
-          v[2 * j + 1] = u.y;
-        }
+      const bool ok = row_ok && t < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+      const int8_t* src = ok ? xp + (img_off + (ih * g.W + iw) * g.Cp) : zero;
+      if (G == 4) {
+        v[j] = *reinterpret_cast<const int*>(src);
+      } else {
+        const int2 u = *reinterpret_cast<const int2*>(src);
+        v[2 * j] = u.x;
+        v[2 * j + 1] = u.y;
       }
     }
     return make_int4(v[0], v[1], v[2], v[3]);
   }
 }
 
-__device__ __forceinline__ int32_t requant(const Epilogue& ep, int32_t v, int oc) {
-  if (ep.bias) v = wadd(v, ep.bias[oc]);
-  if (ep.relu) v = v < 0 ? 0 : v;
-  if (ep.has_shift) v = apply_rshift(ep.rs, v);
-  if (ep.has_clip) v = v > ep.chi ? ep.chi : (v < ep.clo ? ep.clo : v);
-  return v;
-}
-
-template <int WM, int WN, int G>
+template <int WM, int WN, int G, int KS>
 __global__ void __launch_bounds__(256)
 k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void* __restrict__ out,
              const ConvGeom g, const Epilogue ep) {
-  constexpr int BM = 64 * WM;  // output channels per workgroup
-  constexpr int BN = 64 * WN;  // output pixels per workgroup
-  __shared__ __attribute__((aligned(16))) int8_t sA[2][BM * LDK];
-  __shared__ __attribute__((aligned(16))) int8_t sB[2][BN * LDK];
+  constexpr int BM = 64 * WM;        // output channels per workgroup
+  constexpr int BN = 64 * WN;        // output pixels per workgroup
+  constexpr int LDK = KS + 16;       // LDS row pitch in bytes
+  constexpr int CPR = KS / 16;       // 16-byte chunks per row and K step
+  constexpr int RPP = 256 / CPR;     // rows one pass of the workgroup covers
+  constexpr int NA = BM / RPP;       // filter chunks per thread and K step
+  constexpr int NB = BN / RPP;       // activation chunks per thread and K step
+  constexpr int OPITCH = BM + 4;     // pitch of the transposed int8 output tile (odd number of dwords)
+  static_assert(BN * OPITCH <= 2 * BM * LDK, "output tile must fit the filter staging area");
+  __shared__ __attribute__((aligned(16))) int8_t sA[2 * BM * LDK];
+  __shared__ __attribute__((aligned(16))) int8_t sB[2 * BN * LDK];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -93,34 +99,30 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   const int oc0 = (pid % oc_tiles) * BM;
   const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
 
-  // ---- per-thread fetch assignment: chunk column kc (16 B of the 64 B slab),
-  // rows tid/4 + 64*i
-  const int kc = tid & 3;
-  const int frow = tid >> 2;
+  // ---- per-thread fetch assignment: chunk column kc, rows frow + RPP*i
+  const int kc = tid % CPR;
+  const int frow = tid / CPR;
   const int OHW = g.OH * g.OW;
-  bool row_ok[WN];
-  int64_t img_base[WN];
-  int ih0[WN], iw0[WN];
+  bool row_ok[NB];
+  int img_off[NB], ih0[NB], iw0[NB];
 #pragma unroll
-  for (int i = 0; i < WN; ++i) {
-    const int64_t p = px0 + frow + 64 * i;
+  for (int i = 0; i < NB; ++i) {
+    const int64_t p = px0 + frow + RPP * i;
     row_ok[i] = p < g.P;
-    const int64_t pp = row_ok[i] ? p : 0;
-    const int n = (int)(pp / OHW);
-    const int rem = (int)(pp - (int64_t)n * OHW);
+    const int pp = row_ok[i] ? (int)p : 0;
+    const int n = pp / OHW;
+    const int rem = pp - n * OHW;
     const int oh = rem / g.OW, ow = rem - oh * g.OW;
-    img_base[i] = (int64_t)n * g.H * g.W * g.Cp;
+    img_off[i] = n * g.H * g.W * g.Cp;
     ih0[i] = oh * g.SH - g.PH;
     iw0[i] = ow * g.SW - g.PW;
   }
-  const int8_t* wrow[WM];
-#pragma unroll
-  for (int i = 0; i < WM; ++i) wrow[i] = wp + (int64_t)(oc0 + frow + 64 * i) * g.Kp + kc * 16;
+  const int8_t* wbase = wp + (int64_t)(oc0 + frow) * g.Kp + kc * 16;
 
   // position of this thread's chunk inside the (tap, channel) space
-  int kk = kc * 16;
-  int tap = kk / g.Cp, c0 = kk - tap * g.Cp;
+  int tap = (kc * 16) / g.Cp, c0 = kc * 16 - tap * g.Cp;
   int r = tap / g.KW, s = tap - r * g.KW;
+  int kbyte = 0;
 
   v16i acc[WM][WN];
 #pragma unroll
@@ -130,97 +132,163 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  int4 ra[WM], rb[WN];
-  const int nk = g.Kp / KSTEP;
+  // One K step of operands held in registers as a single SSA vector value
+  // (chunks 0..NA-1 filter, NA..NA+NB-1 activations); two of them are in flight.
+  typedef int regs_t __attribute__((ext_vector_type(4 * (NA + NB))));
+  const int nk = g.Kp / KS;
 
-  auto fetch = [&](int kt) {
+  // loads the next K step and advances the (tap, channel) cursor
+  auto fetch = [&]() -> regs_t {
+    regs_t R;
 #pragma unroll
-    for (int i = 0; i < WM; ++i) ra[i] = *reinterpret_cast<const int4*>(wrow[i] + (int64_t)kt * KSTEP);
-#pragma unroll
-    for (int i = 0; i < WN; ++i) rb[i] = fetch_act<G>(xp, g, row_ok[i], img_base[i], ih0[i], iw0[i], tap, r, s, c0);
-    // advance (tap, c0) by one K step
-    if (G == 16) {
-      c0 += KSTEP;
-      while (c0 >= g.Cp) {
-        c0 -= g.Cp;
-        ++tap;
-        if (++s == g.KW) { s = 0; ++r; }
-      }
-    } else {
-      tap += KSTEP / G;
+    for (int i = 0; i < NA; ++i) {
+      const int4 v = *reinterpret_cast<const int4*>(wbase + (int64_t)(RPP * i) * g.Kp + kbyte);
+      R[4 * i] = v.x; R[4 * i + 1] = v.y; R[4 * i + 2] = v.z; R[4 * i + 3] = v.w;
     }
-  };
-  auto stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < WM; ++i) *reinterpret_cast<int4*>(&sA[buf][(frow + 64 * i) * LDK + kc * 16]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < WN; ++i) *reinterpret_cast<int4*>(&sB[buf][(frow + 64 * i) * LDK + kc * 16]) = rb[i];
+    for (int i = 0; i < NB; ++i) {
+      const int4 v = fetch_act<G>(xp, g, row_ok[i], img_off[i], ih0[i], iw0[i], tap, r, s, c0);
+      R[4 * (NA + i)] = v.x; R[4 * (NA + i) + 1] = v.y; R[4 * (NA + i) + 2] = v.z; R[4 * (NA + i) + 3] = v.w;
+    }
+    kbyte += KS;
+    if (G == 16) {
+      // advance the cursor by KS bytes without a loop (lanes sit at different chunks)
+      c0 += g.adv_c;
+      const int carry = c0 >= g.Cp ? 1 : 0;
+      c0 -= carry ? g.Cp : 0;
+      tap += g.adv_tap + carry;
+      s += g.adv_s + carry;
+      const int wrap = s >= g.KW ? 1 : 0;
+      s -= wrap ? g.KW : 0;
+      r += g.adv_r + wrap;
+    } else {
+      tap += KS / G;
+    }
+    return R;
   };
-
-  fetch(0);
-  stage(0);
-  __syncthreads();
-
+  auto stage = [&](const regs_t R, int buf) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+      *reinterpret_cast<int4*>(&sA[(buf * BM + frow + RPP * i) * LDK + kc * 16]) =
+          make_int4(R[4 * i], R[4 * i + 1], R[4 * i + 2], R[4 * i + 3]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      *reinterpret_cast<int4*>(&sB[(buf * BN + frow + RPP * i) * LDK + kc * 16]) =
+          make_int4(R[4 * (NA + i)], R[4 * (NA + i) + 1], R[4 * (NA + i) + 2], R[4 * (NA + i) + 3]);
+  };
   const int lrow = lane & 31;
   const int lgrp = lane >> 5;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) fetch(kt + 1);
+  auto mma = [&](int buf) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KS / 32; ++ks) {
       v4i a[WM], b[WN];
 #pragma unroll
       for (int i = 0; i < WM; ++i)
-        a[i] = *reinterpret_cast<const v4i*>(&sA[cur][((wm * WM + i) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+        a[i] = *reinterpret_cast<const v4i*>(&sA[(buf * BM + (wm * WM + i) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
-        b[j] = *reinterpret_cast<const v4i*>(&sB[cur][((wn * WN + j) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+        b[j] = *reinterpret_cast<const v4i*>(&sB[(buf * BN + (wn * WN + j) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < nk) stage(cur ^ 1);
+  };
+
+  // K step kt: the register set of that parity receives step kt+2, LDS buffer
+  // kt&1 is consumed, the other register set (step kt+1, fetched one step
+  // earlier) moves to the other LDS buffer.  Fetches are unconditional -- a step
+  // past the end reads valid memory (filter rows have slack behind them, taps
+  // past the filter read the zero granule) and is never consumed -- because a conditional
+  // fetch makes the compiler wait for all outstanding loads at the join.
+  regs_t R0 = fetch();
+  regs_t R1 = fetch();
+  stage(R0, 0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt += 2) {
+    R0 = fetch();
+    mma(0);
+    stage(R1, 1);
+    __syncthreads();
+    if (kt + 1 >= nk) break;
+    R1 = fetch();
+    mma(1);
+    stage(R0, 0);
     __syncthreads();
   }
 
   // ---- epilogue.  Accumulator element e of lane l in a 32x32 tile is
   // row (e/4)*8 + (l/32)*4 + e%4 (output channel), column l%32 (pixel).
+  const bool to_i8 = ep.out_mode == OUT_I8_NHWC;
 #pragma unroll
   for (int j = 0; j < WN; ++j) {
-    const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
-    if (p >= g.P) continue;
-    const int n = (int)(p / OHW);
-    const int rem = (int)(p - (int64_t)n * OHW);
+    const int pl = (wn * WN + j) * 32 + lrow;  // pixel inside the tile
+    const int64_t p = px0 + pl;
+    const bool p_ok = p < g.P;
+    const int pp = p_ok ? (int)p : 0;
+    const int n = pp / OHW;
+    const int rem = pp - n * OHW;
+    const int8_t* res = ep.residual ? ep.residual + (int64_t)pp * ep.out_cp : nullptr;
+    int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
-      const int ocb = oc0 + (wm * WM + i) * 32 + lgrp * 4;
-      if (ep.out_mode == OUT_I32_NCHW) {
-        int32_t* y = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int oc = ocb + (e >> 2) * 8 + (e & 3);
-          if (oc < g.OC) y[(int64_t)oc * OHW] = requant(ep, acc[i][j][e], oc);
-        }
-      } else {  // OUT_I8_NHWC: 4 consecutive channels -> one 32-bit store
-        int8_t* y = reinterpret_cast<int8_t*>(out) + p * ep.out_cp;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int oc = ocb + q * 8;
-          if (oc >= ep.out_cp) continue;
-          uint32_t pack = 0;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int32_t v = (oc + e < g.OC) ? requant(ep, acc[i][j][q * 4 + e], oc + e) : 0;
-            pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * e);
+      for (int q = 0; q < 4; ++q) {  // 4 consecutive channels: one residual dword, one packed int8 dword
+        const int ol = (wm * WM + i) * 32 + lgrp * 4 + q * 8;  // channel inside the tile
+        const int oc = oc0 + ol;
+        int4 bv = zero4();
+        if (ep.bias) {
+          if (ep.bias_vec && oc + 3 < g.OC) {
+            bv = *reinterpret_cast<const int4*>(ep.bias + oc);
+          } else {
+            if (oc < g.OC) bv.x = ep.bias[oc];
+            if (oc + 1 < g.OC) bv.y = ep.bias[oc + 1];
+            if (oc + 2 < g.OC) bv.z = ep.bias[oc + 2];
+            if (oc + 3 < g.OC) bv.w = ep.bias[oc + 3];
           }
-          *reinterpret_cast<uint32_t*>(y + oc) = pack;
         }
+        uint32_t rpack = 0;
+        if (res && p_ok && oc < ep.out_cp) rpack = *reinterpret_cast<const uint32_t*>(res + oc);
+        const int32_t b4[4] = {bv.x, bv.y, bv.z, bv.w};
+        uint32_t pack = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          int32_t v = apply_chain(ep.chain, wadd(acc[i][j][q * 4 + e], b4[e]));
+          if (res) v = apply_chain(ep.chain2, wadd(v, (int32_t)(int8_t)(rpack >> (8 * e))));
+          if (oc + e >= g.OC) v = 0;
+          if (!to_i8 && p_ok && oc + e < g.OC) y32[(int64_t)(oc + e) * OHW] = v;
+          pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * e);
+        }
+        if (to_i8) *reinterpret_cast<uint32_t*>(&sA[pl * OPITCH + ol]) = pack;
+      }
+    }
+  }
+  if (to_i8) {
+    __syncthreads();
+    // each thread moves 16 contiguous output bytes of one pixel
+    constexpr int CH = BM / 16;
+    int8_t* y8 = reinterpret_cast<int8_t*>(out);
+#pragma unroll
+    for (int id = tid; id < BN * CH; id += 256) {
+      const int pl = id / CH, c16 = id - pl * CH;
+      const int64_t p = px0 + pl;
+      const int oc = oc0 + c16 * 16;
+      if (p >= g.P || oc >= ep.out_cp) continue;
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&sA[pl * OPITCH + c16 * 16]);
+      int8_t* dst = y8 + p * ep.out_cp + oc;
+      if (oc + 16 <= ep.out_cp && (ep.out_cp & 15) == 0) {
+        *reinterpret_cast<int4*>(dst) = make_int4(src[0], src[1], src[2], src[3]);
+      } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          if (oc + d * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[d] = src[d];
       }
     }
   }
 }
+
+constexpr int KSTEP = 64;  // granularity the packed filter rows are padded to
 
 // ---------------------------------------------------------------- packing
 // int32 NCHW -> int8 NHWC (channels padded to cp with zeros); narrowing is
@@ -349,7 +417,7 @@ void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp) {
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw) {
   int ocp, kp;
   weight_dims(oc, ic, kh, kw, &ocp, &kp);
-  return ((size_t)ocp * kp + 255) / 256 * 256;
+  return ((size_t)ocp * kp + 512 + 255) / 256 * 256;  // 512: fetches run up to two K steps past the end
 }
 
 int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStream_t s) {
@@ -377,25 +445,43 @@ int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, h
 }
 
 template <int WM, int WN>
-static void launch_tile(int gran, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+static void launch_tile(int gran, bool wide, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                         const ConvGeom& g, const Epilogue& ep) {
-  if (gran == 16) k_conv_igemm<WM, WN, 16><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
-  else if (gran == 8) k_conv_igemm<WM, WN, 8><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
-  else k_conv_igemm<WM, WN, 4><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  if (gran == 16) {
+    // 128-byte K steps halve the number of barriers; the 128x128 tile keeps 64 (LDS budget)
+    if constexpr (WM + WN < 4) {
+      if (wide) {
+        k_conv_igemm<WM, WN, 16, 128><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+        return;
+      }
+    }
+    k_conv_igemm<WM, WN, 16, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  } else if (gran == 8) {
+    k_conv_igemm<WM, WN, 8, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  } else {
+    k_conv_igemm<WM, WN, 4, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  }
 }
 
-int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, hipStream_t s) {
+int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
+  const Epilogue& ep0 = ep_in;
   if (g.N < 1 || g.H < 1 || g.W < 1 || g.OC < 1 || g.OH < 1 || g.OW < 1 || g.KH < 1 || g.KW < 1 || g.SH < 1 ||
       g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
     return arg_error("conv geometry");
   if (g.Cp != 4 && g.Cp != 8 && (g.Cp % 16) != 0) return arg_error("conv channel padding");
   if (((uintptr_t)xp | (uintptr_t)wp) & 15) return arg_error("conv operand alignment");
-  if (ep.out_mode == OUT_I8_NHWC && (ep.out_cp % 4 != 0 || ep.out_cp < g.OC || ((uintptr_t)out & 3)))
+  if ((ep0.out_mode == OUT_I8_NHWC || ep0.residual) && (ep0.out_cp % 4 != 0 || ep0.out_cp < g.OC))
     return arg_error("conv int8 output layout");
+  if (((uintptr_t)out | (uintptr_t)ep0.residual) & 3) return arg_error("conv output alignment");
+  if (ep0.out_mode == OUT_I8_NHWC && (ep0.out_cp & 15) == 0 && ((uintptr_t)out & 15)) return arg_error("conv output alignment");
   g.taps = g.KH * g.KW;
   g.K = g.taps * g.Cp;
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
+  if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
+  Epilogue ep = ep_in;
+  ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
+  const bool wide = (g.Kp % 128) == 0;
   const int gran = g.Cp >= 16 ? 16 : g.Cp;
   // Tile choice: the largest tile that still yields >= 2 workgroups per CU;
   // small layers fall back to smaller tiles to keep all 256 CUs busy.
@@ -403,15 +489,26 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   int wm = g.OC > 64 ? 2 : 1, wn = 2;
   if (blocks(64 * wm, 64 * wn) < 512 && wn == 2) wn = 1;
   if (blocks(64 * wm, 64 * wn) < 512 && wm == 2) wm = 1;
+  // tuning hook: CVM_HIP_TILE="wm,wn" forces a tile shape (read once)
+  static const char* forced = getenv("CVM_HIP_TILE");
+  if (forced && forced[0] >= '1' && forced[0] <= '2' && forced[1] == ',' && forced[2] >= '1' && forced[2] <= '2') {
+    wm = forced[0] - '0';
+    wn = forced[2] - '0';
+  }
   const int64_t nb = blocks(64 * wm, 64 * wn);
   if (nb > 0x7fffffff) return arg_error("conv grid too large");
   const unsigned grid = (unsigned)nb;
   // algorithmic work of this launch: 2 * pixels * OC * (true channels * taps); padding not counted
   KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
-  if (wm == 2 && wn == 2) launch_tile<2, 2>(gran, grid, s, xp, wp, out, g, ep);
-  else if (wm == 1 && wn == 2) launch_tile<1, 2>(gran, grid, s, xp, wp, out, g, ep);
-  else if (wm == 2 && wn == 1) launch_tile<2, 1>(gran, grid, s, xp, wp, out, g, ep);
-  else launch_tile<1, 1>(gran, grid, s, xp, wp, out, g, ep);
+  const int ks = (wide && wm + wn < 4) ? 128 : 64;
+  g.adv_c = ks % g.Cp;
+  g.adv_tap = ks / g.Cp;
+  g.adv_r = g.adv_tap / g.KW;
+  g.adv_s = g.adv_tap % g.KW;
+  if (wm == 2 && wn == 2) launch_tile<2, 2>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else if (wm == 1 && wn == 2) launch_tile<1, 2>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else if (wm == 2 && wn == 1) launch_tile<2, 1>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else launch_tile<1, 1>(gran, wide, grid, s, xp, wp, out, g, ep);
   return check_launch("conv_igemm");
 }
 

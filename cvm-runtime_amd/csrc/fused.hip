@@ -1,0 +1,278 @@
+// Entry points of the fused int8 path: int8 NHWC activations between layers,
+// requantisation chains folded into the producing kernel.  The arithmetic of
+// every stage is the operator's own (int32, wrapping), so results equal the
+// node-by-node execution bit for bit.
+#include "conv_mfma.h"
+
+namespace cvmhip {
+
+__device__ __forceinline__ uint32_t pack4(int32_t a, int32_t b, int32_t c, int32_t d) {
+  return (uint32_t)(uint8_t)(int8_t)a | ((uint32_t)(uint8_t)(int8_t)b << 8) | ((uint32_t)(uint8_t)(int8_t)c << 16) |
+         ((uint32_t)(uint8_t)(int8_t)d << 24);
+}
+__device__ __forceinline__ int32_t byte_of(uint32_t w, int e) { return (int32_t)(int8_t)(w >> (8 * e)); }
+
+// out = chain(a + b): one thread per (pixel, 4-channel group)
+__global__ void __launch_bounds__(256)
+k_add_i8(const uint32_t* __restrict__ a, const uint32_t* __restrict__ b, void* __restrict__ out, int out_is_i8,
+         int64_t total, int c, int cp, int hw, DevChain chain) {
+  const int c4n = cp / 4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t u = a[i], v = b[i];
+    int32_t r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = apply_chain(chain, byte_of(u, e) + byte_of(v, e));
+    if (out_is_i8) {
+      reinterpret_cast<uint32_t*>(out)[i] = pack4(r[0], r[1], r[2], r[3]);
+    } else {
+      const int c4 = (int)(i % c4n);
+      const int64_t pixel = i / c4n;
+      const int64_t n = pixel / hw;
+      const int pix = (int)(pixel - n * hw);
+      int32_t* y = reinterpret_cast<int32_t*>(out) + (n * c) * hw + pix;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c4 * 4 + e < c) y[(int64_t)(c4 * 4 + e) * hw] = r[e];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t total, int c4n, int h, int w, int oh,
+              int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int c4 = (int)(i % c4n);
+    int64_t t = i / c4n;
+    const int q = (int)(t % ow);
+    t /= ow;
+    const int p = (int)(t % oh);
+    const int64_t n = t / oh;
+    int32_t m[4] = {-128, -128, -128, -128};
+    for (int r = 0; r < kh; ++r) {
+      const int ih = p * sh + r - ph;
+      if (ih < 0 || ih >= h) continue;
+      for (int s = 0; s < kw; ++s) {
+        const int iw = q * sw + s - pw;
+        if (iw < 0 || iw >= w) continue;
+        const uint32_t v = x[((n * h + ih) * w + iw) * c4n + c4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int32_t b = byte_of(v, e);
+          m[e] = b > m[e] ? b : m[e];
+        }
+      }
+    }
+    y[i] = pack4(m[0], m[1], m[2], m[3]);
+  }
+}
+
+// out[n][c] = chain(sum_hw x[n][hw][c]): one thread per (n, 4-channel group)
+__global__ void __launch_bounds__(256)
+k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i8, int64_t total, int c, int c4n,
+            int hw, DevChain chain) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int c4 = (int)(i % c4n);
+    const int64_t n = i / c4n;
+    int32_t acc[4] = {0, 0, 0, 0};
+    const uint32_t* p = x + n * hw * c4n + c4;
+    for (int t = 0; t < hw; ++t) {
+      const uint32_t v = p[(int64_t)t * c4n];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = apply_chain(chain, acc[e]);
+    if (out_is_i8) {
+      reinterpret_cast<uint32_t*>(out)[i] = pack4(acc[0], acc[1], acc[2], acc[3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c4 * 4 + e < c) reinterpret_cast<int32_t*>(out)[n * c + c4 * 4 + e] = acc[e];
+    }
+  }
+}
+
+// depthwise: one thread per (output pixel, 4-channel group); filter is [tap][cp] int8
+__global__ void __launch_bounds__(256)
+k_depthwise_i8(const uint32_t* __restrict__ x, const uint32_t* __restrict__ wp, const int32_t* __restrict__ bias,
+               void* __restrict__ out, int out_is_i8, int64_t total, int c, int c4n, int h, int w, int oh, int ow,
+               int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw, DevChain chain) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int c4 = (int)(i % c4n);
+    int64_t t = i / c4n;
+    const int q = (int)(t % ow);
+    t /= ow;
+    const int p = (int)(t % oh);
+    const int64_t n = t / oh;
+    int32_t acc[4] = {0, 0, 0, 0};
+    for (int r = 0; r < kh; ++r) {
+      const int ih = p * sh + r * dh - ph;
+      if (ih < 0 || ih >= h) continue;
+      for (int s = 0; s < kw; ++s) {
+        const int iw = q * sw + s * dw - pw;
+        if (iw < 0 || iw >= w) continue;
+        const uint32_t v = x[((n * h + ih) * w + iw) * c4n + c4];
+        const uint32_t f = wp[(r * kw + s) * c4n + c4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e) * byte_of(f, e);
+      }
+    }
+    int32_t rr[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int ch = c4 * 4 + e;
+      rr[e] = ch < c ? apply_chain(chain, wadd(acc[e], bias ? bias[ch] : 0)) : 0;
+    }
+    if (out_is_i8) {
+      reinterpret_cast<uint32_t*>(out)[i] = pack4(rr[0], rr[1], rr[2], rr[3]);
+    } else {
+      int32_t* y = reinterpret_cast<int32_t*>(out) + ((n * c) * oh + p) * ow + q;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c4 * 4 + e < c) y[(int64_t)(c4 * 4 + e) * oh * ow] = rr[e];
+    }
+  }
+}
+
+// int32 [c][1][kh][kw] -> int8 [tap][cp]
+__global__ void __launch_bounds__(256)
+k_pack_depthwise(const int32_t* __restrict__ w, int8_t* __restrict__ wp, int64_t total, int c, int cp, int taps) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int ch = (int)(i % cp);
+    const int tap = (int)(i / cp);
+    wp[i] = ch < c ? (int8_t)w[(int64_t)ch * taps + tap] : 0;
+  }
+}
+
+}  // namespace cvmhip
+
+using namespace cvmhip;
+
+extern "C" {
+
+int cvmhip_pad_channels(int channels) { return pad_channels(channels); }
+
+int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream) {
+  if (!x || !xp || n < 1 || c < 1 || hw < 1 || ((uintptr_t)xp & 3)) return arg_error("pack_nhwc_i8");
+  return pack_activations(x, reinterpret_cast<int8_t*>(xp), n, c, hw, as_stream(stream));
+}
+
+int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void* stream) {
+  if (!x || !xp || n < 1 || c < 1 || hw < 1) return arg_error("unpack_nhwc_i8");
+  return unpack_activations(reinterpret_cast<const int8_t*>(xp), x, n, c, hw, as_stream(stream));
+}
+
+int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                     const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
+                     int n, int ic, int h, int wd, int oc, int kh, int kw,
+                     int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
+  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+    return arg_error("conv2d_i8 attributes");
+  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("conv2d_i8 kernel exceeds input");
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
+  g.OC = oc;
+  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  Epilogue ep = {};
+  ep.bias = bias;
+  if (!make_chain(chain, &ep.chain) || !make_chain(chain2, &ep.chain2)) return arg_error("conv2d_i8 chain");
+  ep.residual = reinterpret_cast<const int8_t*>(residual);
+  ep.out_mode = out_is_i8 ? OUT_I8_NHWC : OUT_I32_NCHW;
+  ep.out_cp = pad_channels(oc);
+  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep,
+                    as_stream(stream));
+}
+
+size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw) {
+  return ((size_t)pad_channels(c) * kh * kw + 255) / 256 * 256;
+}
+
+int cvmhip_pack_depthwise_weights(const int32_t* w, void* wp, int c, int kh, int kw, void* stream) {
+  if (!w || !wp || c < 1 || kh < 1 || kw < 1) return arg_error("pack_depthwise_weights");
+  const int cp = pad_channels(c);
+  const int64_t total = (int64_t)cp * kh * kw;
+  k_pack_depthwise<<<grid_for(total, 256), 256, 0, as_stream(stream)>>>(w, reinterpret_cast<int8_t*>(wp), total, c, cp,
+                                                                       kh * kw);
+  return check_launch("pack_depthwise");
+}
+
+int cvmhip_depthwise_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                               void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
+                               int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  if (!xp || !wp || !out) return arg_error("depthwise_conv2d_i8 null tensor");
+  if (n < 1 || c < 1 || h < 1 || wd < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0 ||
+      dil_h < 1 || dil_w < 1 || h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("depthwise_conv2d_i8 attributes");
+  if (((uintptr_t)xp | (uintptr_t)wp | (uintptr_t)out) & 3) return arg_error("depthwise_conv2d_i8 alignment");
+  DevChain ch;
+  if (!make_chain(chain, &ch)) return arg_error("depthwise_conv2d_i8 chain");
+  const int oh = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  const int ow = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  const int c4n = pad_channels(c) / 4;
+  const int64_t total = (int64_t)n * oh * ow * c4n;
+  hipStream_t s = as_stream(stream);
+  KernelTimer timer("k_depthwise_i8", (double)n * c * ((double)h * wd + (double)oh * ow), s);  // bytes in + out
+  k_depthwise_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(
+      reinterpret_cast<const uint32_t*>(xp), reinterpret_cast<const uint32_t*>(wp), bias, out, out_is_i8, total, c, c4n,
+      h, wd, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, ch);
+  return check_launch("depthwise_conv2d_i8");
+}
+
+int cvmhip_add_i8(const void* a, const void* b, const cvmhip_chain* chain, void* out, int out_is_i8,
+                  int n, int c, int hw, void* stream) {
+  if (!a || !b || !out || n < 1 || c < 1 || hw < 1) return arg_error("add_i8");
+  if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)out) & 3) return arg_error("add_i8 alignment");
+  DevChain ch;
+  if (!make_chain(chain, &ch)) return arg_error("add_i8 chain");
+  const int cp = pad_channels(c);
+  const int64_t total = (int64_t)n * hw * (cp / 4);
+  hipStream_t s = as_stream(stream);
+  KernelTimer timer("k_add_i8", (double)n * c * hw * 3.0, s);
+  k_add_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(a), reinterpret_cast<const uint32_t*>(b),
+                                                out, out_is_i8, total, c, cp, hw, ch);
+  return check_launch("add_i8");
+}
+
+int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, int oh, int ow,
+                         int kh, int kw, int stride_h, int stride_w, int pad_h, int pad_w, void* stream) {
+  if (!xp || !yp || n < 1 || c < 1 || h < 1 || w < 1 || oh < 1 || ow < 1 || kh < 1 || kw < 1 || stride_h < 1 ||
+      stride_w < 1 || pad_h < 0 || pad_w < 0 || pad_h >= kh || pad_w >= kw)
+    return arg_error("max_pool2d_i8");
+  // every window must touch the input, otherwise the int32 result (INT32_MIN) has no int8 form
+  if ((oh - 1) * stride_h - pad_h >= h || (ow - 1) * stride_w - pad_w >= w) return arg_error("max_pool2d_i8 window");
+  if (((uintptr_t)xp | (uintptr_t)yp) & 3) return arg_error("max_pool2d_i8 alignment");
+  const int c4n = pad_channels(c) / 4;
+  const int64_t total = (int64_t)n * oh * ow * c4n;
+  hipStream_t s = as_stream(stream);
+  KernelTimer timer("k_max_pool_i8", (double)n * c * ((double)h * w + (double)oh * ow), s);
+  k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
+                                                            reinterpret_cast<uint32_t*>(yp), total, c4n, h, w, oh, ow,
+                                                            kh, kw, stride_h, stride_w, pad_h, pad_w);
+  return check_launch("max_pool2d_i8");
+}
+
+int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int out_is_i8,
+                     int n, int c, int hw, void* stream) {
+  if (!xp || !out || n < 1 || c < 1 || hw < 1) return arg_error("sum_hw_i8");
+  if (((uintptr_t)xp | (uintptr_t)out) & 3) return arg_error("sum_hw_i8 alignment");
+  DevChain ch;
+  if (!make_chain(chain, &ch)) return arg_error("sum_hw_i8 chain");
+  const int c4n = pad_channels(c) / 4;
+  const int64_t total = (int64_t)n * c4n;
+  hipStream_t s = as_stream(stream);
+  k_sum_hw_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, c, c4n,
+                                                   hw, ch);
+  return check_launch("sum_hw_i8");
+}
+
+}  // extern "C"

@@ -108,5 +108,86 @@ __device__ __forceinline__ int32_t apply_rshift(const RShift& r, int32_t t) {
   }
 }
 
+// A requantisation chain prepared for the device.  Every stage the graph can
+// put behind a producer -- relu, cvm_clip, clip, and each regime of
+// cvm_right_shift -- has the form
+//     v = (clamp(v, lo, hi) >> s1) + add) >> s2          (add wraps)
+//   relu            : clamp to [0, INT32_MAX]
+//   clip / cvm_clip : clamp to [lo, hi]
+//   cvm_right_shift : regime "saturate"  clamp to the pre-shifted bounds, s1 = b-1, add = 1, s2 = 1
+//                     (the rounding shift is monotonic and maps the bounds to -max / max, so
+//                      clamping first equals the reference's compare-then-shift)
+//                     regime "p + b >= 32"  no clamp, s1 = b-1, add = 1, s2 = 1
+//                     regime "b >= 31"      no clamp, s1 = 31
+//                     regime "max == 0"     clamp to [0, 0]
+// so the device code is branch-free.  Adjacent pure clamps are merged on the host.
+struct DevStage {
+  int32_t lo, hi;
+  int32_t s1, add, s2;
+};
+struct DevChain {
+  int count;
+  DevStage st[4];
+};
+
+__device__ __forceinline__ int32_t apply_stage(const DevStage& s, int32_t v) {
+  v = v < s.lo ? s.lo : v;
+  v = v > s.hi ? s.hi : v;
+  return wadd(v >> s.s1, s.add) >> s.s2;
+}
+
+__device__ __forceinline__ int32_t apply_chain(const DevChain& c, int32_t v) {
+  // count is uniform across the launch: scalar branches only
+  if (c.count > 0) v = apply_stage(c.st[0], v);
+  if (c.count > 1) v = apply_stage(c.st[1], v);
+  if (c.count > 2) v = apply_stage(c.st[2], v);
+  if (c.count > 3) v = apply_stage(c.st[3], v);
+  return v;
+}
+
+inline bool stage_is_clamp(const DevStage& s) { return s.s1 == 0 && s.add == 0 && s.s2 == 0; }
+
+// host: validates and converts the C-ABI chain; returns false on a bad stage
+inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
+  out->count = 0;
+  if (!in) return true;
+  if (in->count < 0 || in->count > 4) return false;
+  for (int i = 0; i < in->count; ++i) {
+    const cvmhip_stage& s = in->stage[i];
+    DevStage d = {INT32_MIN, INT32_MAX, 0, 0, 0};
+    if (s.kind == CVMHIP_STAGE_RELU) {
+      d.lo = 0;
+    } else if (s.kind == CVMHIP_STAGE_CLIP) {
+      // max(min(v, hi), lo): with lo > hi the result is always lo
+      d.lo = s.lo;
+      d.hi = s.hi < s.lo ? s.lo : s.hi;
+    } else if (s.kind == CVMHIP_STAGE_RSHIFT) {
+      if (s.precision < 1 || s.precision > 32 || s.shift_bit < 1 || s.shift_bit > 32) return false;
+      const RShift r = make_rshift(s.precision, s.shift_bit);
+      if (r.mode == 0) { d.lo = d.hi = 0; }
+      else if (r.mode == 1) { d.s1 = 31; }
+      else {
+        d.s1 = r.sh; d.add = 1; d.s2 = 1;
+        if (r.mode == 3) { d.lo = r.x_min; d.hi = r.x_max; }
+      }
+    } else {
+      return false;
+    }
+    // merge a pure clamp into a preceding pure clamp, or into the clamp of the stage that follows it
+    if (out->count > 0 && stage_is_clamp(out->st[out->count - 1])) {
+      DevStage& p = out->st[out->count - 1];
+      // clamp(clamp(v, p.lo, p.hi), d.lo, d.hi)
+      int32_t lo = p.lo > d.lo ? p.lo : d.lo, hi = p.hi < d.hi ? p.hi : d.hi;
+      if (lo > hi) lo = hi = (p.hi < d.lo ? d.lo : d.hi);  // disjoint ranges: constant result
+      d.lo = lo;
+      d.hi = hi;
+      p = d;
+    } else {
+      out->st[out->count++] = d;
+    }
+  }
+  return true;
+}
+
 }  // namespace cvmhip
 #endif

@@ -1,0 +1,474 @@
+// Load-time planning of the fused executor.
+//
+// The reference runs one kernel per node on int32 NCHW tensors.  Inside a
+// verified graph, conv2d/dense operands are proven to fit 8 bits, and the
+// nodes that follow a conv2d / dense / elemwise_add / sum are almost always a
+// short chain of relu / cvm_right_shift / cvm_clip / clip whose result is again
+// 8 bits wide.  The planner therefore
+//   * groups  producer -> chain  into one launch whose epilogue applies the
+//     chain to the int32 accumulator (the chain's intermediate tensors are
+//     never written),
+//   * keeps group outputs that are provably within [-128, 127] as int8 NHWC
+//     between layers, converting (pack / unpack) only where a node outside the
+//     fused set, or a graph head, needs the int32 NCHW tensor,
+//   * folds a residual elemwise_add (and its own chain) into the epilogue of
+//     the convolution that produces one of its addends,
+//   * turns flatten -> dense over a 4-D tensor into a convolution whose kernel
+//     covers the whole feature map.
+// Every value a later node or the caller can observe is computed by the same
+// integer arithmetic as in node-by-node execution.
+#include <algorithm>
+#include <climits>
+
+#include "graph_runtime.h"
+
+namespace cvmrt {
+
+namespace {
+
+const uint32_t kNone = UINT32_MAX;
+
+void Check(int rc, const char* what) {
+  if (rc == CVMHIP_OK) return;
+  if (rc < CVMHIP_ERR_RUNTIME) CVM_VERIFY(false) << what << ": " << cvmhip_last_error();
+  CVM_CHECK(false) << what << ": " << cvmhip_last_error();
+}
+
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  ~DeviceBuffer() { if (ptr) cvmhip_free(ptr); }
+};
+
+struct Bound { int64_t lo = INT32_MIN, hi = INT32_MAX; };
+
+bool FitsI8(const Bound& b) { return b.lo >= -128 && b.hi <= 127; }
+
+// value range after one chain stage (only ranges that the stage itself guarantees)
+bool ChainStage(const Node& n, cvmhip_stage* st, Bound* b) {
+  const OpAttrs& a = n.attrs;
+  if (n.func_name == "relu") {
+    st->kind = CVMHIP_STAGE_RELU;
+    b->lo = std::max<int64_t>(b->lo, 0);
+    b->hi = std::max<int64_t>(b->hi, 0);
+    return true;
+  }
+  if (n.func_name == "cvm_right_shift") {
+    const int p = (int)a.i("precision"), s = (int)a.i("shift_bit");
+    st->kind = CVMHIP_STAGE_RSHIFT;
+    st->precision = p;
+    st->shift_bit = s;
+    const int64_t r = (static_cast<int64_t>(1) << (p - 1)) - 1;
+    if (r == 0) { b->lo = b->hi = 0; }
+    else if (s >= 31 || p + s >= 32) { *b = Bound(); }  // these regimes do not clip (elemwise.cc:131-137)
+    else { b->lo = -r; b->hi = r; }
+    return true;
+  }
+  if (n.func_name == "cvm_clip") {
+    const int p = (int)a.i("precision");
+    const int64_t r = (static_cast<int64_t>(1) << (p - 1)) - 1;
+    st->kind = CVMHIP_STAGE_CLIP;
+    st->lo = static_cast<int32_t>(-r);
+    st->hi = static_cast<int32_t>(r);
+    b->lo = std::max(b->lo, -r);
+    b->hi = std::min(b->hi, r);
+    return true;
+  }
+  if (n.func_name == "clip") {
+    st->kind = CVMHIP_STAGE_CLIP;
+    st->lo = (int32_t)a.i("a_min");
+    st->hi = (int32_t)a.i("a_max");
+    b->lo = std::max<int64_t>(b->lo, st->lo);
+    b->hi = std::min<int64_t>(b->hi, st->hi);
+    return true;
+  }
+  return false;
+}
+
+// operators that only move or select input values
+bool ValuePreserving(const std::string& op) {
+  static const char* kOps[] = {"relu", "max_pool2d", "flatten", "reshape", "expand_dims", "squeeze", "transpose",
+                               "concatenate", "strided_slice", "slice_like", "repeat", "tile", "upsampling"};
+  for (const char* o : kOps)
+    if (op == o) return true;
+  return false;
+}
+
+bool ConsumesI8(const std::string& op) {
+  return op == "conv2d" || op == "dense" || op == "elemwise_add" || op == "max_pool2d" || op == "sum" || op == "flatten";
+}
+
+}  // namespace
+
+void HipGraphRuntime::BuildPlan() {
+  const uint32_t ne = num_node_entries_;
+  std::vector<std::vector<uint32_t>> uses(ne);
+  std::vector<bool> is_head(ne, false), has_i8(ne, false), has_i32(ne, false), safe(ne, false);
+  std::vector<bool> absorbed(nodes_.size(), false);
+  std::vector<uint32_t> fold_src(ne, kNone);     // flatten output -> the 4-D tensor it flattens
+  std::vector<int> producer_step(ne, -1);        // plan index of the step that writes the entry's i8 form
+  std::vector<size_t> exec_of(nodes_.size(), SIZE_MAX);
+  for (size_t i = 0; i < execs_.size(); ++i) exec_of[execs_[i].nid] = i;
+  for (uint32_t nid = 0; nid < nodes_.size(); ++nid)
+    for (const NodeEntry& e : nodes_[nid].inputs) uses[entry_id(e)].push_back(nid);
+  for (const NodeEntry& e : outputs_) is_head[entry_id(e)] = true;
+
+  i8_ptr_.assign(ne, nullptr);
+  std::vector<size_t> i8_off(ne, SIZE_MAX);
+  size_t i8_bytes = 0;
+  auto i8_alloc = [&](uint32_t eid) {
+    if (i8_off[eid] != SIZE_MAX) return;
+    const Shape& s = shape_[eid];
+    const int64_t npix = s.size() == 4 ? s[0] * s[2] * s[3] : s[0];
+    i8_off[eid] = i8_bytes;
+    i8_bytes += cvmhip_packed_act_bytes(npix, (int)s[1]);
+  };
+  auto i8_capable_shape = [&](uint32_t eid) { return shape_[eid].size() == 4 || shape_[eid].size() == 2; };
+  auto pix = [&](uint32_t eid) { return shape_[eid].size() == 4 ? (int)(shape_[eid][2] * shape_[eid][3]) : 1; };
+
+  std::vector<PlanStep> plan;
+  auto need_i32 = [&](uint32_t eid) {
+    if (has_i32[eid]) return;
+    CVM_CHECK(has_i8[eid]);
+    PlanStep st;
+    st.kind = PlanStep::UNPACK;
+    st.label = "unpack_nhwc_i8";
+    st.src = st.dst = eid;
+    st.n = (int)shape_[eid][0];
+    st.c = (int)shape_[eid][1];
+    st.h = pix(eid);
+    plan.push_back(st);
+    has_i32[eid] = true;
+  };
+  auto need_i8 = [&](uint32_t eid) {
+    if (has_i8[eid]) return;
+    CVM_CHECK(has_i32[eid] && i8_capable_shape(eid));
+    i8_alloc(eid);
+    PlanStep st;
+    st.kind = PlanStep::PACK;
+    st.label = "pack_nhwc_i8";
+    st.src = st.dst = eid;
+    st.n = (int)shape_[eid][0];
+    st.c = (int)shape_[eid][1];
+    st.h = pix(eid);
+    producer_step[eid] = (int)plan.size();
+    plan.push_back(st);
+    has_i8[eid] = true;
+  };
+
+  // follows the unary chain behind `start`; returns the entry the group finally writes
+  auto follow_chain = [&](uint32_t start, cvmhip_chain* chain, Bound* bound) {
+    uint32_t cur = start;
+    chain->count = 0;
+    while (chain->count < 4 && uses[cur].size() == 1 && !is_head[cur]) {
+      const uint32_t cn = uses[cur][0];
+      const Node& c = nodes_[cn];
+      if (absorbed[cn] || c.inputs.size() != 1) break;
+      cvmhip_stage st = {};
+      Bound nb = *bound;
+      if (!ChainStage(c, &st, &nb)) break;
+      chain->stage[chain->count++] = st;
+      *bound = nb;
+      absorbed[cn] = true;
+      cur = entry_id(cn, 0);
+    }
+    return cur;
+  };
+  // where should a fused group leave its result?
+  auto wants_i8 = [&](uint32_t eid, const Bound& b) {
+    if (!FitsI8(b) || !i8_capable_shape(eid)) return false;
+    for (uint32_t cn : uses[eid])
+      if (ConsumesI8(nodes_[cn].func_name)) return true;
+    return false;
+  };
+  auto finish_output = [&](PlanStep* st, uint32_t out, const Bound& b) {
+    st->dst = out;
+    st->out_i8 = wants_i8(out, b);
+    if (st->out_i8) {
+      i8_alloc(out);
+      has_i8[out] = true;
+      safe[out] = true;
+      producer_step[out] = (int)plan.size();
+    } else {
+      has_i32[out] = true;
+      safe[out] = FitsI8(b);
+    }
+  };
+
+  for (uint32_t nid = 0; nid < nodes_.size(); ++nid) {
+    const Node& n = nodes_[nid];
+    if (n.is_variable()) {
+      const uint32_t eid = entry_id(nid, 0);
+      has_i32[eid] = true;
+      safe[eid] = precision_[eid] <= 8;  // `data` is clamped, parameters are range-checked on load
+      continue;
+    }
+    if (absorbed[nid]) continue;
+    const uint32_t out0 = entry_id(nid, 0);
+    const std::string& op = n.func_name;
+    const OpAttrs& a = n.attrs;
+    const size_t ex = exec_of[nid];
+    bool done = false;
+
+    if (op == "conv2d" || op == "dense") {
+      const uint32_t xe = entry_id(n.inputs[0]), we = entry_id(n.inputs[1]);
+      const bool has_bias = n.inputs.size() == 3;
+      const bool params_const = nodes_[n.inputs[1].node_id].is_variable() && !nodes_[n.inputs[1].node_id].is_data() &&
+                                (!has_bias || (nodes_[n.inputs[2].node_id].is_variable() && !nodes_[n.inputs[2].node_id].is_data()));
+      PlanStep st;
+      st.label = op;
+      st.bias = has_bias ? entry_ptr_[entry_id(n.inputs[2])] : nullptr;
+      bool ok = params_const;
+      uint32_t src = xe;
+      if (ok && op == "conv2d") {
+        const Shape &x = shape_[xe], &w = shape_[we];
+        const int groups = (int)a.i("groups");
+        ok = w.size() == 4 && w[0] == a.i("channels") && w[1] == x[1] / groups && w[2] == a.t("kernel_size")[0] &&
+             w[3] == a.t("kernel_size")[1];
+        st.n = (int)x[0]; st.c = (int)x[1]; st.h = (int)x[2]; st.w = (int)x[3];
+        st.oc = (int)w[0]; st.kh = (int)w[2]; st.kw = (int)w[3];
+        st.sh = (int)a.t("strides")[0]; st.sw = (int)a.t("strides")[1];
+        st.ph = (int)a.t("padding")[0]; st.pw = (int)a.t("padding")[1];
+        st.dh = (int)a.t("dilation")[0]; st.dw = (int)a.t("dilation")[1];
+        if (groups == 1) {
+          st.kind = PlanStep::CONV;
+        } else if (groups == x[1] && w[0] == x[1] && w[1] == 1 && safe[xe]) {
+          st.kind = PlanStep::DWCONV;  // exact only for operands known to fit int8: this path does not narrow
+        } else {
+          ok = false;
+        }
+      } else if (ok) {
+        st.kind = PlanStep::CONV;
+        if (fold_src[xe] != kNone) {  // flatten(4-D) -> dense == convolution over the whole map
+          src = fold_src[xe];
+          const Shape& x = shape_[src];
+          st.n = (int)x[0]; st.c = (int)x[1]; st.h = (int)x[2]; st.w = (int)x[3];
+          st.kh = st.h; st.kw = st.w;
+        } else {
+          const Shape& x = shape_[xe];
+          st.n = (int)x[0]; st.c = (int)x[1]; st.h = st.w = 1;
+        }
+        st.oc = (int)shape_[we][0];
+        ok = shape_[we].size() == 2 && shape_[we][1] == (int64_t)st.c * st.kh * st.kw;
+      }
+      if (ok) {
+        need_i8(src);
+        auto buf = std::make_shared<DeviceBuffer>();
+        if (st.kind == PlanStep::CONV) {
+          Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_weight_bytes(st.oc, st.c, st.kh, st.kw)), "filter buffer");
+          Check(cvmhip_pack_weights(entry_ptr_[we], buf->ptr, st.oc, st.c, st.kh, st.kw, stream_), "filter pack");
+        } else {
+          Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_depthwise_bytes(st.c, st.kh, st.kw)), "filter buffer");
+          Check(cvmhip_pack_depthwise_weights(entry_ptr_[we], buf->ptr, st.c, st.kh, st.kw, stream_), "filter pack");
+        }
+        st.weights = buf;
+        st.src = src;
+        st.src2 = kNone;
+        Bound b;
+        const uint32_t out = follow_chain(out0, &st.chain, &b);
+        finish_output(&st, out, b);
+        plan.push_back(st);
+        done = true;
+      }
+    } else if (op == "elemwise_add") {
+      const uint32_t ae = entry_id(n.inputs[0]), be = entry_id(n.inputs[1]);
+      if (has_i8[ae] && has_i8[be] && safe[ae] && safe[be] && ae != be) {
+        cvmhip_chain chain;
+        Bound b;
+        b.lo = -256;
+        b.hi = 254;
+        const uint32_t out = follow_chain(out0, &chain, &b);
+        // fold into the convolution that produced one addend, when the other addend exists by then
+        bool folded = false;
+        for (int swap = 0; swap < 2 && !folded; ++swap) {
+          const uint32_t x = swap ? be : ae, r = swap ? ae : be;
+          const int ps = producer_step[x], pr = producer_step[r];
+          if (ps < 0 || pr < 0 || pr >= ps) continue;
+          PlanStep& cs = plan[ps];
+          if (cs.kind != PlanStep::CONV || cs.dst != x || !cs.out_i8 || cs.src2 != kNone) continue;
+          if (uses[x].size() != 1 || is_head[x]) continue;
+          cs.src2 = r;
+          cs.chain2 = chain;
+          cs.label += "+add";
+          // the conv now writes the add group's output instead of its own
+          has_i8[x] = false;
+          cs.dst = out;
+          cs.out_i8 = wants_i8(out, b);
+          if (cs.out_i8) {
+            i8_alloc(out);
+            has_i8[out] = true;
+            safe[out] = true;
+            producer_step[out] = ps;
+          } else {
+            has_i32[out] = true;
+            safe[out] = FitsI8(b);
+          }
+          folded = true;
+        }
+        if (!folded) {
+          PlanStep st;
+          st.kind = PlanStep::ADD;
+          st.label = "elemwise_add";
+          st.src = ae;
+          st.src2 = be;
+          st.chain = chain;
+          st.n = (int)shape_[ae][0];
+          st.c = (int)shape_[ae][1];
+          st.h = pix(ae);
+          finish_output(&st, out, b);
+          plan.push_back(st);
+        }
+        done = true;
+      }
+    } else if (op == "max_pool2d") {
+      const uint32_t xe = entry_id(n.inputs[0]);
+      if (has_i8[xe] && safe[xe]) {
+        PlanStep st;
+        st.kind = PlanStep::POOL;
+        st.label = op;
+        st.src = xe;
+        const Shape &x = shape_[xe], &y = shape_[out0], &pad = a.t("padding");
+        st.n = (int)x[0]; st.c = (int)x[1]; st.h = (int)x[2]; st.w = (int)x[3];
+        st.oh = (int)y[2]; st.ow = (int)y[3];
+        st.kh = (int)a.t("pool_size")[0]; st.kw = (int)a.t("pool_size")[1];
+        st.sh = (int)a.t("strides")[0]; st.sw = (int)a.t("strides")[1];
+        st.ph = (int)pad[0]; st.pw = pad.size() == 2 ? (int)pad[1] : (int)pad[0];
+        Bound b;
+        b.lo = -128;
+        b.hi = 127;
+        finish_output(&st, out0, b);
+        if (st.out_i8) {
+          plan.push_back(st);
+          done = true;
+        } else {  // nobody downstream reads int8: leave the node to the int32 kernel
+          has_i32[out0] = false;
+        }
+      }
+    } else if (op == "sum") {
+      const uint32_t xe = entry_id(n.inputs[0]);
+      Shape ax = a.t("axis");
+      for (auto& v : ax) v = v < 0 ? v + 4 : v;
+      std::sort(ax.begin(), ax.end());
+      if (has_i8[xe] && safe[xe] && shape_[xe].size() == 4 && ax == Shape{2, 3} && !a.b("exclude")) {
+        PlanStep st;
+        st.kind = PlanStep::SUM;
+        st.label = op;
+        st.src = xe;
+        st.n = (int)shape_[xe][0];
+        st.c = (int)shape_[xe][1];
+        st.h = pix(xe);
+        Bound b;
+        const uint32_t out = follow_chain(out0, &st.chain, &b);
+        // (N, C) and (N, C, 1, 1) share one memory image
+        const Shape& os = shape_[out];
+        const bool flat = os.size() == 2 || (os.size() == 4 && os[2] == 1 && os[3] == 1);
+        st.dst = out;
+        st.out_i8 = flat && wants_i8(out, b);
+        if (st.out_i8) {
+          i8_alloc(out);
+          has_i8[out] = true;
+          safe[out] = true;
+          producer_step[out] = (int)plan.size();
+        } else {
+          has_i32[out] = true;
+          safe[out] = FitsI8(b);
+        }
+        plan.push_back(st);
+        done = true;
+      }
+    } else if (op == "flatten") {
+      const uint32_t xe = entry_id(n.inputs[0]);
+      if (has_i8[xe] && !is_head[out0] && uses[out0].size() == 1) {
+        const Node& c = nodes_[uses[out0][0]];
+        const Shape& x = shape_[xe];
+        bool to_dense = c.func_name == "dense" && entry_id(c.inputs[0]) == out0;
+        for (size_t k = 1; to_dense && k < c.inputs.size(); ++k)
+          to_dense = nodes_[c.inputs[k].node_id].is_variable() && !nodes_[c.inputs[k].node_id].is_data();
+        if (to_dense && x.size() == 4 && (x[2] > 1 || x[3] > 1) && x[2] <= 64 && x[3] <= 64) {
+          fold_src[out0] = xe;  // the dense becomes a convolution over xe
+          done = true;
+        } else if (to_dense && (x.size() == 2 || (x.size() == 4 && x[2] == 1 && x[3] == 1))) {
+          i8_off[out0] = i8_off[xe];  // same bytes, other logical shape
+          has_i8[out0] = true;
+          safe[out0] = safe[xe];
+          producer_step[out0] = producer_step[xe];
+          done = true;
+        }
+      }
+    }
+
+    if (done) continue;
+    // ---- the node runs as its own int32 kernel
+    for (const NodeEntry& e : n.inputs) need_i32(entry_id(e));
+    PlanStep st;
+    st.kind = PlanStep::NODE;
+    st.label = op;
+    st.exec_index = ex;
+    plan.push_back(st);
+    bool all_safe = true;
+    for (const NodeEntry& e : n.inputs) all_safe = all_safe && safe[entry_id(e)];
+    for (uint32_t i = 0; i < n.num_outputs; ++i) {
+      const uint32_t eid = entry_id(nid, i);
+      has_i32[eid] = true;
+      cvmhip_stage tmp = {};
+      Bound b;
+      if (ValuePreserving(op)) safe[eid] = all_safe;
+      else if (n.inputs.size() == 1 && ChainStage(n, &tmp, &b)) safe[eid] = FitsI8(b);
+    }
+  }
+  for (const NodeEntry& e : outputs_) need_i32(entry_id(e));
+
+  if (i8_bytes > 0) {
+    Check(cvmhip_alloc(&i8_slab_, i8_bytes), "allocate int8 activation storage");
+    for (uint32_t e = 0; e < ne; ++e)
+      if (i8_off[e] != SIZE_MAX) i8_ptr_[e] = static_cast<char*>(i8_slab_) + i8_off[e];
+  }
+  plan_ = std::move(plan);
+  fused_ = true;
+}
+
+void HipGraphRuntime::RunStep(PlanStep& st) {
+  switch (st.kind) {
+    case PlanStep::NODE: {
+      Exec& ex = execs_[st.exec_index];
+      ex.kernel->run(ex.call);
+      break;
+    }
+    case PlanStep::PACK:
+      Check(cvmhip_pack_nhwc_i8(entry_ptr_[st.src], i8_ptr_[st.dst], st.n, st.c, st.h, stream_), "pack");
+      break;
+    case PlanStep::UNPACK:
+      Check(cvmhip_unpack_nhwc_i8(i8_ptr_[st.src], entry_ptr_[st.dst], st.n, st.c, st.h, stream_), "unpack");
+      break;
+    case PlanStep::CONV: {
+      void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
+      Check(cvmhip_conv2d_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res,
+                             &st.chain2, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh,
+                             st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "conv2d_i8");
+      break;
+    }
+    case PlanStep::DWCONV: {
+      void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      Check(cvmhip_depthwise_conv2d_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias,
+                                       &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.kh, st.kw, st.sh,
+                                       st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "depthwise_conv2d_i8");
+      break;
+    }
+    case PlanStep::ADD: {
+      void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      Check(cvmhip_add_i8(i8_ptr_[st.src], i8_ptr_[st.src2], &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, stream_), "add_i8");
+      break;
+    }
+    case PlanStep::POOL:
+      Check(cvmhip_max_pool2d_i8(i8_ptr_[st.src], i8_ptr_[st.dst], st.n, st.c, st.h, st.w, st.oh, st.ow, st.kh, st.kw,
+                                 st.sh, st.sw, st.ph, st.pw, stream_), "max_pool2d_i8");
+      break;
+    case PlanStep::SUM: {
+      void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      Check(cvmhip_sum_hw_i8(i8_ptr_[st.src], &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, stream_), "sum_hw_i8");
+      break;
+    }
+  }
+}
+
+}  // namespace cvmrt

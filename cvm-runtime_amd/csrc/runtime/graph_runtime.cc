@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <iostream>
 #include <unordered_set>
@@ -440,7 +441,9 @@ HipGraphRuntime::HipGraphRuntime(const std::string& graph_json, int device_id, b
 }
 
 void HipGraphRuntime::Release() {
+  plan_.clear();
   execs_.clear();  // releases per-node device state before the stream goes away
+  if (i8_slab_) { cvmhip_free(i8_slab_); i8_slab_ = nullptr; }
   if (stream_) cvmhip_stream_sync(stream_);
   if (workspace_) cvmhip_free(workspace_);
   if (slab_) cvmhip_free(slab_);
@@ -594,13 +597,19 @@ void HipGraphRuntime::LoadParams(const std::string& blob) {
   }
   for (Exec& ex : execs_)
     if (ex.kernel->prepare) ex.kernel->prepare(ex.call);
+  const char* fuse = std::getenv("CVM_HIP_FUSE");
+  if (fuse == nullptr || std::string(fuse) != "0") BuildPlan();
   HipCheck(cvmhip_stream_sync(stream_), "prepare operators");
   params_loaded_ = true;
 }
 
 // ---------------------------------------------------------------- execution
 void HipGraphRuntime::Run() {
-  for (Exec& ex : execs_) ex.kernel->run(ex.call);
+  if (fused_) {
+    for (PlanStep& st : plan_) RunStep(st);
+  } else {
+    for (Exec& ex : execs_) ex.kernel->run(ex.call);
+  }
 }
 
 std::map<std::string, double> HipGraphRuntime::ProfileRun() {
@@ -608,13 +617,15 @@ std::map<std::string, double> HipGraphRuntime::ProfileRun() {
   void *e0 = nullptr, *e1 = nullptr;
   HipCheck(cvmhip_event_create(&e0), "event");
   HipCheck(cvmhip_event_create(&e1), "event");
-  for (Exec& ex : execs_) {
+  const size_t count = fused_ ? plan_.size() : execs_.size();
+  for (size_t i = 0; i < count; ++i) {
     HipCheck(cvmhip_event_record(e0, stream_), "event");
-    ex.kernel->run(ex.call);
+    if (fused_) RunStep(plan_[i]);
+    else execs_[i].kernel->run(execs_[i].call);
     HipCheck(cvmhip_event_record(e1, stream_), "event");
     float ms = 0;
     HipCheck(cvmhip_event_elapsed_ms(e0, e1, &ms), "event");
-    times[ex.call.op] += ms;
+    times[fused_ ? plan_[i].label : execs_[i].call.op] += ms;
   }
   cvmhip_event_destroy(e0);
   cvmhip_event_destroy(e1);

@@ -15,6 +15,7 @@
 #include <string>
 #include <vector>
 
+#include "../../../include/cvm_hip_ops.h"
 #include "base.h"
 #include "json.h"
 #include "op_schema.h"
@@ -87,6 +88,19 @@ struct Node {
   bool is_data() const { return is_variable() && name == "data"; }
 };
 
+// One launch of the fused executor (fused_plan.cc).
+struct PlanStep {
+  enum Kind { NODE, PACK, UNPACK, CONV, DWCONV, ADD, POOL, SUM } kind = NODE;
+  std::string label;            // operator name for the time table
+  size_t exec_index = 0;        // NODE: index into execs_
+  uint32_t src = 0, src2 = 0, dst = 0;  // entry ids (src2: residual / second addend; UINT32_MAX = none)
+  bool out_i8 = false;
+  cvmhip_chain chain{}, chain2{};
+  const int32_t* bias = nullptr;
+  std::shared_ptr<void> weights;  // packed filter (device)
+  int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;
+};
+
 class HipGraphRuntime {
  public:
   // with_device == false parses and verifies only (gas estimation from a graph file)
@@ -120,6 +134,9 @@ class HipGraphRuntime {
   // elapsed device milliseconds of `iterations` back-to-back Run() calls
   float TimeRuns(int iterations);
   size_t NumNodes() const { return nodes_.size(); }
+  // number of launches per Run(): nodes when unfused, plan steps when fused
+  size_t NumSteps() const { return fused_ ? plan_.size() : execs_.size(); }
+  bool fused() const { return fused_; }
 
  private:
   uint32_t entry_id(uint32_t nid, uint32_t index) const { return node_row_ptr_[nid] + index; }
@@ -159,6 +176,14 @@ class HipGraphRuntime {
   struct Exec { uint32_t nid; const OpKernel* kernel; OpCall call; };
   std::vector<Exec> execs_;
   bool params_loaded_ = false;
+
+  // ---- fused executor: int8 NHWC activations + folded requantisation chains
+  void BuildPlan();
+  void RunStep(PlanStep& st);
+  bool fused_ = false;
+  std::vector<PlanStep> plan_;
+  std::vector<void*> i8_ptr_;      // per entry: int8 NHWC form (nullptr if never materialised)
+  void* i8_slab_ = nullptr;
 };
 
 }  // namespace cvmrt
