@@ -288,3 +288,130 @@ def non_max_suppression(x, valid_count, y, iou_threshold=50, force_suppress=Fals
                                        int(bool(force_suppress)), ctypes.c_void_p(ws.data_ptr()),
                                        ctypes.c_size_t(ws.numel()), _stream()))
     return y
+
+
+# ---------------------------------------------------------------- fused int8 path
+# int8 NHWC tensors are torch int8 tensors of shape (n, h*w, cp); filters are
+# opaque byte buffers made by pack_weights / pack_depthwise_weights.
+
+class Stage(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int32), ("precision", ctypes.c_int32), ("shift_bit", ctypes.c_int32),
+                ("lo", ctypes.c_int32), ("hi", ctypes.c_int32)]
+
+
+class Chain(ctypes.Structure):
+    _fields_ = [("count", ctypes.c_int32), ("stage", Stage * 4)]
+
+
+def chain(*stages):
+    """stages: ("relu",) | ("cvm_right_shift", precision, shift_bit) | ("cvm_clip", precision) | ("clip", lo, hi)"""
+    c = Chain()
+    c.count = len(stages)
+    for i, st in enumerate(stages):
+        if st[0] == "relu":
+            c.stage[i] = Stage(1, 0, 0, 0, 0)
+        elif st[0] == "cvm_right_shift":
+            c.stage[i] = Stage(2, st[1], st[2], 0, 0)
+        elif st[0] == "cvm_clip":
+            r = (1 << (st[1] - 1)) - 1
+            c.stage[i] = Stage(3, 0, 0, -r, r)
+        elif st[0] == "clip":
+            c.stage[i] = Stage(3, 0, 0, st[1], st[2])
+        else:
+            raise ValueError(st)
+    return c
+
+
+def _vp(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def pad_channels(c):
+    return lib().cvmhip_pad_channels(c)
+
+
+def pack_nhwc_i8(x):
+    n, c, h, w = x.shape
+    xp = torch.empty((n, h * w, pad_channels(c)), dtype=torch.int8, device=x.device)
+    check(lib().cvmhip_pack_nhwc_i8(_ptr(x), _vp(xp), n, c, h * w, _stream()))
+    return xp
+
+
+def unpack_nhwc_i8(xp, c, h, w):
+    n = xp.shape[0]
+    x = torch.empty((n, c, h, w), dtype=torch.int32, device=xp.device)
+    check(lib().cvmhip_unpack_nhwc_i8(_vp(xp), _ptr(x), n, c, h * w, _stream()))
+    return x
+
+
+def pack_weights(w):
+    oc, ic, kh, kw = w.shape
+    wp = _workspace(lib().cvmhip_packed_weight_bytes(oc, ic, kh, kw), w.device)
+    check(lib().cvmhip_pack_weights(_ptr(w), _vp(wp), oc, ic, kh, kw, _stream()))
+    return wp
+
+
+def conv2d_i8(xp, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=None, chain2=None, out_is_i8=True,
+              strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    n = xp.shape[0]
+    oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    if out_is_i8:
+        out = torch.empty((n, oh * ow, pad_channels(oc)), dtype=torch.int8, device=xp.device)
+    else:
+        out = torch.empty((n, oc, oh, ow), dtype=torch.int32, device=xp.device)
+    check(lib().cvmhip_conv2d_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
+                                 _vp(residual), ctypes.byref(chain2) if chain2 else None, _vp(out), int(out_is_i8),
+                                 n, ic, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                 dilation[0], dilation[1], _stream()))
+    return out
+
+
+def pack_depthwise_weights(w):
+    c, one, kh, kw = w.shape
+    wp = _workspace(lib().cvmhip_packed_depthwise_bytes(c, kh, kw), w.device)
+    check(lib().cvmhip_pack_depthwise_weights(_ptr(w), _vp(wp), c, kh, kw, _stream()))
+    return wp
+
+
+def depthwise_conv2d_i8(xp, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_i8=True,
+                        strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    n = xp.shape[0]
+    oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    if out_is_i8:
+        out = torch.empty((n, oh * ow, pad_channels(c)), dtype=torch.int8, device=xp.device)
+    else:
+        out = torch.empty((n, c, oh, ow), dtype=torch.int32, device=xp.device)
+    check(lib().cvmhip_depthwise_conv2d_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
+                                           _vp(out), int(out_is_i8), n, c, h, w, kh, kw, strides[0], strides[1],
+                                           padding[0], padding[1], dilation[0], dilation[1], _stream()))
+    return out
+
+
+def add_i8(a, b, c, h, w, chain1=None, out_is_i8=True):
+    n = a.shape[0]
+    if out_is_i8:
+        out = torch.empty_like(a)
+    else:
+        out = torch.empty((n, c, h, w), dtype=torch.int32, device=a.device)
+    check(lib().cvmhip_add_i8(_vp(a), _vp(b), ctypes.byref(chain1) if chain1 else None, _vp(out), int(out_is_i8),
+                              n, c, h * w, _stream()))
+    return out
+
+
+def max_pool2d_i8(xp, c, h, w, pool_size, strides, padding, oh, ow):
+    n = xp.shape[0]
+    out = torch.empty((n, oh * ow, xp.shape[2]), dtype=torch.int8, device=xp.device)
+    check(lib().cvmhip_max_pool2d_i8(_vp(xp), _vp(out), n, c, h, w, oh, ow, pool_size[0], pool_size[1],
+                                     strides[0], strides[1], padding[0], padding[1], _stream()))
+    return out
+
+
+def sum_hw_i8(xp, c, hw, chain1=None, out_is_i8=False):
+    n = xp.shape[0]
+    if out_is_i8:
+        out = torch.empty((n, 1, xp.shape[2]), dtype=torch.int8, device=xp.device)
+    else:
+        out = torch.empty((n, c), dtype=torch.int32, device=xp.device)
+    check(lib().cvmhip_sum_hw_i8(_vp(xp), ctypes.byref(chain1) if chain1 else None, _vp(out), int(out_is_i8),
+                                 n, c, hw, _stream()))
+    return out

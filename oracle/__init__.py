@@ -159,7 +159,7 @@ def cvm_precision(x):
 def elemwise(op, a, b):
     a, b = _a(a), _a(b)
     c = np.empty_like(a)
-    rc = lib().cvmo_elemwise(0 if op == "elemwise_add" else 1, _p(a), _p(b), _p(c),
+    rc = lib().cvmo_elemwise({"elemwise_add": 0, "elemwise_sub": 1}[op], _p(a), _p(b), _p(c),
                              ctypes.c_int64(a.size))
     assert rc == 0
     return c

@@ -1,0 +1,207 @@
+"""GPU parity of the fused int8 entry points (include/cvm_hip_ops.h, "fused int8
+path") against the CPU oracle running the same nodes one by one, and of the
+fused graph executor against the node-by-node executor.  Bit-exact."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import oracle.graph as og
+from cvm_runtime_amd import graphgen, hipops, runtime, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def T(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(dev)
+
+
+def nhwc_to_nchw(t, c, h, w):
+    """int8 NHWC (n, h*w, cp) device tensor -> int32 NCHW numpy, padding channels dropped (and checked zero)."""
+    torch.cuda.synchronize()
+    a = t.cpu().numpy().astype(np.int32)
+    n = a.shape[0]
+    assert not a[:, :, c:].any(), "padding channels must stay zero"
+    return np.ascontiguousarray(a[:, :, :c].reshape(n, h, w, c).transpose(0, 3, 1, 2))
+
+
+def run_chain(v, stages):
+    for st in stages:
+        if st[0] == "relu":
+            v = oracle.relu(v)
+        elif st[0] == "cvm_right_shift":
+            v = oracle.cvm_right_shift(v, st[1], st[2])
+        elif st[0] == "cvm_clip":
+            v = oracle.cvm_clip(v, st[1])
+        else:
+            v = oracle.clip(v, st[1], st[2])
+    return v
+
+
+def eq(got, ref, what):
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    if not np.array_equal(got, ref):
+        bad = np.argwhere(got != ref)
+        raise AssertionError("%s: %d of %d differ, first at %s: got %d want %d" % (
+            what, len(bad), ref.size, bad[0], got[tuple(bad[0])], ref[tuple(bad[0])]))
+
+
+@pytest.mark.parametrize("c", [1, 3, 5, 8, 20, 64])
+def test_pack_unpack_round_trip(c, dev):
+    x = synth.tensor("pack-%d" % c, "x", (3, c, 7, 5), -128, 127)
+    xp = hipops.pack_nhwc_i8(T(x, dev))
+    assert xp.shape[2] == hipops.pad_channels(c) and xp.shape[2] >= c
+    eq(nhwc_to_nchw(xp, c, 7, 5), x, "pack")
+    y = hipops.unpack_nhwc_i8(xp, c, 7, 5)
+    torch.cuda.synchronize()
+    eq(y.cpu().numpy(), x, "unpack")
+
+
+def test_pack_narrows_like_static_cast(dev):
+    # values outside int8 are truncated exactly as the reference's static_cast<int8_t> (ops.cc:234)
+    x = np.array([127, 128, 255, 256, -128, -129, 1000, -1000, 2**31 - 1, -2**31], np.int64).astype(np.int32).reshape(1, 10, 1, 1)
+    xp = hipops.pack_nhwc_i8(T(x, dev))
+    eq(nhwc_to_nchw(xp, 10, 1, 1), x.astype(np.int8).astype(np.int32), "narrow")
+
+
+FUSED_CONV = [
+    # n, ic, h, w, oc, k, stride, pad, bias, chain, residual chain, int8 out
+    (2, 64, 14, 14, 64, 3, 1, 1, True, [("relu",), ("cvm_right_shift", 8, 9)], None, True),
+    (2, 64, 14, 14, 256, 1, 1, 0, False, [("cvm_right_shift", 8, 7)], [("relu",), ("cvm_right_shift", 8, 1)], True),
+    (1, 3, 33, 31, 16, 7, 2, 3, True, [("relu",), ("cvm_right_shift", 8, 10), ("cvm_clip", 8)], None, True),
+    (3, 8, 9, 9, 24, 3, 2, 1, True, [("cvm_right_shift", 8, 6), ("clip", -100, 90)], None, True),
+    (1, 32, 12, 12, 40, 3, 1, 1, True, [("cvm_right_shift", 16, 3)], None, False),      # int32 NCHW output, wide values
+    (1, 32, 12, 12, 40, 3, 1, 1, False, [], None, False),                                # no chain at all
+    (2, 128, 7, 7, 130, 1, 1, 0, True, [("cvm_right_shift", 8, 8)], [("cvm_right_shift", 8, 1), ("relu",)], True),
+    (1, 16, 6, 6, 20, 3, 1, 1, True, [("cvm_right_shift", 8, 31)], None, True),          # shift regime b >= 31
+    (1, 16, 6, 6, 20, 3, 1, 1, True, [("cvm_right_shift", 8, 24), ("cvm_clip", 8)], None, True),  # regime p + b >= 32
+    (16, 512, 7, 7, 512, 3, 1, 1, True, [("relu",), ("cvm_right_shift", 8, 12)], None, True),      # deep K (4608), few pixels
+    (4, 1024, 14, 14, 256, 1, 1, 0, False, [("relu",), ("cvm_right_shift", 8, 11)], None, True),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_CONV, ids=lambda c: "n%dc%dh%dw%d_o%dk%d" % c[:6])
+def test_conv2d_i8(case, dev):
+    n, ic, h, w, oc, k, st, pd, bias, ch1, ch2, i8 = case
+    cid = "fconv-%s" % (case[:8],)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768) if bias else None
+    ref = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1), ch1)
+    oh, ow = ref.shape[2:]
+    res_t = None
+    if ch2 is not None:
+        r = synth.tensor(cid, "r", ref.shape, -127, 127)
+        ref = run_chain(oracle.elemwise("elemwise_add", ref, r), ch2)
+        res_t = hipops.pack_nhwc_i8(T(r, dev))
+    xp = hipops.pack_nhwc_i8(T(x, dev))
+    wp = hipops.pack_weights(T(wt, dev))
+    out = hipops.conv2d_i8(xp, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None,
+                           hipops.chain(*ch1) if ch1 else None, res_t, hipops.chain(*ch2) if ch2 else None,
+                           out_is_i8=i8, strides=(st, st), padding=(pd, pd))
+    if i8:
+        assert ref.min() >= -128 and ref.max() <= 127, "case must be representable"
+        eq(nhwc_to_nchw(out, oc, oh, ow), ref, "conv2d_i8")
+    else:
+        torch.cuda.synchronize()
+        eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32")
+
+
+@pytest.mark.parametrize("case", [(2, 32, 19, 17, 3, 1, 1), (1, 96, 16, 16, 3, 2, 1), (1, 5, 9, 9, 3, 1, 0), (1, 256, 8, 8, 5, 1, 2)],
+                         ids=lambda c: "n%dc%dh%dw%dk%ds%dp%d" % c)
+def test_depthwise_conv2d_i8(case, dev):
+    n, c, h, w, k, st, pd = case
+    cid = "fdw-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (c, 1, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (c,), -3000, 3000)
+    stages = [("relu",), ("cvm_right_shift", 8, 10)]
+    ref = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), c), stages)
+    xp = hipops.pack_nhwc_i8(T(x, dev))
+    wp = hipops.pack_depthwise_weights(T(wt, dev))
+    out = hipops.depthwise_conv2d_i8(xp, c, h, w, wp, k, k, T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
+    eq(nhwc_to_nchw(out, c, ref.shape[2], ref.shape[3]), ref, "depthwise int8")
+    out32 = hipops.depthwise_conv2d_i8(xp, c, h, w, wp, k, k, T(b, dev), None, False, (st, st), (pd, pd))
+    torch.cuda.synchronize()
+    eq(out32.cpu().numpy(), oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), c), "depthwise int32")
+
+
+@pytest.mark.parametrize("c", [3, 16, 70])
+def test_add_i8(c, dev):
+    a = synth.tensor("fadd-%d" % c, "a", (2, c, 5, 7), -127, 127)
+    b = synth.tensor("fadd-%d" % c, "b", (2, c, 5, 7), -127, 127)
+    stages = [("relu",), ("cvm_right_shift", 8, 1)]
+    ref = run_chain(oracle.elemwise("elemwise_add", a, b), stages)
+    ap, bp = hipops.pack_nhwc_i8(T(a, dev)), hipops.pack_nhwc_i8(T(b, dev))
+    eq(nhwc_to_nchw(hipops.add_i8(ap, bp, c, 5, 7, hipops.chain(*stages), True), c, 5, 7), ref, "add int8")
+    out = hipops.add_i8(ap, bp, c, 5, 7, None, False)
+    torch.cuda.synchronize()
+    eq(out.cpu().numpy(), oracle.elemwise("elemwise_add", a, b), "add int32")
+
+
+@pytest.mark.parametrize("case", [(2, 64, 16, 16, 3, 2, 1, False), (1, 24, 9, 11, 2, 2, 0, False), (1, 8, 10, 10, 3, 2, 1, True)],
+                         ids=lambda c: "n%dc%dh%dw%dk%ds%dp%dceil%d" % c)
+def test_max_pool2d_i8(case, dev):
+    n, c, h, w, k, st, pd, ceil = case
+    x = synth.tensor("fpool-%s" % (case,), "x", (n, c, h, w), -128, 127)
+    ref = oracle.max_pool2d(x, (k, k), (st, st), (pd, pd), ceil)
+    oh, ow = ref.shape[2:]
+    out = hipops.max_pool2d_i8(hipops.pack_nhwc_i8(T(x, dev)), c, h, w, (k, k), (st, st), (pd, pd), oh, ow)
+    eq(nhwc_to_nchw(out, c, oh, ow), ref, "max_pool int8")
+
+
+@pytest.mark.parametrize("c", [10, 64, 2048])
+def test_sum_hw_i8(c, dev):
+    x = synth.tensor("fsum-%d" % c, "x", (3, c, 7, 7), -127, 127)
+    ref = oracle.reduce("sum", x, (2, 3), False, False)
+    xp = hipops.pack_nhwc_i8(T(x, dev))
+    out = hipops.sum_hw_i8(xp, c, 49, None, False)
+    torch.cuda.synchronize()
+    eq(out.cpu().numpy(), ref, "sum int32")
+    stages = [("cvm_right_shift", 8, 6)]
+    out8 = hipops.sum_hw_i8(xp, c, 49, hipops.chain(*stages), True)
+    eq(nhwc_to_nchw(out8, c, 1, 1)[:, :, 0, 0], run_chain(ref, stages), "sum int8")
+
+
+def test_bad_arguments_are_refused(dev):
+    x = hipops.pack_nhwc_i8(T(np.zeros((1, 16, 4, 4), np.int32), dev))
+    w = hipops.pack_weights(T(np.zeros((16, 16, 3, 3), np.int32), dev))
+    from cvm_runtime_amd import CvmHipError
+    with pytest.raises(CvmHipError):
+        hipops.conv2d_i8(x, 16, 4, 4, w, 16, 3, 3, dilation=(2, 2))      # dilated 3x3 window exceeds the 4x4 input
+    bad = hipops.Chain()
+    bad.count = 5
+    with pytest.raises(CvmHipError):
+        hipops.conv2d_i8(x, 16, 4, 4, w, 16, 3, 3, chain1=bad, padding=(1, 1))
+
+
+@pytest.mark.parametrize("name", ["resnet20", "resnet50", "vgg16", "ssd"])
+def test_fused_executor_equals_node_by_node(name, dev):
+    """The load-time planner must not change a single output value: run the same
+    model with the planner on and off (CVM_HIP_FUSE=0) and compare with the oracle."""
+    if name == "resnet20":
+        g, heads = graphgen.resnet20_cifar(2)
+    elif name == "resnet50":
+        g, heads = graphgen.resnet50(2, width=16, size=64, classes=50, config_id="fuse-eq-r50")
+    elif name == "vgg16":
+        g, heads = graphgen.vgg16(1, size=32, width=8, fc=64, classes=20, config_id="fuse-eq-vgg")
+    else:
+        g, heads = graphgen.ssd_mobilenet(size=128, alpha=0.25, config_id="fuse-eq-ssd", neg_ids=True)
+    js, pb = g.build(heads)
+    x = synth.tensor("fuse-eq-" + name, "data", g.shape((0, 0)), -127, 127)
+    outs = {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_FUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(x.astype(np.int8).tobytes())
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FUSE", None)
+    assert outs["1"] == outs["0"]
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
