@@ -68,7 +68,14 @@ __device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const C
   }
 }
 
-template <int WM, int WN, int G, int KS>
+// clamp(v, lo, hi) for lo <= hi in one instruction
+__device__ __forceinline__ int32_t clamp3(int32_t v, int32_t lo, int32_t hi) {
+  int32_t r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+  return r;
+}
+
+template <int WM, int WN, int G, int KS, int OUT>
 __global__ void __launch_bounds__(256)
 k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void* __restrict__ out,
              const ConvGeom g, const Epilogue ep) {
@@ -124,13 +131,34 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   int r = tap / g.KW, s = tap - r * g.KW;
   int kbyte = 0;
 
+  // Accumulator element e of lane l in a 32x32 tile is row (e/4)*8 + (l/32)*4 + e%4
+  // (output channel), column l%32 (pixel).  Accumulators start at the bias of
+  // their channel, so the epilogue has no bias pass.
+  const int lrow = lane & 31;
+  const int lgrp = lane >> 5;
   v16i acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
+  for (int i = 0; i < WM; ++i) {
+    v16i b;
 #pragma unroll
-    for (int j = 0; j < WN; ++j)
+    for (int q = 0; q < 4; ++q) {
+      const int oc = oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4;
+      int4 bv = zero4();
+      if (ep.bias) {
+        if (ep.bias_vec && oc + 3 < g.OC) {
+          bv = *reinterpret_cast<const int4*>(ep.bias + oc);
+        } else {
+          if (oc < g.OC) bv.x = ep.bias[oc];
+          if (oc + 1 < g.OC) bv.y = ep.bias[oc + 1];
+          if (oc + 2 < g.OC) bv.z = ep.bias[oc + 2];
+          if (oc + 3 < g.OC) bv.w = ep.bias[oc + 3];
+        }
+      }
+      b[q * 4] = bv.x; b[q * 4 + 1] = bv.y; b[q * 4 + 2] = bv.z; b[q * 4 + 3] = bv.w;
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    for (int j = 0; j < WN; ++j) acc[i][j] = b;
+  }
 
   // One K step of operands held in registers as a single SSA vector value
   // (chunks 0..NA-1 filter, NA..NA+NB-1 activations); two of them are in flight.
@@ -176,8 +204,6 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
       *reinterpret_cast<int4*>(&sB[(buf * BN + frow + RPP * i) * LDK + kc * 16]) =
           make_int4(R[4 * (NA + i)], R[4 * (NA + i) + 1], R[4 * (NA + i) + 2], R[4 * (NA + i) + 3]);
   };
-  const int lrow = lane & 31;
-  const int lgrp = lane >> 5;
   auto mma = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < KS / 32; ++ks) {
@@ -218,55 +244,101 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     __syncthreads();
   }
 
-  // ---- epilogue.  Accumulator element e of lane l in a 32x32 tile is
-  // row (e/4)*8 + (l/32)*4 + e%4 (output channel), column l%32 (pixel).
-  const bool to_i8 = ep.out_mode == OUT_I8_NHWC;
+  // ---- epilogue: v = chain(acc); if (residual) v = chain2(v + residual).
+  // A chain runs stage by stage over all accumulators of the thread: the stage
+  // parameters are wave-uniform, so each stage costs four vector instructions
+  // per value (one for a pure clamp).
+  auto run_chain = [&](const DevChain& c) __attribute__((always_inline)) {
+    // the stages are copied to scalar registers first: indexing the kernel
+    // argument with the loop counter would move it to private memory
+    const DevStage q0 = c.st[0], q1 = c.st[1], q2 = c.st[2], q3 = c.st[3];
+#pragma unroll 1
+    for (int t = 0; t < c.count; ++t) {
+      DevStage st;
+      st.lo = t == 0 ? q0.lo : t == 1 ? q1.lo : t == 2 ? q2.lo : q3.lo;
+      st.hi = t == 0 ? q0.hi : t == 1 ? q1.hi : t == 2 ? q2.hi : q3.hi;
+      st.s1 = t == 0 ? q0.s1 : t == 1 ? q1.s1 : t == 2 ? q2.s1 : q3.s1;
+      st.add = t == 0 ? q0.add : t == 1 ? q1.add : t == 2 ? q2.add : q3.add;
+      st.s2 = t == 0 ? q0.s2 : t == 1 ? q1.s2 : t == 2 ? q2.s2 : q3.s2;
+      if ((st.s1 | st.add | st.s2) == 0) {
 #pragma unroll
-  for (int j = 0; j < WN; ++j) {
-    const int pl = (wn * WN + j) * 32 + lrow;  // pixel inside the tile
-    const int64_t p = px0 + pl;
-    const bool p_ok = p < g.P;
-    const int pp = p_ok ? (int)p : 0;
-    const int n = pp / OHW;
-    const int rem = pp - n * OHW;
-    const int8_t* res = ep.residual ? ep.residual + (int64_t)pp * ep.out_cp : nullptr;
-    int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
+        for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int i = 0; i < WM; ++i) {
+          for (int j = 0; j < WN; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {  // 4 consecutive channels: one residual dword, one packed int8 dword
-        const int ol = (wm * WM + i) * 32 + lgrp * 4 + q * 8;  // channel inside the tile
-        const int oc = oc0 + ol;
-        int4 bv = zero4();
-        if (ep.bias) {
-          if (ep.bias_vec && oc + 3 < g.OC) {
-            bv = *reinterpret_cast<const int4*>(ep.bias + oc);
-          } else {
-            if (oc < g.OC) bv.x = ep.bias[oc];
-            if (oc + 1 < g.OC) bv.y = ep.bias[oc + 1];
-            if (oc + 2 < g.OC) bv.z = ep.bias[oc + 2];
-            if (oc + 3 < g.OC) bv.w = ep.bias[oc + 3];
-          }
-        }
-        uint32_t rpack = 0;
-        if (res && p_ok && oc < ep.out_cp) rpack = *reinterpret_cast<const uint32_t*>(res + oc);
-        const int32_t b4[4] = {bv.x, bv.y, bv.z, bv.w};
-        uint32_t pack = 0;
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = clamp3(acc[i][j][e], st.lo, st.hi);
+      } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          int32_t v = apply_chain(ep.chain, wadd(acc[i][j][q * 4 + e], b4[e]));
-          if (res) v = apply_chain(ep.chain2, wadd(v, (int32_t)(int8_t)(rpack >> (8 * e))));
-          if (oc + e >= g.OC) v = 0;
-          if (!to_i8 && p_ok && oc + e < g.OC) y32[(int64_t)(oc + e) * OHW] = v;
-          pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * e);
-        }
-        if (to_i8) *reinterpret_cast<uint32_t*>(&sA[pl * OPITCH + ol]) = pack;
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              acc[i][j][e] = wadd(clamp3(acc[i][j][e], st.lo, st.hi) >> st.s1, st.add) >> st.s2;
       }
     }
+  };
+  if (ep.residual) {
+    // one dword = the residual of 4 consecutive channels; loads are issued before the first chain runs
+    uint32_t rp[WM][WN][4];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
+      const int8_t* res = ep.residual + (p < g.P ? p : 0) * ep.out_cp;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int oc = oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4;
+          rp[i][j][q] = *reinterpret_cast<const uint32_t*>(res + (oc < ep.out_cp ? oc : 0));
+        }
+    }
+    run_chain(ep.chain);
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          acc[i][j][e] = wadd(acc[i][j][e], (int32_t)(int8_t)(rp[i][j][e >> 2] >> (8 * (e & 3))));
+    run_chain(ep.chain2);
+  } else {
+    run_chain(ep.chain);
   }
-  if (to_i8) {
+
+  if (OUT == OUT_I32_NCHW) {
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
+      if (p >= g.P) continue;
+      const int n = (int)p / OHW;
+      const int rem = (int)p - n * OHW;
+      int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int oc = oc0 + (wm * WM + i) * 32 + (e >> 2) * 8 + lgrp * 4 + (e & 3);
+          if (oc < g.OC) y32[(int64_t)oc * OHW] = acc[i][j][e];
+        }
+    }
+  } else {
+    // int8 NHWC: transpose the tile through LDS (the filter staging area is free
+    // after the last barrier of the K loop) so that global stores are 16 contiguous bytes per thread
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int pl = (wn * WN + j) * 32 + lrow;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ol = (wm * WM + i) * 32 + q * 8 + lgrp * 4;
+          const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)acc[i][j][q * 4 + 1], (uint32_t)acc[i][j][q * 4], 0x0c0c0400u);
+          const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)acc[i][j][q * 4 + 3], (uint32_t)acc[i][j][q * 4 + 2], 0x0c0c0400u);
+          *reinterpret_cast<uint32_t*>(&sA[pl * OPITCH + ol]) = __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
+        }
+    }
     __syncthreads();
-    // each thread moves 16 contiguous output bytes of one pixel
     constexpr int CH = BM / 16;
     int8_t* y8 = reinterpret_cast<int8_t*>(out);
 #pragma unroll
@@ -276,13 +348,22 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
       const int oc = oc0 + c16 * 16;
       if (p >= g.P || oc >= ep.out_cp) continue;
       const uint32_t* src = reinterpret_cast<const uint32_t*>(&sA[pl * OPITCH + c16 * 16]);
+      uint32_t d[4] = {src[0], src[1], src[2], src[3]};
+      if (oc + 16 > g.OC) {
+        // padding channels of the NHWC tensor stay zero whatever the chain maps 0 to
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int keep = g.OC - (oc + 4 * k);
+          d[k] = keep >= 4 ? d[k] : (keep <= 0 ? 0u : d[k] & ((1u << (8 * keep)) - 1u));
+        }
+      }
       int8_t* dst = y8 + p * ep.out_cp + oc;
       if (oc + 16 <= ep.out_cp && (ep.out_cp & 15) == 0) {
-        *reinterpret_cast<int4*>(dst) = make_int4(src[0], src[1], src[2], src[3]);
+        *reinterpret_cast<int4*>(dst) = make_int4(d[0], d[1], d[2], d[3]);
       } else {
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
-          if (oc + d * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[d] = src[d];
+        for (int k = 0; k < 4; ++k)
+          if (oc + k * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[k] = d[k];
       }
     }
   }
@@ -444,23 +525,32 @@ int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, h
   return check_launch("pack_weights");
 }
 
-template <int WM, int WN>
+template <int WM, int WN, int OUT>
 static void launch_tile(int gran, bool wide, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                         const ConvGeom& g, const Epilogue& ep) {
   if (gran == 16) {
     // 128-byte K steps halve the number of barriers; the 128x128 tile keeps 64 (LDS budget)
     if constexpr (WM + WN < 4) {
       if (wide) {
-        k_conv_igemm<WM, WN, 16, 128><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+        k_conv_igemm<WM, WN, 16, 128, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
         return;
       }
     }
-    k_conv_igemm<WM, WN, 16, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+    k_conv_igemm<WM, WN, 16, 64, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
   } else if (gran == 8) {
-    k_conv_igemm<WM, WN, 8, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+    k_conv_igemm<WM, WN, 8, 64, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
   } else {
-    k_conv_igemm<WM, WN, 4, 64><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+    k_conv_igemm<WM, WN, 4, 64, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
   }
+}
+
+template <int OUT>
+static void launch_out(int wm, int wn, int gran, bool wide, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp,
+                       void* out, const ConvGeom& g, const Epilogue& ep) {
+  if (wm == 2 && wn == 2) launch_tile<2, 2, OUT>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else if (wm == 1 && wn == 2) launch_tile<1, 2, OUT>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else if (wm == 2 && wn == 1) launch_tile<2, 1, OUT>(gran, wide, grid, s, xp, wp, out, g, ep);
+  else launch_tile<1, 1, OUT>(gran, wide, grid, s, xp, wp, out, g, ep);
 }
 
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
@@ -505,10 +595,8 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   g.adv_tap = ks / g.Cp;
   g.adv_r = g.adv_tap / g.KW;
   g.adv_s = g.adv_tap % g.KW;
-  if (wm == 2 && wn == 2) launch_tile<2, 2>(gran, wide, grid, s, xp, wp, out, g, ep);
-  else if (wm == 1 && wn == 2) launch_tile<1, 2>(gran, wide, grid, s, xp, wp, out, g, ep);
-  else if (wm == 2 && wn == 1) launch_tile<2, 1>(gran, wide, grid, s, xp, wp, out, g, ep);
-  else launch_tile<1, 1>(gran, wide, grid, s, xp, wp, out, g, ep);
+  if (ep.out_mode == OUT_I8_NHWC) launch_out<OUT_I8_NHWC>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
+  else launch_out<OUT_I32_NCHW>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
   return check_launch("conv_igemm");
 }
 
