@@ -7,10 +7,10 @@
 
 namespace cvmhip {
 
-enum { OUT_I32_NCHW = 0, OUT_I8_NHWC = 1 };
+enum { OUT_I32_NCHW = 0, OUT_I8_ACT = 1 };
 
 struct ConvGeom {
-  int N, H, W, Cp;         // input: int8 NHWC, channels padded to Cp
+  int N, H, W, Cp;         // input: int8 activations in the layout above, channels padded to Cp
   int C;                   // true channel count (0 = unknown, only used to count algorithmic work)
   int OC, OH, OW;          // output extent
   int KH, KW, SH, SW, PH, PW, DH, DW;
@@ -25,11 +25,43 @@ struct Epilogue {
   const int32_t* bias;     // device pointer or nullptr
   int bias_vec;            // set by conv_igemm: bias is 16-byte aligned
   DevChain chain;
-  const int8_t* residual;  // int8 NHWC with pitch out_cp, or nullptr
+  const int8_t* residual;  // int8 activations with out_cp channels, or nullptr
   DevChain chain2;
-  int out_mode;            // OUT_I32_NCHW or OUT_I8_NHWC
-  int out_cp;              // channel pitch of int8 NHWC output / residual (multiple of 4, >= OC)
+  int out_mode;            // OUT_I32_NCHW or OUT_I8_ACT
+  int out_cp;              // padded channel count of the int8 output / residual (>= OC)
 };
+
+// ---- int8 activation layout.  Channels are padded to Cp = 4, 8, 16 or a
+// multiple of 32.  Cp <= 16: plain NHWC.  Cp % 32 == 0: "pixel-blocked" -- the
+// tensor is cut into blocks of 32 consecutive pixels (linear index over n, h, w)
+// x 32 channels, and a block is stored as the 1 KiB a wavefront feeds to
+// v_mfma_i32_32x32x32_i8: lane l holds pixel (l & 31), channels (l >> 5)*16 .. +15.
+//   offset(p, c) = ((p/32)*(Cp/32) + c/32)*1024 + ((c/16)%2)*512 + (p%32)*16 + c%16
+// Any 16 channel-aligned bytes of one pixel are contiguous in both forms, and a
+// 1x1 convolution reads its operand as whole contiguous blocks.
+__host__ __device__ inline bool act_blocked(int cp) { return (cp & 31) == 0; }
+__host__ __device__ inline int64_t act_offset(int64_t p, int c, int cp) {
+  if (!act_blocked(cp)) return p * cp + c;
+  return ((p >> 5) * (cp >> 5) + (c >> 5)) * 1024 + ((c >> 4) & 1) * 512 + (p & 31) * 16 + (c & 15);
+}
+__host__ __device__ inline int64_t act_bytes(int64_t npix, int cp) {
+  return act_blocked(cp) ? ((npix + 31) & ~(int64_t)31) * cp : npix * cp;
+}
+// dword i of the buffer -> pixel and first of its 4 channels
+__host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c) {
+  if (!act_blocked(cp)) {
+    const int c4n = cp >> 2;
+    *p = i / c4n;
+    *c = (int)(i - *p * c4n) * 4;
+  } else {
+    const int ctiles = cp >> 5;
+    const int64_t blk = i >> 8;
+    const int w = (int)(i & 255);
+    const int64_t ptile = blk / ctiles;
+    *p = ptile * 32 + ((w >> 2) & 31);
+    *c = (int)(blk - ptile * ctiles) * 32 + (w >> 7) * 16 + (w & 3) * 4;
+  }
+}
 
 int pad_channels(int c);
 size_t packed_act_bytes(int64_t npix, int c);

@@ -1,22 +1,27 @@
 // conv2d / dense on gfx950 as an exact int8 x int8 -> int32 implicit GEMM.
 //
-//   D[oc][px] = sum_k Wp[oc][k] * Xcol[px][k],   k = (kh, kw, c),  px = (n, oh, ow)
+//   D[oc][px] = sum_k W[oc][k] * Xcol[px][k],   k = (kh, kw, c),  px = (n, oh, ow)
 //
-// Data layout
-//   Xp : int8 NHWC activations, channels padded to Cp (4, 8 or a multiple of 16)
-//   Wp : int8 [OCp][Kp] filter rows, k ordered (kh, kw, c) with c padded to Cp,
-//        Kp = K rounded up to 64, OCp = OC rounded up to 128; padding is zero
-//   D  : int32 NCHW (the operator contract) or int8 NHWC (fused requantised output)
+// Data layout: everything that feeds v_mfma_i32_32x32x32_i8 lives in memory in
+// the order the instruction wants it ("fragment order": a block of 32 rows x 32
+// bytes of K is the 1 KiB where lane l holds row l & 31, bytes (l >> 5)*16..+15).
+//   X : int8 activations, pixel-blocked when Cp % 32 == 0, NHWC for Cp = 4, 8, 16
+//       (conv_mfma.h: act_offset)
+//   W : int8 filter in fragment order, k ordered (kh, kw, c) with c padded to Cp,
+//       K padded to 64, OC to 128 (k_pack_weights)
+//   D : int32 NCHW (the operator contract) or int8 activations in the layout above
+//       (fused requantised output)
 //
-// One workgroup = 4 wavefronts (2 x 2) and computes a (64*WM) x (64*WN) tile of
-// D with v_mfma_i32_32x32x32_i8.  Each K step stages a KS-byte slab (64 or 128)
-// of both operands in LDS (row pitch KS+16 bytes, so the 16-byte MFMA operand
-// reads of 8 consecutive lanes hit disjoint banks); the im2col addressing
-// happens while the slab is fetched, so no column buffer ever exists in HBM.
-// Global fetches run two K steps ahead of the MFMAs (registers hold step t+1
-// and t+2 while LDS holds t and t+1), with one barrier per step.  The int8
-// epilogue transposes the tile through LDS so that every lane writes 16
-// contiguous output bytes.
+// Two kernels, same arithmetic (integer sums commute, so they agree bit for bit):
+//   k_conv_igemm  workgroup tile (64*WM) x (64*WN), operands staged in LDS in
+//                 fragment order (global -> LDS -> MFMA registers are straight
+//                 1 KiB block copies for the filter and, for 1x1 convolutions, the
+//                 activations), registers prefetch two K steps ahead, one barrier
+//                 per step.  Serves every layout and the large layers.
+//   k_conv_wave   no LDS and no barrier in the K loop: each wavefront streams its
+//                 own fragments from memory, the wavefronts of a workgroup split
+//                 K and meet in LDS once.  Serves layers whose grid is too small
+//                 to hide the per-step latency of the tiled kernel.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -31,21 +36,117 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ int4 zero4() { return make_int4(0, 0, 0, 0); }
 
 // Source of every out-of-image (padding) granule: loads stay unconditional and
-// the data needs no fix-up before it goes to LDS, so nothing but the loads
-// themselves sits between a fetch and the matrix instructions of that K step.
+// the data needs no fix-up afterwards.
 __device__ __attribute__((aligned(16))) int g_zero_granule[4] = {0, 0, 0, 0};  // never written
+
+// clamp(v, lo, hi) for lo <= hi in one instruction
+__device__ __forceinline__ int32_t clamp3(int32_t v, int32_t lo, int32_t hi) {
+  int32_t r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+  return r;
+}
+
+// A requantisation chain over N values held in registers, stage by stage: the
+// stage parameters are wave-uniform, so a stage costs four vector instructions
+// per value.  The stages are copied to scalar registers first; indexing the
+// kernel argument with the loop counter would move it to private memory.
+template <int N>
+__device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
+  const DevStage q0 = c.st[0], q1 = c.st[1], q2 = c.st[2], q3 = c.st[3];
+#pragma unroll 1
+  for (int t = 0; t < c.count; ++t) {
+    const int32_t lo = t == 0 ? q0.lo : t == 1 ? q1.lo : t == 2 ? q2.lo : q3.lo;
+    const int32_t hi = t == 0 ? q0.hi : t == 1 ? q1.hi : t == 2 ? q2.hi : q3.hi;
+    const int32_t s1 = t == 0 ? q0.s1 : t == 1 ? q1.s1 : t == 2 ? q2.s1 : q3.s1;
+    const int32_t ad = t == 0 ? q0.add : t == 1 ? q1.add : t == 2 ? q2.add : q3.add;
+    const int32_t s2 = t == 0 ? q0.s2 : t == 1 ? q1.s2 : t == 2 ? q2.s2 : q3.s2;
+    if ((s1 | ad | s2) == 0) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], lo, hi);
+    } else {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = wadd(clamp3(v[e], lo, hi) >> s1, ad) >> s2;
+    }
+  }
+}
+
+// bias of 4 consecutive output channels starting at oc (zero past OC or without bias)
+__device__ __forceinline__ int4 bias4(const Epilogue& ep, int OC, int oc) {
+  int4 bv = zero4();
+  if (ep.bias) {
+    if (ep.bias_vec && oc + 3 < OC) {
+      bv = *reinterpret_cast<const int4*>(ep.bias + oc);
+    } else {
+      if (oc < OC) bv.x = ep.bias[oc];
+      if (oc + 1 < OC) bv.y = ep.bias[oc + 1];
+      if (oc + 2 < OC) bv.z = ep.bias[oc + 2];
+      if (oc + 3 < OC) bv.w = ep.bias[oc + 3];
+    }
+  }
+  return bv;
+}
+
+// low bytes of four values -> one dword
+__device__ __forceinline__ uint32_t pack_bytes(int32_t a, int32_t b, int32_t c, int32_t d) {
+  const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+  const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
+}
+
+// residual of 4 consecutive channels of pixel p (clamped to valid memory)
+__device__ __forceinline__ uint32_t residual4(const Epilogue& ep, int64_t P, int64_t p, int oc) {
+  return *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ep.out_cp ? oc : 0, ep.out_cp));
+}
+
+// The int8 output tile sits in LDS as sOut[pixel][OPITCH] (channels contiguous);
+// NT threads move it to the output tensor in 16-byte granules, 32 consecutive
+// pixels per half wavefront (512 contiguous bytes of a pixel-blocked tensor).
+template <int BM, int BN, int NT>
+__device__ __forceinline__ void store_tile_i8(const int8_t* sOut, int opitch, void* out, const ConvGeom& g, const Epilogue& ep,
+                                              int oc0, int64_t px0, int tid) {
+  constexpr int CH = BM / 16;
+  int8_t* y8 = reinterpret_cast<int8_t*>(out);
+#pragma unroll
+  for (int id = tid; id < BN * CH; id += NT) {
+    const int rr = id & 31;
+    const int c16 = (id >> 5) % CH;
+    const int pl = ((id >> 5) / CH) * 32 + rr;
+    const int64_t p = px0 + pl;
+    const int oc = oc0 + c16 * 16;
+    if (p >= g.P || oc >= ep.out_cp) continue;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(sOut + pl * opitch + c16 * 16);
+    uint32_t d[4] = {src[0], src[1], src[2], src[3]};
+    if (oc + 16 > g.OC) {
+      // padding channels of the tensor stay zero whatever the chain maps 0 to
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int keep = g.OC - (oc + 4 * k);
+        d[k] = keep >= 4 ? d[k] : (keep <= 0 ? 0u : d[k] & ((1u << (8 * keep)) - 1u));
+      }
+    }
+    int8_t* dst = y8 + act_offset(p, oc, ep.out_cp);
+    if (ep.out_cp >= 16) {
+      *reinterpret_cast<int4*>(dst) = make_int4(d[0], d[1], d[2], d[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (oc + k * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[k] = d[k];
+    }
+  }
+}
 
 // Fetch the 16 consecutive k-bytes of one im2col row that start at filter tap
 // (r, s), channel c0.  G = bytes that are contiguous in memory for one filter
-// tap: 16 when Cp % 16 == 0, else Cp itself (4 or 8) and the chunk spans 16/G taps.
+// tap: 16 when Cp % 16 == 0, else Cp itself (4 or 8) and the granule spans 16/G taps.
+// img_pix = linear pixel index of the image's first pixel.
 template <int G>
-__device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const ConvGeom& g, bool row_ok, int img_off,
+__device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const ConvGeom& g, bool row_ok, int img_pix,
                                           int ih0, int iw0, int tap, int r, int s, int c0) {
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   if (G == 16) {
     const int ih = ih0 + r * g.DH, iw = iw0 + s * g.DW;
     const bool ok = row_ok && tap < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-    const int8_t* src = ok ? xp + (img_off + (ih * g.W + iw) * g.Cp + c0) : zero;
+    const int8_t* src = ok ? xp + act_offset(img_pix + ih * g.W + iw, c0, g.Cp) : zero;
     return *reinterpret_cast<const int4*>(src);
   } else {
     int v[4] = {0, 0, 0, 0};
@@ -55,7 +156,7 @@ __device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const C
       const int rr = t / g.KW, ss = t - rr * g.KW;
       const int ih = ih0 + rr * g.DH, iw = iw0 + ss * g.DW;
       const bool ok = row_ok && t < g.taps && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-      const int8_t* src = ok ? xp + (img_off + (ih * g.W + iw) * g.Cp) : zero;
+      const int8_t* src = ok ? xp + (int64_t)(img_pix + ih * g.W + iw) * g.Cp : zero;
       if (G == 4) {
         v[j] = *reinterpret_cast<const int*>(src);
       } else {
@@ -68,33 +169,28 @@ __device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const C
   }
 }
 
-// clamp(v, lo, hi) for lo <= hi in one instruction
-__device__ __forceinline__ int32_t clamp3(int32_t v, int32_t lo, int32_t hi) {
-  int32_t r;
-  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
-  return r;
-}
-
 template <int WM, int WN, int G, int KS, int OUT>
 __global__ void __launch_bounds__(256)
 k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void* __restrict__ out,
              const ConvGeom g, const Epilogue ep) {
   constexpr int BM = 64 * WM;        // output channels per workgroup
   constexpr int BN = 64 * WN;        // output pixels per workgroup
-  constexpr int LDK = KS + 16;       // LDS row pitch in bytes
-  constexpr int CPR = KS / 16;       // 16-byte chunks per row and K step
-  constexpr int RPP = 256 / CPR;     // rows one pass of the workgroup covers
-  constexpr int NA = BM / RPP;       // filter chunks per thread and K step
-  constexpr int NB = BN / RPP;       // activation chunks per thread and K step
-  constexpr int OPITCH = BM + 4;     // pitch of the transposed int8 output tile (odd number of dwords)
-  static_assert(BN * OPITCH <= 2 * BM * LDK, "output tile must fit the filter staging area");
-  __shared__ __attribute__((aligned(16))) int8_t sA[2 * BM * LDK];
-  __shared__ __attribute__((aligned(16))) int8_t sB[2 * BN * LDK];
+  constexpr int CH32 = KS / 32;      // 32-byte chunks of K per step
+  constexpr int NA = BM * KS / 4096; // 16-byte granules per thread and K step, filter
+  constexpr int NB = BN * KS / 4096; //   ... activations
+  constexpr int OPITCH = BM + 4;     // pitch of the int8 output tile (odd number of dwords)
+  static_assert(BN * OPITCH <= 2 * (BM + BN) * KS, "output tile must fit the staging area");
+  // two buffers of each operand in fragment order: granule index = ((tile32*CH32 + chunk)*64 + lane)
+  __shared__ __attribute__((aligned(16))) int8_t smem[2 * (BM + BN) * KS];
+  int8_t* sA = smem;
+  int8_t* sB = smem + 2 * BM * KS;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane & 31;
+  const int lgrp = lane >> 5;
 
   // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so
   // give each XCD a contiguous run of tiles (neighbouring tiles share the
@@ -106,27 +202,32 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   const int oc0 = (pid % oc_tiles) * BM;
   const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
 
-  // ---- per-thread fetch assignment: chunk column kc, rows frow + RPP*i
-  const int kc = tid % CPR;
-  const int frow = tid / CPR;
+  // ---- per-thread fetch assignment.  Granule tid + 256*i of an operand: lane
+  // part (tid & 63) = row (tid & 31) and 16-byte half (tid >> 5) & 1; wave + 4*i
+  // enumerates (32-row tile, chunk).  The 16-byte K column of a thread is fixed.
+  const int chunk = wave % CH32;
+  const int kc = chunk * 2 + lgrp;
   const int OHW = g.OH * g.OW;
   bool row_ok[NB];
-  int img_off[NB], ih0[NB], iw0[NB];
+  int img_pix[NB], ih0[NB], iw0[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const int64_t p = px0 + frow + RPP * i;
+    const int64_t p = px0 + ((wave + 4 * i) / CH32) * 32 + lrow;
     row_ok[i] = p < g.P;
     const int pp = row_ok[i] ? (int)p : 0;
     const int n = pp / OHW;
     const int rem = pp - n * OHW;
     const int oh = rem / g.OW, ow = rem - oh * g.OW;
-    img_off[i] = n * g.H * g.W * g.Cp;
+    img_pix[i] = n * g.H * g.W;
     ih0[i] = oh * g.SH - g.PH;
     iw0[i] = ow * g.SW - g.PW;
   }
-  const int8_t* wbase = wp + (int64_t)(oc0 + frow) * g.Kp + kc * 16;
+  const int nch1 = g.Kp / 32 + 1;
+  int wrow[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) wrow[i] = ((oc0 / 32 + (wave + 4 * i) / CH32) * nch1 + chunk) * 1024 + lane * 16;
 
-  // position of this thread's chunk inside the (tap, channel) space
+  // position of this thread's granule inside the (tap, channel) space
   int tap = (kc * 16) / g.Cp, c0 = kc * 16 - tap * g.Cp;
   int r = tap / g.KW, s = tap - r * g.KW;
   int kbyte = 0;
@@ -134,26 +235,13 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   // Accumulator element e of lane l in a 32x32 tile is row (e/4)*8 + (l/32)*4 + e%4
   // (output channel), column l%32 (pixel).  Accumulators start at the bias of
   // their channel, so the epilogue has no bias pass.
-  const int lrow = lane & 31;
-  const int lgrp = lane >> 5;
   v16i acc[WM][WN];
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     v16i b;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int oc = oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4;
-      int4 bv = zero4();
-      if (ep.bias) {
-        if (ep.bias_vec && oc + 3 < g.OC) {
-          bv = *reinterpret_cast<const int4*>(ep.bias + oc);
-        } else {
-          if (oc < g.OC) bv.x = ep.bias[oc];
-          if (oc + 1 < g.OC) bv.y = ep.bias[oc + 1];
-          if (oc + 2 < g.OC) bv.z = ep.bias[oc + 2];
-          if (oc + 3 < g.OC) bv.w = ep.bias[oc + 3];
-        }
-      }
+      const int4 bv = bias4(ep, g.OC, oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4);
       b[q * 4] = bv.x; b[q * 4 + 1] = bv.y; b[q * 4 + 2] = bv.z; b[q * 4 + 3] = bv.w;
     }
 #pragma unroll
@@ -161,7 +249,7 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   }
 
   // One K step of operands held in registers as a single SSA vector value
-  // (chunks 0..NA-1 filter, NA..NA+NB-1 activations); two of them are in flight.
+  // (granules 0..NA-1 filter, NA..NA+NB-1 activations); two of them are in flight.
   typedef int regs_t __attribute__((ext_vector_type(4 * (NA + NB))));
   const int nk = g.Kp / KS;
 
@@ -170,17 +258,17 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     regs_t R;
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const int4 v = *reinterpret_cast<const int4*>(wbase + (int64_t)(RPP * i) * g.Kp + kbyte);
+      const int4 v = *reinterpret_cast<const int4*>(wp + wrow[i] + kbyte);
       R[4 * i] = v.x; R[4 * i + 1] = v.y; R[4 * i + 2] = v.z; R[4 * i + 3] = v.w;
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int4 v = fetch_act<G>(xp, g, row_ok[i], img_off[i], ih0[i], iw0[i], tap, r, s, c0);
+      const int4 v = fetch_act<G>(xp, g, row_ok[i], img_pix[i], ih0[i], iw0[i], tap, r, s, c0);
       R[4 * (NA + i)] = v.x; R[4 * (NA + i) + 1] = v.y; R[4 * (NA + i) + 2] = v.z; R[4 * (NA + i) + 3] = v.w;
     }
-    kbyte += KS;
+    kbyte += CH32 * 1024;
     if (G == 16) {
-      // advance the cursor by KS bytes without a loop (lanes sit at different chunks)
+      // advance the cursor by KS bytes without a loop (lanes sit at different granules)
       c0 += g.adv_c;
       const int carry = c0 >= g.Cp ? 1 : 0;
       c0 -= carry ? g.Cp : 0;
@@ -197,23 +285,23 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   auto stage = [&](const regs_t R, int buf) {
 #pragma unroll
     for (int i = 0; i < NA; ++i)
-      *reinterpret_cast<int4*>(&sA[(buf * BM + frow + RPP * i) * LDK + kc * 16]) =
+      *reinterpret_cast<int4*>(&sA[buf * BM * KS + (tid + 256 * i) * 16]) =
           make_int4(R[4 * i], R[4 * i + 1], R[4 * i + 2], R[4 * i + 3]);
 #pragma unroll
     for (int i = 0; i < NB; ++i)
-      *reinterpret_cast<int4*>(&sB[(buf * BN + frow + RPP * i) * LDK + kc * 16]) =
+      *reinterpret_cast<int4*>(&sB[buf * BN * KS + (tid + 256 * i) * 16]) =
           make_int4(R[4 * (NA + i)], R[4 * (NA + i) + 1], R[4 * (NA + i) + 2], R[4 * (NA + i) + 3]);
   };
   auto mma = [&](int buf) {
 #pragma unroll
-    for (int ks = 0; ks < KS / 32; ++ks) {
+    for (int ks = 0; ks < CH32; ++ks) {
       v4i a[WM], b[WN];
 #pragma unroll
       for (int i = 0; i < WM; ++i)
-        a[i] = *reinterpret_cast<const v4i*>(&sA[(buf * BM + (wm * WM + i) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+        a[i] = *reinterpret_cast<const v4i*>(&sA[buf * BM * KS + (((wm * WM + i) * CH32 + ks) * 64 + lane) * 16]);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
-        b[j] = *reinterpret_cast<const v4i*>(&sB[(buf * BN + (wn * WN + j) * 32 + lrow) * LDK + ks * 32 + lgrp * 16]);
+        b[j] = *reinterpret_cast<const v4i*>(&sB[buf * BN * KS + (((wn * WN + j) * CH32 + ks) * 64 + lane) * 16]);
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -225,9 +313,9 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   // K step kt: the register set of that parity receives step kt+2, LDS buffer
   // kt&1 is consumed, the other register set (step kt+1, fetched one step
   // earlier) moves to the other LDS buffer.  Fetches are unconditional -- a step
-  // past the end reads valid memory (filter rows have slack behind them, taps
-  // past the filter read the zero granule) and is never consumed -- because a conditional
-  // fetch makes the compiler wait for all outstanding loads at the join.
+  // past the end reads valid memory (the filter has slack behind it, taps past
+  // the filter read the zero granule) and is never consumed -- because a
+  // conditional fetch makes the compiler wait for all outstanding loads at the join.
   regs_t R0 = fetch();
   regs_t R1 = fetch();
   stage(R0, 0);
@@ -244,66 +332,30 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     __syncthreads();
   }
 
-  // ---- epilogue: v = chain(acc); if (residual) v = chain2(v + residual).
-  // A chain runs stage by stage over all accumulators of the thread: the stage
-  // parameters are wave-uniform, so each stage costs four vector instructions
-  // per value (one for a pure clamp).
-  auto run_chain = [&](const DevChain& c) __attribute__((always_inline)) {
-    // the stages are copied to scalar registers first: indexing the kernel
-    // argument with the loop counter would move it to private memory
-    const DevStage q0 = c.st[0], q1 = c.st[1], q2 = c.st[2], q3 = c.st[3];
-#pragma unroll 1
-    for (int t = 0; t < c.count; ++t) {
-      DevStage st;
-      st.lo = t == 0 ? q0.lo : t == 1 ? q1.lo : t == 2 ? q2.lo : q3.lo;
-      st.hi = t == 0 ? q0.hi : t == 1 ? q1.hi : t == 2 ? q2.hi : q3.hi;
-      st.s1 = t == 0 ? q0.s1 : t == 1 ? q1.s1 : t == 2 ? q2.s1 : q3.s1;
-      st.add = t == 0 ? q0.add : t == 1 ? q1.add : t == 2 ? q2.add : q3.add;
-      st.s2 = t == 0 ? q0.s2 : t == 1 ? q1.s2 : t == 2 ? q2.s2 : q3.s2;
-      if ((st.s1 | st.add | st.s2) == 0) {
+  // ---- epilogue: v = chain(acc); if (residual) v = chain2(v + residual)
+  int32_t val[WM * WN * 16];
 #pragma unroll
-        for (int i = 0; i < WM; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-          for (int j = 0; j < WN; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = clamp3(acc[i][j][e], st.lo, st.hi);
-      } else {
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-#pragma unroll
-          for (int j = 0; j < WN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-              acc[i][j][e] = wadd(clamp3(acc[i][j][e], st.lo, st.hi) >> st.s1, st.add) >> st.s2;
-      }
-    }
-  };
+      for (int e = 0; e < 16; ++e) val[(i * WN + j) * 16 + e] = acc[i][j][e];
   if (ep.residual) {
     // one dword = the residual of 4 consecutive channels; loads are issued before the first chain runs
-    uint32_t rp[WM][WN][4];
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
-      const int8_t* res = ep.residual + (p < g.P ? p : 0) * ep.out_cp;
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int oc = oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4;
-          rp[i][j][q] = *reinterpret_cast<const uint32_t*>(res + (oc < ep.out_cp ? oc : 0));
-        }
-    }
-    run_chain(ep.chain);
+    uint32_t rp[WM * WN * 4];
 #pragma unroll
     for (int i = 0; i < WM; ++i)
 #pragma unroll
       for (int j = 0; j < WN; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          acc[i][j][e] = wadd(acc[i][j][e], (int32_t)(int8_t)(rp[i][j][e >> 2] >> (8 * (e & 3))));
-    run_chain(ep.chain2);
+        for (int q = 0; q < 4; ++q)
+          rp[(i * WN + j) * 4 + q] = residual4(ep, g.P, px0 + (wn * WN + j) * 32 + lrow, oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4);
+    run_chain(ep.chain, val);
+#pragma unroll
+    for (int e = 0; e < WM * WN * 16; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
+    run_chain(ep.chain2, val);
   } else {
-    run_chain(ep.chain);
+    run_chain(ep.chain, val);
   }
 
   if (OUT == OUT_I32_NCHW) {
@@ -319,12 +371,12 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int oc = oc0 + (wm * WM + i) * 32 + (e >> 2) * 8 + lgrp * 4 + (e & 3);
-          if (oc < g.OC) y32[(int64_t)oc * OHW] = acc[i][j][e];
+          if (oc < g.OC) y32[(int64_t)oc * OHW] = val[(i * WN + j) * 16 + e];
         }
     }
   } else {
-    // int8 NHWC: transpose the tile through LDS (the filter staging area is free
-    // after the last barrier of the K loop) so that global stores are 16 contiguous bytes per thread
+    // int8: the tile goes through LDS (the staging area is free after the last
+    // barrier of the K loop) so that global stores are 16 contiguous bytes per thread
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
       const int pl = (wn * WN + j) * 32 + lrow;
@@ -333,99 +385,328 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int ol = (wm * WM + i) * 32 + q * 8 + lgrp * 4;
-          const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)acc[i][j][q * 4 + 1], (uint32_t)acc[i][j][q * 4], 0x0c0c0400u);
-          const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)acc[i][j][q * 4 + 3], (uint32_t)acc[i][j][q * 4 + 2], 0x0c0c0400u);
-          *reinterpret_cast<uint32_t*>(&sA[pl * OPITCH + ol]) = __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
+          const int b = (i * WN + j) * 16 + q * 4;
+          *reinterpret_cast<uint32_t*>(&smem[pl * OPITCH + ol]) = pack_bytes(val[b], val[b + 1], val[b + 2], val[b + 3]);
         }
     }
     __syncthreads();
-    constexpr int CH = BM / 16;
-    int8_t* y8 = reinterpret_cast<int8_t*>(out);
-#pragma unroll
-    for (int id = tid; id < BN * CH; id += 256) {
-      const int pl = id / CH, c16 = id - pl * CH;
-      const int64_t p = px0 + pl;
-      const int oc = oc0 + c16 * 16;
-      if (p >= g.P || oc >= ep.out_cp) continue;
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(&sA[pl * OPITCH + c16 * 16]);
-      uint32_t d[4] = {src[0], src[1], src[2], src[3]};
-      if (oc + 16 > g.OC) {
-        // padding channels of the NHWC tensor stay zero whatever the chain maps 0 to
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int keep = g.OC - (oc + 4 * k);
-          d[k] = keep >= 4 ? d[k] : (keep <= 0 ? 0u : d[k] & ((1u << (8 * keep)) - 1u));
-        }
-      }
-      int8_t* dst = y8 + p * ep.out_cp + oc;
-      if (oc + 16 <= ep.out_cp && (ep.out_cp & 15) == 0) {
-        *reinterpret_cast<int4*>(dst) = make_int4(d[0], d[1], d[2], d[3]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (oc + k * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[k] = d[k];
-      }
-    }
+    store_tile_i8<BM, BN, 256>(smem, OPITCH, out, g, ep, oc0, px0, tid);
   }
 }
 
-constexpr int KSTEP = 64;  // granularity the packed filter rows are padded to
+// ---------------------------------------------------------------- wavefront-private kernel
+// Layers whose grid is small (few pixels, deep K) are bound by the latency of
+// the global -> LDS -> barrier chain of the tiled kernel above, not by MFMA
+// rate.  This kernel has no LDS and no barrier in its K loop: every wavefront
+// streams its own operands straight from memory into MFMA registers (filter and
+// pixel-blocked activations are both stored in fragment order, so a load is
+// 16 bytes per lane and, for a 1x1 convolution, 1 KiB contiguous per wavefront)
+// and keeps two batches of D chunks (32 bytes of K each) in flight.  The NW
+// wavefronts of a workgroup split the K range KSPLIT ways and the pixel axis
+// NW/KSPLIT ways; partial sums meet in LDS once, after the loop.
+// Requires Cp % 32 == 0 (pixel-blocked input; a chunk never straddles two filter
+// taps) and, when the convolution pads, at most 32 taps (per-lane validity mask).
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, bool NOPAD>
+__global__ void __launch_bounds__(NW * 64, MINW)
+k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
+            const ConvGeom g, const Epilogue ep) {
+  constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
+  constexpr int BM = 32 * TM;             // output channels per workgroup
+  constexpr int WPIX = 32 * TN;           // pixels per wavefront
+  constexpr int BN = WPIX * PS;           // pixels per workgroup
+  constexpr int U = TM * TN * 4;          // groups of 4 accumulator registers (4 consecutive channels) per wavefront
+  constexpr int NU = U / KSPLIT;          // groups one wavefront finalises
+  constexpr int OPITCH = BM + 4;
+  static_assert(NW % KSPLIT == 0 && U % KSPLIT == 0, "split must divide the work");
+  __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
+  __shared__ __attribute__((aligned(16))) int8_t sOut[OUT == OUT_I8_ACT ? BN * OPITCH : 16];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kw_ = wave % KSPLIT, pw_ = wave / KSPLIT;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+
+  int pid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
+  const int oc_tiles = (g.OC + BM - 1) / BM;
+  const int oc0 = (pid % oc_tiles) * BM;
+  const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
+  const int OHW = g.OH * g.OW;
+  const int ctiles = g.Cp >> 5;
+
+  // per-lane pixel: linear index of the first input pixel of its receptive field,
+  // and which taps fall inside the image
+  int base_p[TN];
+  unsigned vmask[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int64_t p = px0 + (pw_ * TN + j) * 32 + lrow;
+    const bool ok = p < g.P;
+    const int pp = ok ? (int)p : 0;
+    const int n = pp / OHW;
+    const int rem = pp - n * OHW;
+    const int oh = rem / g.OW, ow = rem - oh * g.OW;
+    const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
+    base_p[j] = (n * g.H + ih0) * g.W + iw0;
+    unsigned m = 0;
+    if (!NOPAD) {
+      int rr = 0, ss = 0;
+      for (int t = 0; t < g.taps; ++t) {
+        const int ih = ih0 + rr * g.DH, iw = iw0 + ss * g.DW;
+        m |= (ok && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W ? 1u : 0u) << t;
+        if (++ss == g.KW) { ss = 0; ++rr; }
+      }
+    }
+    vmask[j] = m;
+  }
+
+  // K range of this wavefront, in chunks of 32 bytes; chunks past the true K are never visited
+  const int nch = g.Kp >> 5;
+  const int nlive = g.K >> 5;
+  const int per = (nlive + KSPLIT - 1) / KSPLIT;
+  const int c_begin = kw_ * per;
+  const int c_end = c_begin + per < nlive ? c_begin + per : nlive;
+  const int niter = (per + D - 1) / D;
+  int cur = c_begin;
+  int tap = (cur * 32) / g.Cp;
+  int ch = cur * 32 - tap * g.Cp;
+  int r = tap / g.KW, s = tap - r * g.KW;
+
+  const int8_t* wa[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + i) * (nch + 1)) * 1024 + lane * 16;
+  const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
+
+  // bias of the groups this wavefront finalises, fetched before the K loop
+  int gi[NU], gj[NU], gq[NU];
+  int4 bias_v[NU];
+#pragma unroll
+  for (int m = 0; m < NU; ++m) {
+    const int u = KSPLIT == 1 ? m : kw_ + KSPLIT * m;
+    gi[m] = u / (TN * 4);
+    gj[m] = (u >> 2) % TN;
+    gq[m] = u & 3;
+    bias_v[m] = bias4(ep, g.OC, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
+  }
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  // one batch = D chunks of both operands, one SSA value (see k_conv_igemm)
+  typedef int regs_t __attribute__((ext_vector_type(4 * (TM + TN) * D)));
+  auto fetch = [&]() __attribute__((always_inline)) -> regs_t {
+    regs_t R;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const bool live = cur < c_end;
+      // a chunk past the end multiplies the all-zero filter chunk with a valid activation address
+      const int chunk = live ? cur : nch;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int4 v = *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024);
+        const int b = (d * (TM + TN) + i) * 4;
+        R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
+      }
+      const int soff = live ? (r * g.DH) * g.W + s * g.DW : 0;  // in pixels
+      const int coff = live ? (ch >> 5) * 1024 : 0;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int pin = base_p[j] + soff;
+        const int8_t* src = xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + coff + lgrp * 512 + (pin & 31) * 16);
+        if (!NOPAD) src = (live && ((vmask[j] >> tap) & 1u)) ? src : zero;
+        const int4 v = *reinterpret_cast<const int4*>(src);
+        const int b = (d * (TM + TN) + TM + j) * 4;
+        R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
+      }
+      if (live) {
+        ++cur;
+        ch += 32;
+        if (ch >= g.Cp) {
+          ch = 0;
+          ++tap;
+          if (++s == g.KW) { s = 0; ++r; }
+        }
+      }
+    }
+    return R;
+  };
+  auto consume = [&](const regs_t R) __attribute__((always_inline)) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      v4i a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int o = (d * (TM + TN) + i) * 4;
+        a[i] = v4i{R[o], R[o + 1], R[o + 2], R[o + 3]};
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int o = (d * (TM + TN) + TM + j) * 4;
+        b[j] = v4i{R[o], R[o + 1], R[o + 2], R[o + 3]};
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  regs_t R0 = fetch();
+  regs_t R1;
+  for (int it = 0; it < niter; it += 2) {
+    R1 = fetch();
+    consume(R0);
+    if (it + 1 >= niter) break;
+    R0 = fetch();
+    consume(R1);
+  }
+
+  // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS
+  if (KSPLIT > 1) {
+    int* mine = sPart + wave * U * 256;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<int4*>(mine + (((i * TN + j) * 4 + q) * 64 + lane) * 4) =
+              make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+    __syncthreads();
+  }
+
+  // ---- finalise: wavefront kw_ owns the groups u = kw_ + KSPLIT * m of its tile
+  int32_t val[NU * 4];
+#pragma unroll
+  for (int m = 0; m < NU; ++m) {
+    int4 sum = bias_v[m];
+    if (KSPLIT == 1) {
+      // u == m is a compile-time constant here: plain register reads
+      const v16i& a = acc[m / (TN * 4)][(m >> 2) % TN];
+      const int q = (m & 3) * 4;
+      sum.x = wadd(sum.x, a[q]); sum.y = wadd(sum.y, a[q + 1]); sum.z = wadd(sum.z, a[q + 2]); sum.w = wadd(sum.w, a[q + 3]);
+    } else {
+      const int u = kw_ + KSPLIT * m;
+#pragma unroll
+      for (int k = 0; k < KSPLIT; ++k) {
+        const int4 v = *reinterpret_cast<const int4*>(sPart + (((pw_ * KSPLIT + k) * U + u) * 64 + lane) * 4);
+        sum.x = wadd(sum.x, v.x); sum.y = wadd(sum.y, v.y); sum.z = wadd(sum.z, v.z); sum.w = wadd(sum.w, v.w);
+      }
+    }
+    val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
+  }
+  if (ep.residual) {
+    uint32_t rp[NU];
+#pragma unroll
+    for (int m = 0; m < NU; ++m)
+      rp[m] = residual4(ep, g.P, px0 + (pw_ * TN + gj[m]) * 32 + lrow, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
+    run_chain(ep.chain, val);
+#pragma unroll
+    for (int e = 0; e < NU * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
+    run_chain(ep.chain2, val);
+  } else {
+    run_chain(ep.chain, val);
+  }
+
+  if (OUT == OUT_I32_NCHW) {
+#pragma unroll
+    for (int m = 0; m < NU; ++m) {
+      const int64_t p = px0 + (pw_ * TN + gj[m]) * 32 + lrow;
+      if (p >= g.P) continue;
+      const int n = (int)p / OHW;
+      const int rem = (int)p - n * OHW;
+      const int oc = oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4;
+      int32_t* y32 = reinterpret_cast<int32_t*>(out) + ((int64_t)n * g.OC + oc) * OHW + rem;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (oc + e < g.OC) y32[(int64_t)e * OHW] = val[m * 4 + e];
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < NU; ++m) {
+      const int pl = (pw_ * TN + gj[m]) * 32 + lrow;
+      const int ol = gi[m] * 32 + gq[m] * 8 + lgrp * 4;
+      *reinterpret_cast<uint32_t*>(&sOut[pl * OPITCH + ol]) = pack_bytes(val[m * 4], val[m * 4 + 1], val[m * 4 + 2], val[m * 4 + 3]);
+    }
+    __syncthreads();
+    store_tile_i8<BM, BN, NW * 64>(sOut, OPITCH, out, g, ep, oc0, px0, tid);
+  }
+}
+
+constexpr int KSTEP = 64;  // granularity K is padded to
 
 // ---------------------------------------------------------------- packing
-// int32 NCHW -> int8 NHWC (channels padded to cp with zeros); narrowing is
-// static_cast<int8_t>, the reference's own (ops.cc:234).
-__global__ void __launch_bounds__(256) k_pack_nhwc(const int32_t* __restrict__ x, int8_t* __restrict__ xp, int64_t total,
-                                                   int c, int hw, int cp) {
-  const int c4n = cp / 4;
+// int32 NCHW -> int8 activations (layout of conv_mfma.h, padding channels zero);
+// narrowing is static_cast<int8_t>, the reference's own (ops.cc:234).  One
+// thread per dword of the destination.
+__global__ void __launch_bounds__(256) k_pack_act(const int32_t* __restrict__ x, uint32_t* __restrict__ xp, int64_t total,
+                                                  int64_t npix, int c, int hw, int cp) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int pix = (int)(i % hw);
-    const int64_t t = i / hw;
-    const int c4 = (int)(t % c4n);
-    const int64_t n = t / c4n;
+    int64_t p;
+    int c0;
+    act_decode(i, cp, &p, &c0);
+    if (p >= npix) continue;
+    const int64_t n = p / hw;
+    const int pix = (int)(p - n * hw);
     uint32_t pack = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int ch = c4 * 4 + j;
-      const int32_t v = ch < c ? x[((int64_t)n * c + ch) * hw + pix] : 0;
+      const int ch = c0 + j;
+      const int32_t v = ch < c ? x[(n * c + ch) * hw + pix] : 0;
       pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
     }
-    *reinterpret_cast<uint32_t*>(xp + ((int64_t)n * hw + pix) * cp + c4 * 4) = pack;
+    xp[i] = pack;
   }
 }
 
-// int32 OIHW -> int8 [OCp][Kp], k = (r*KW + s)*Cp + c, zero padded
+// int32 OIHW -> int8 filter in MFMA-fragment order.  With k = (r*KW + s)*Cp + c the
+// matrix [OCp][Kp] is cut into 32-row tiles and 32-byte K chunks; one chunk of
+// one tile is stored as the 1 KiB a wavefront feeds to v_mfma_i32_32x32x32_i8:
+// lane l holds row (l & 31), bytes (l >> 5)*16 .. +15 of the chunk.  Each tile
+// has nch + 1 chunks; the last one is all zero (a K range that ends early reads
+// it instead of branching).  Layout: [OCp/32][nch + 1][64][16].
 __global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict__ w, int8_t* __restrict__ wp, int64_t total,
-                                                      int oc, int ic, int taps, int cp, int kp) {
-  const int k4n = kp / 4;
+                                                      int oc, int ic, int taps, int cp, int nch) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int k4 = (int)(i % k4n);
-    const int64_t o = i / k4n;
-    const int k = k4 * 4;
+    const int d = (int)(i & 3);
+    const int lane = (int)((i >> 2) & 63);
+    const int64_t t = i >> 8;
+    const int chunk = (int)(t % (nch + 1));
+    const int64_t tile = t / (nch + 1);
+    const int64_t o = tile * 32 + (lane & 31);
+    const int k = chunk * 32 + (lane >> 5) * 16 + d * 4;
     const int tap = k / cp, c = k - tap * cp;
     uint32_t pack = 0;
-    if (o < oc && tap < taps) {
+    if (o < oc && tap < taps && chunk < nch) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int32_t v = (c + j < ic) ? w[((int64_t)o * ic + c + j) * taps + tap] : 0;
         pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
       }
     }
-    *reinterpret_cast<uint32_t*>(wp + o * kp + k) = pack;
+    reinterpret_cast<uint32_t*>(wp)[i] = pack;
   }
 }
 
-// int8 NHWC (padded to cp) -> int32 NCHW
-__global__ void __launch_bounds__(256) k_unpack_nchw(const int8_t* __restrict__ xp, int32_t* __restrict__ x, int64_t total,
-                                                     int c, int hw, int cp) {
+// int8 activations -> int32 NCHW
+__global__ void __launch_bounds__(256) k_unpack_act(const int8_t* __restrict__ xp, int32_t* __restrict__ x, int64_t total,
+                                                    int c, int hw, int cp) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
     const int pix = (int)(i % hw);
     const int64_t t = i / hw;
     const int ch = (int)(t % c);
     const int64_t n = t / c;
-    x[i] = xp[((int64_t)n * hw + pix) * cp + ch];
+    x[i] = xp[act_offset(n * hw + pix, ch, cp)];
   }
 }
 
@@ -484,10 +765,11 @@ k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const 
 int pad_channels(int c) {
   if (c <= 4) return 4;
   if (c <= 8) return 8;
-  return (c + 15) / 16 * 16;
+  if (c <= 16) return 16;
+  return (c + 31) / 32 * 32;
 }
 
-size_t packed_act_bytes(int64_t npix, int c) { return ((size_t)npix * pad_channels(c) + 255) / 256 * 256; }
+size_t packed_act_bytes(int64_t npix, int c) { return ((size_t)act_bytes(npix, pad_channels(c)) + 255) / 256 * 256; }
 
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp) {
   const int cp = pad_channels(ic);
@@ -498,30 +780,34 @@ void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp) {
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw) {
   int ocp, kp;
   weight_dims(oc, ic, kh, kw, &ocp, &kp);
-  return ((size_t)ocp * kp + 512 + 255) / 256 * 256;  // 512: fetches run up to two K steps past the end
+  // one zero chunk per 32-row tile, and 8 KiB of slack: the pipelined fetch of
+  // the LDS kernel reads up to two K steps past the last tile and never uses them
+  return (size_t)(ocp / 32) * (kp / 32 + 1) * 1024 + 8192;
 }
 
 int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStream_t s) {
   const int cp = pad_channels(c);
-  const int64_t total = (int64_t)n * (cp / 4) * hw;
+  const int64_t npix = (int64_t)n * hw;
+  const int64_t total = act_bytes(npix, cp) / 4;
   if (total == 0) return CVMHIP_OK;
-  KernelTimer timer("k_pack_nhwc", (double)n * c * hw * 5.0, s);  // bytes: 4 read + 1 written per element
-  k_pack_nhwc<<<grid_for(total, 256), 256, 0, s>>>(x, xp, total, c, hw, cp);
-  return check_launch("pack_nhwc");
+  KernelTimer timer("k_pack_act", (double)n * c * hw * 5.0, s);  // bytes: 4 read + 1 written per element
+  k_pack_act<<<grid_for(total, 256), 256, 0, s>>>(x, reinterpret_cast<uint32_t*>(xp), total, npix, c, hw, cp);
+  return check_launch("pack_act");
 }
 
 int unpack_activations(const int8_t* xp, int32_t* x, int n, int c, int hw, hipStream_t s) {
   const int64_t total = (int64_t)n * c * hw;
   if (total == 0) return CVMHIP_OK;
-  k_unpack_nchw<<<grid_for(total, 256), 256, 0, s>>>(xp, x, total, c, hw, pad_channels(c));
-  return check_launch("unpack_nchw");
+  k_unpack_act<<<grid_for(total, 256), 256, 0, s>>>(xp, x, total, c, hw, pad_channels(c));
+  return check_launch("unpack_act");
 }
 
 int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, hipStream_t s) {
   int ocp, kp;
   weight_dims(oc, ic, kh, kw, &ocp, &kp);
-  const int64_t total = (int64_t)ocp * (kp / 4);
-  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, ic, kh * kw, pad_channels(ic), kp);
+  const int nch = kp / 32;
+  const int64_t total = (int64_t)(ocp / 32) * (nch + 1) * 256;  // dwords
+  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, ic, kh * kw, pad_channels(ic), nch);
   return check_launch("pack_weights");
 }
 
@@ -553,17 +839,72 @@ static void launch_out(int wm, int wn, int gran, bool wide, unsigned grid, hipSt
   else launch_tile<1, 1, OUT>(gran, wide, grid, s, xp, wp, out, g, ep);
 }
 
+// ---- wavefront-private kernel: configurations and choice
+struct WaveCfg { int tm, tn, ksplit, nw; };
+static const WaveCfg kWaveCfgs[] = {
+    {2, 2, 1, 4}, {2, 2, 2, 4}, {2, 2, 4, 4}, {2, 2, 8, 8}, {1, 2, 4, 4}, {1, 2, 8, 8}, {1, 2, 1, 4},
+};
+constexpr int kNumWaveCfgs = sizeof(kWaveCfgs) / sizeof(kWaveCfgs[0]);
+
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW>
+static void launch_wave_cfg(bool i8, bool nopad, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+                            const ConvGeom& g, const Epilogue& ep) {
+  if (i8) {
+    if (nopad) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I8_ACT, true><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+    else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I8_ACT, false><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+  } else {
+    if (nopad) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I32_NCHW, true><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+    else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I32_NCHW, false><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+  }
+}
+
+static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
+  const int bm = 32 * c.tm, bn = 32 * c.tn * (c.nw / c.ksplit);
+  return (int64_t)((g.OC + bm - 1) / bm) * ((g.P + bn - 1) / bn);
+}
+
+// The smallest K split of the largest tile that puts about 1.5 wavefronts on
+// every SIMD of the chip; a wavefront must keep at least two chunks of K.
+static int choose_wave_cfg(const ConvGeom& g) {
+  const int nlive = g.K / 32;
+  int best = 0;
+  int64_t best_waves = 0;
+  for (int i = 0; i < kNumWaveCfgs; ++i) {
+    const WaveCfg& c = kWaveCfgs[i];
+    if (c.ksplit > 1 && nlive < 2 * c.ksplit) continue;
+    const int64_t waves = wave_cfg_blocks(c, g) * c.nw;
+    if (waves >= 1536) return i;
+    if (waves > best_waves) { best_waves = waves; best = i; }
+  }
+  return best;
+}
+
+static void launch_wave(int cfg, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+                        const ConvGeom& g, const Epilogue& ep) {
+  const bool i8 = ep.out_mode == OUT_I8_ACT;
+  const bool nopad = g.PH == 0 && g.PW == 0;
+  switch (cfg) {
+    case 0: launch_wave_cfg<2, 2, 1, 4, 2, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 1: launch_wave_cfg<2, 2, 2, 4, 4, 1>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 2: launch_wave_cfg<2, 2, 4, 4, 4, 1>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 3: launch_wave_cfg<2, 2, 8, 8, 2, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 4: launch_wave_cfg<1, 2, 4, 4, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 5: launch_wave_cfg<1, 2, 8, 8, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    default: launch_wave_cfg<1, 2, 1, 4, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+  }
+}
+
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
   const Epilogue& ep0 = ep_in;
   if (g.N < 1 || g.H < 1 || g.W < 1 || g.OC < 1 || g.OH < 1 || g.OW < 1 || g.KH < 1 || g.KW < 1 || g.SH < 1 ||
       g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
     return arg_error("conv geometry");
-  if (g.Cp != 4 && g.Cp != 8 && (g.Cp % 16) != 0) return arg_error("conv channel padding");
+  if (g.Cp != 4 && g.Cp != 8 && g.Cp != 16 && (g.Cp % 32) != 0) return arg_error("conv channel padding");
   if (((uintptr_t)xp | (uintptr_t)wp) & 15) return arg_error("conv operand alignment");
-  if ((ep0.out_mode == OUT_I8_NHWC || ep0.residual) && (ep0.out_cp % 4 != 0 || ep0.out_cp < g.OC))
+  if ((ep0.out_mode == OUT_I8_ACT || ep0.residual) && ep0.out_cp != pad_channels(g.OC))
     return arg_error("conv int8 output layout");
   if (((uintptr_t)out | (uintptr_t)ep0.residual) & 3) return arg_error("conv output alignment");
-  if (ep0.out_mode == OUT_I8_NHWC && (ep0.out_cp & 15) == 0 && ((uintptr_t)out & 15)) return arg_error("conv output alignment");
+  if (ep0.out_mode == OUT_I8_ACT && ep0.out_cp >= 16 && ((uintptr_t)out & 15)) return arg_error("conv output alignment");
   g.taps = g.KH * g.KW;
   g.K = g.taps * g.Cp;
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
@@ -585,6 +926,23 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
     wm = forced[0] - '0';
     wn = forced[2] - '0';
   }
+  // kernel choice: "wave" (no LDS in the K loop) when the layout allows it, else the LDS-tiled kernel;
+  // test and tuning hooks: CVM_HIP_CONV=lds forces the tiled kernel, CVM_HIP_WAVECFG=<index> a configuration
+  const char* conv_kind = getenv("CVM_HIP_CONV");
+  const char* wave_forced = getenv("CVM_HIP_WAVECFG");
+  const bool wave_ok = (g.Cp % 32) == 0 && ((g.PH == 0 && g.PW == 0) || g.taps <= 32);
+  bool use_wave = wave_ok;
+  if (conv_kind && conv_kind[0] == 'l') use_wave = false;
+  if (conv_kind && conv_kind[0] == 'w') use_wave = wave_ok;
+  if (use_wave) {
+    int cfg = choose_wave_cfg(g);
+    if (wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
+    const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
+    if (wnb > 0x7fffffff) return arg_error("conv grid too large");
+    KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+    launch_wave(cfg, (unsigned)wnb, s, xp, wp, out, g, ep);
+    return check_launch("conv_wave");
+  }
   const int64_t nb = blocks(64 * wm, 64 * wn);
   if (nb > 0x7fffffff) return arg_error("conv grid too large");
   const unsigned grid = (unsigned)nb;
@@ -595,7 +953,7 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   g.adv_tap = ks / g.Cp;
   g.adv_r = g.adv_tap / g.KW;
   g.adv_s = g.adv_tap % g.KW;
-  if (ep.out_mode == OUT_I8_NHWC) launch_out<OUT_I8_NHWC>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
+  if (ep.out_mode == OUT_I8_ACT) launch_out<OUT_I8_ACT>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
   else launch_out<OUT_I32_NCHW>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
   return check_launch("conv_igemm");
 }

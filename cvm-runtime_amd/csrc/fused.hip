@@ -1,4 +1,4 @@
-// Entry points of the fused int8 path: int8 NHWC activations between layers,
+// Entry points of the fused int8 path: int8 activations (layout: conv_mfma.h) between layers,
 // requantisation chains folded into the producing kernel.  The arithmetic of
 // every stage is the operator's own (int32, wrapping), so results equal the
 // node-by-node execution bit for bit.
@@ -12,11 +12,13 @@ __device__ __forceinline__ uint32_t pack4(int32_t a, int32_t b, int32_t c, int32
 }
 __device__ __forceinline__ int32_t byte_of(uint32_t w, int e) { return (int32_t)(int8_t)(w >> (8 * e)); }
 
-// out = chain(a + b): one thread per (pixel, 4-channel group)
+// All kernels below run one thread per dword (4 channels of one pixel) of the
+// int8 result, in memory order, whatever the layout (conv_mfma.h: act_decode).
+
+// out = chain(a + b)
 __global__ void __launch_bounds__(256)
 k_add_i8(const uint32_t* __restrict__ a, const uint32_t* __restrict__ b, void* __restrict__ out, int out_is_i8,
-         int64_t total, int c, int cp, int hw, DevChain chain) {
-  const int c4n = cp / 4;
+         int64_t total, int64_t npix, int c, int cp, int hw, DevChain chain) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
     const uint32_t u = a[i], v = b[i];
@@ -26,25 +28,29 @@ k_add_i8(const uint32_t* __restrict__ a, const uint32_t* __restrict__ b, void* _
     if (out_is_i8) {
       reinterpret_cast<uint32_t*>(out)[i] = pack4(r[0], r[1], r[2], r[3]);
     } else {
-      const int c4 = (int)(i % c4n);
-      const int64_t pixel = i / c4n;
+      int64_t pixel;
+      int c0;
+      act_decode(i, cp, &pixel, &c0);
+      if (pixel >= npix) continue;
       const int64_t n = pixel / hw;
       const int pix = (int)(pixel - n * hw);
       int32_t* y = reinterpret_cast<int32_t*>(out) + (n * c) * hw + pix;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (c4 * 4 + e < c) y[(int64_t)(c4 * 4 + e) * hw] = r[e];
+        if (c0 + e < c) y[(int64_t)(c0 + e) * hw] = r[e];
     }
   }
 }
 
 __global__ void __launch_bounds__(256)
-k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t total, int c4n, int h, int w, int oh,
-              int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
+k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t total, int64_t npix_out, int cp, int h, int w,
+              int oh, int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int c4 = (int)(i % c4n);
-    int64_t t = i / c4n;
+    int64_t t;
+    int c0;
+    act_decode(i, cp, &t, &c0);
+    if (t >= npix_out) continue;
     const int q = (int)(t % ow);
     t /= ow;
     const int p = (int)(t % oh);
@@ -56,7 +62,7 @@ k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t 
       for (int s = 0; s < kw; ++s) {
         const int iw = q * sw + s - pw;
         if (iw < 0 || iw >= w) continue;
-        const uint32_t v = x[((n * h + ih) * w + iw) * c4n + c4];
+        const uint32_t v = x[act_offset((n * h + ih) * w + iw, c0, cp) >> 2];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int32_t b = byte_of(v, e);
@@ -68,18 +74,19 @@ k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t 
   }
 }
 
-// out[n][c] = chain(sum_hw x[n][hw][c]): one thread per (n, 4-channel group)
+// out[n][c] = chain(sum_hw x[n][hw][c]); the result is a tensor of n "pixels"
 __global__ void __launch_bounds__(256)
-k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i8, int64_t total, int c, int c4n,
+k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i8, int64_t total, int nimg, int c, int cp,
             int hw, DevChain chain) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int c4 = (int)(i % c4n);
-    const int64_t n = i / c4n;
+    int64_t n;
+    int c0;
+    act_decode(i, cp, &n, &c0);
+    if (n >= nimg) continue;
     int32_t acc[4] = {0, 0, 0, 0};
-    const uint32_t* p = x + n * hw * c4n + c4;
     for (int t = 0; t < hw; ++t) {
-      const uint32_t v = p[(int64_t)t * c4n];
+      const uint32_t v = x[act_offset(n * hw + t, c0, cp) >> 2];
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e);
     }
@@ -90,20 +97,23 @@ k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (c4 * 4 + e < c) reinterpret_cast<int32_t*>(out)[n * c + c4 * 4 + e] = acc[e];
+        if (c0 + e < c) reinterpret_cast<int32_t*>(out)[n * c + c0 + e] = acc[e];
     }
   }
 }
 
-// depthwise: one thread per (output pixel, 4-channel group); filter is [tap][cp] int8
+// depthwise convolution; filter is [tap][cp] int8
 __global__ void __launch_bounds__(256)
 k_depthwise_i8(const uint32_t* __restrict__ x, const uint32_t* __restrict__ wp, const int32_t* __restrict__ bias,
-               void* __restrict__ out, int out_is_i8, int64_t total, int c, int c4n, int h, int w, int oh, int ow,
-               int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw, DevChain chain) {
+               void* __restrict__ out, int out_is_i8, int64_t total, int64_t npix_out, int c, int cp, int h, int w, int oh,
+               int ow, int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw, DevChain chain) {
+  const int c4n = cp >> 2;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int c4 = (int)(i % c4n);
-    int64_t t = i / c4n;
+    int64_t t;
+    int c0;
+    act_decode(i, cp, &t, &c0);
+    if (t >= npix_out) continue;
     const int q = (int)(t % ow);
     t /= ow;
     const int p = (int)(t % oh);
@@ -115,8 +125,8 @@ k_depthwise_i8(const uint32_t* __restrict__ x, const uint32_t* __restrict__ wp, 
       for (int s = 0; s < kw; ++s) {
         const int iw = q * sw + s * dw - pw;
         if (iw < 0 || iw >= w) continue;
-        const uint32_t v = x[((n * h + ih) * w + iw) * c4n + c4];
-        const uint32_t f = wp[(r * kw + s) * c4n + c4];
+        const uint32_t v = x[act_offset((n * h + ih) * w + iw, c0, cp) >> 2];
+        const uint32_t f = wp[(r * kw + s) * c4n + (c0 >> 2)];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e) * byte_of(f, e);
       }
@@ -124,7 +134,7 @@ k_depthwise_i8(const uint32_t* __restrict__ x, const uint32_t* __restrict__ wp, 
     int32_t rr[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int ch = c4 * 4 + e;
+      const int ch = c0 + e;
       rr[e] = ch < c ? apply_chain(chain, wadd(acc[e], bias ? bias[ch] : 0)) : 0;
     }
     if (out_is_i8) {
@@ -133,7 +143,7 @@ k_depthwise_i8(const uint32_t* __restrict__ x, const uint32_t* __restrict__ wp, 
       int32_t* y = reinterpret_cast<int32_t*>(out) + ((n * c) * oh + p) * ow + q;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (c4 * 4 + e < c) y[(int64_t)(c4 * 4 + e) * oh * ow] = rr[e];
+        if (c0 + e < c) y[(int64_t)(c0 + e) * oh * ow] = rr[e];
     }
   }
 }
@@ -187,7 +197,7 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
   ep.bias = bias;
   if (!make_chain(chain, &ep.chain) || !make_chain(chain2, &ep.chain2)) return arg_error("conv2d_i8 chain");
   ep.residual = reinterpret_cast<const int8_t*>(residual);
-  ep.out_mode = out_is_i8 ? OUT_I8_NHWC : OUT_I32_NCHW;
+  ep.out_mode = out_is_i8 ? OUT_I8_ACT : OUT_I32_NCHW;
   ep.out_cp = pad_channels(oc);
   return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep,
                     as_stream(stream));
@@ -218,12 +228,13 @@ int cvmhip_depthwise_conv2d_i8(const void* xp, const void* wp, const int32_t* bi
   if (!make_chain(chain, &ch)) return arg_error("depthwise_conv2d_i8 chain");
   const int oh = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
   const int ow = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
-  const int c4n = pad_channels(c) / 4;
-  const int64_t total = (int64_t)n * oh * ow * c4n;
+  const int cp = pad_channels(c);
+  const int64_t npix = (int64_t)n * oh * ow;
+  const int64_t total = act_bytes(npix, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_depthwise_i8", (double)n * c * ((double)h * wd + (double)oh * ow), s);  // bytes in + out
   k_depthwise_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(
-      reinterpret_cast<const uint32_t*>(xp), reinterpret_cast<const uint32_t*>(wp), bias, out, out_is_i8, total, c, c4n,
+      reinterpret_cast<const uint32_t*>(xp), reinterpret_cast<const uint32_t*>(wp), bias, out, out_is_i8, total, npix, c, cp,
       h, wd, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, ch);
   return check_launch("depthwise_conv2d_i8");
 }
@@ -235,11 +246,12 @@ int cvmhip_add_i8(const void* a, const void* b, const cvmhip_chain* chain, void*
   DevChain ch;
   if (!make_chain(chain, &ch)) return arg_error("add_i8 chain");
   const int cp = pad_channels(c);
-  const int64_t total = (int64_t)n * hw * (cp / 4);
+  const int64_t npix = (int64_t)n * hw;
+  const int64_t total = act_bytes(npix, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_add_i8", (double)n * c * hw * 3.0, s);
   k_add_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(a), reinterpret_cast<const uint32_t*>(b),
-                                                out, out_is_i8, total, c, cp, hw, ch);
+                                                out, out_is_i8, total, npix, c, cp, hw, ch);
   return check_launch("add_i8");
 }
 
@@ -251,12 +263,13 @@ int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, i
   // every window must touch the input, otherwise the int32 result (INT32_MIN) has no int8 form
   if ((oh - 1) * stride_h - pad_h >= h || (ow - 1) * stride_w - pad_w >= w) return arg_error("max_pool2d_i8 window");
   if (((uintptr_t)xp | (uintptr_t)yp) & 3) return arg_error("max_pool2d_i8 alignment");
-  const int c4n = pad_channels(c) / 4;
-  const int64_t total = (int64_t)n * oh * ow * c4n;
+  const int cp = pad_channels(c);
+  const int64_t npix = (int64_t)n * oh * ow;
+  const int64_t total = act_bytes(npix, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_max_pool_i8", (double)n * c * ((double)h * w + (double)oh * ow), s);
   k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
-                                                            reinterpret_cast<uint32_t*>(yp), total, c4n, h, w, oh, ow,
+                                                            reinterpret_cast<uint32_t*>(yp), total, npix, cp, h, w, oh, ow,
                                                             kh, kw, stride_h, stride_w, pad_h, pad_w);
   return check_launch("max_pool2d_i8");
 }
@@ -267,10 +280,10 @@ int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int o
   if (((uintptr_t)xp | (uintptr_t)out) & 3) return arg_error("sum_hw_i8 alignment");
   DevChain ch;
   if (!make_chain(chain, &ch)) return arg_error("sum_hw_i8 chain");
-  const int c4n = pad_channels(c) / 4;
-  const int64_t total = (int64_t)n * c4n;
+  const int cp = pad_channels(c);
+  const int64_t total = act_bytes(n, cp) / 4;
   hipStream_t s = as_stream(stream);
-  k_sum_hw_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, c, c4n,
+  k_sum_hw_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
                                                    hw, ch);
   return check_launch("sum_hw_i8");
 }

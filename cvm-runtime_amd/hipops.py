@@ -291,7 +291,9 @@ def non_max_suppression(x, valid_count, y, iou_threshold=50, force_suppress=Fals
 
 
 # ---------------------------------------------------------------- fused int8 path
-# int8 NHWC tensors are torch int8 tensors of shape (n, h*w, cp); filters are
+# int8 activation tensors are flat torch int8 buffers in the library's own
+# layout (NHWC for up to 16 padded channels, else blocks of 32 pixels x 32
+# channels in MFMA fragment order; act_offset below restates it); filters are
 # opaque byte buffers made by pack_weights / pack_depthwise_weights.
 
 class Stage(ctypes.Structure):
@@ -330,15 +332,25 @@ def pad_channels(c):
     return lib().cvmhip_pad_channels(c)
 
 
-def pack_nhwc_i8(x):
+def act_offset(p, c, cp):
+    """Byte offset of channel c of pixel p (numpy arrays allowed) in an int8 activation buffer."""
+    if cp % 32:
+        return p * cp + c
+    return ((p >> 5) * (cp >> 5) + (c >> 5)) * 1024 + ((c >> 4) & 1) * 512 + (p & 31) * 16 + (c & 15)
+
+
+def _act_buffer(npix, c, dev):
+    return torch.zeros(lib().cvmhip_packed_act_bytes(ctypes.c_int64(npix), c), dtype=torch.int8, device=dev)
+
+
+def pack_act_i8(x):
     n, c, h, w = x.shape
-    xp = torch.empty((n, h * w, pad_channels(c)), dtype=torch.int8, device=x.device)
+    xp = _act_buffer(n * h * w, c, x.device)
     check(lib().cvmhip_pack_nhwc_i8(_ptr(x), _vp(xp), n, c, h * w, _stream()))
     return xp
 
 
-def unpack_nhwc_i8(xp, c, h, w):
-    n = xp.shape[0]
+def unpack_act_i8(xp, n, c, h, w):
     x = torch.empty((n, c, h, w), dtype=torch.int32, device=xp.device)
     check(lib().cvmhip_unpack_nhwc_i8(_vp(xp), _ptr(x), n, c, h * w, _stream()))
     return x
@@ -351,12 +363,11 @@ def pack_weights(w):
     return wp
 
 
-def conv2d_i8(xp, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=None, chain2=None, out_is_i8=True,
+def conv2d_i8(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=None, chain2=None, out_is_i8=True,
               strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
-    n = xp.shape[0]
     oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
     if out_is_i8:
-        out = torch.empty((n, oh * ow, pad_channels(oc)), dtype=torch.int8, device=xp.device)
+        out = _act_buffer(n * oh * ow, oc, xp.device)
     else:
         out = torch.empty((n, oc, oh, ow), dtype=torch.int32, device=xp.device)
     check(lib().cvmhip_conv2d_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
@@ -373,12 +384,11 @@ def pack_depthwise_weights(w):
     return wp
 
 
-def depthwise_conv2d_i8(xp, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_i8=True,
+def depthwise_conv2d_i8(xp, n, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_i8=True,
                         strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
-    n = xp.shape[0]
     oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
     if out_is_i8:
-        out = torch.empty((n, oh * ow, pad_channels(c)), dtype=torch.int8, device=xp.device)
+        out = _act_buffer(n * oh * ow, c, xp.device)
     else:
         out = torch.empty((n, c, oh, ow), dtype=torch.int32, device=xp.device)
     check(lib().cvmhip_depthwise_conv2d_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
@@ -387,10 +397,9 @@ def depthwise_conv2d_i8(xp, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_
     return out
 
 
-def add_i8(a, b, c, h, w, chain1=None, out_is_i8=True):
-    n = a.shape[0]
+def add_i8(a, b, n, c, h, w, chain1=None, out_is_i8=True):
     if out_is_i8:
-        out = torch.empty_like(a)
+        out = torch.zeros_like(a)
     else:
         out = torch.empty((n, c, h, w), dtype=torch.int32, device=a.device)
     check(lib().cvmhip_add_i8(_vp(a), _vp(b), ctypes.byref(chain1) if chain1 else None, _vp(out), int(out_is_i8),
@@ -398,18 +407,16 @@ def add_i8(a, b, c, h, w, chain1=None, out_is_i8=True):
     return out
 
 
-def max_pool2d_i8(xp, c, h, w, pool_size, strides, padding, oh, ow):
-    n = xp.shape[0]
-    out = torch.empty((n, oh * ow, xp.shape[2]), dtype=torch.int8, device=xp.device)
+def max_pool2d_i8(xp, n, c, h, w, pool_size, strides, padding, oh, ow):
+    out = _act_buffer(n * oh * ow, c, xp.device)
     check(lib().cvmhip_max_pool2d_i8(_vp(xp), _vp(out), n, c, h, w, oh, ow, pool_size[0], pool_size[1],
                                      strides[0], strides[1], padding[0], padding[1], _stream()))
     return out
 
 
-def sum_hw_i8(xp, c, hw, chain1=None, out_is_i8=False):
-    n = xp.shape[0]
+def sum_hw_i8(xp, n, c, hw, chain1=None, out_is_i8=False):
     if out_is_i8:
-        out = torch.empty((n, 1, xp.shape[2]), dtype=torch.int8, device=xp.device)
+        out = _act_buffer(n, c, xp.device)
     else:
         out = torch.empty((n, c), dtype=torch.int32, device=xp.device)
     check(lib().cvmhip_sum_hw_i8(_vp(xp), ctypes.byref(chain1) if chain1 else None, _vp(out), int(out_is_i8),

@@ -18,13 +18,16 @@ def T(a, dev):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(dev)
 
 
-def nhwc_to_nchw(t, c, h, w):
-    """int8 NHWC (n, h*w, cp) device tensor -> int32 NCHW numpy, padding channels dropped (and checked zero)."""
+def act_to_nchw(t, n, c, h, w):
+    """int8 activation buffer (library layout) -> int32 NCHW numpy; padding channels are checked to be zero."""
     torch.cuda.synchronize()
-    a = t.cpu().numpy().astype(np.int32)
-    n = a.shape[0]
-    assert not a[:, :, c:].any(), "padding channels must stay zero"
-    return np.ascontiguousarray(a[:, :, :c].reshape(n, h, w, c).transpose(0, 3, 1, 2))
+    a = t.cpu().numpy()
+    cp = hipops.pad_channels(c)
+    p = np.arange(n * h * w, dtype=np.int64)[:, None]
+    ch = np.arange(cp, dtype=np.int64)[None, :]
+    full = a[hipops.act_offset(p, ch, cp)].astype(np.int32)          # (pixels, cp)
+    assert not full[:, c:].any(), "padding channels must stay zero"
+    return np.ascontiguousarray(full[:, :c].reshape(n, h, w, c).transpose(0, 3, 1, 2))
 
 
 def run_chain(v, stages):
@@ -48,13 +51,13 @@ def eq(got, ref, what):
             what, len(bad), ref.size, bad[0], got[tuple(bad[0])], ref[tuple(bad[0])]))
 
 
-@pytest.mark.parametrize("c", [1, 3, 5, 8, 20, 64])
+@pytest.mark.parametrize("c", [1, 3, 5, 8, 13, 20, 64, 100])
 def test_pack_unpack_round_trip(c, dev):
     x = synth.tensor("pack-%d" % c, "x", (3, c, 7, 5), -128, 127)
-    xp = hipops.pack_nhwc_i8(T(x, dev))
-    assert xp.shape[2] == hipops.pad_channels(c) and xp.shape[2] >= c
-    eq(nhwc_to_nchw(xp, c, 7, 5), x, "pack")
-    y = hipops.unpack_nhwc_i8(xp, c, 7, 5)
+    xp = hipops.pack_act_i8(T(x, dev))
+    assert hipops.pad_channels(c) >= c
+    eq(act_to_nchw(xp, 3, c, 7, 5), x, "pack")
+    y = hipops.unpack_act_i8(xp, 3, c, 7, 5)
     torch.cuda.synchronize()
     eq(y.cpu().numpy(), x, "unpack")
 
@@ -62,8 +65,8 @@ def test_pack_unpack_round_trip(c, dev):
 def test_pack_narrows_like_static_cast(dev):
     # values outside int8 are truncated exactly as the reference's static_cast<int8_t> (ops.cc:234)
     x = np.array([127, 128, 255, 256, -128, -129, 1000, -1000, 2**31 - 1, -2**31], np.int64).astype(np.int32).reshape(1, 10, 1, 1)
-    xp = hipops.pack_nhwc_i8(T(x, dev))
-    eq(nhwc_to_nchw(xp, 10, 1, 1), x.astype(np.int8).astype(np.int32), "narrow")
+    xp = hipops.pack_act_i8(T(x, dev))
+    eq(act_to_nchw(xp, 1, 10, 1, 1), x.astype(np.int8).astype(np.int32), "narrow")
 
 
 FUSED_CONV = [
@@ -82,8 +85,19 @@ FUSED_CONV = [
 ]
 
 
+@pytest.fixture(params=["auto", "lds", "wave"])
+def conv_kernel(request):
+    """Both implicit-GEMM kernels must give the same bits: force each in turn (the library reads the hook per call)."""
+    if request.param == "auto":
+        os.environ.pop("CVM_HIP_CONV", None)
+    else:
+        os.environ["CVM_HIP_CONV"] = request.param
+    yield request.param
+    os.environ.pop("CVM_HIP_CONV", None)
+
+
 @pytest.mark.parametrize("case", FUSED_CONV, ids=lambda c: "n%dc%dh%dw%d_o%dk%d" % c[:6])
-def test_conv2d_i8(case, dev):
+def test_conv2d_i8(case, conv_kernel, dev):
     n, ic, h, w, oc, k, st, pd, bias, ch1, ch2, i8 = case
     cid = "fconv-%s" % (case[:8],)
     x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
@@ -95,18 +109,49 @@ def test_conv2d_i8(case, dev):
     if ch2 is not None:
         r = synth.tensor(cid, "r", ref.shape, -127, 127)
         ref = run_chain(oracle.elemwise("elemwise_add", ref, r), ch2)
-        res_t = hipops.pack_nhwc_i8(T(r, dev))
-    xp = hipops.pack_nhwc_i8(T(x, dev))
+        res_t = hipops.pack_act_i8(T(r, dev))
+    xp = hipops.pack_act_i8(T(x, dev))
     wp = hipops.pack_weights(T(wt, dev))
-    out = hipops.conv2d_i8(xp, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None,
+    out = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None,
                            hipops.chain(*ch1) if ch1 else None, res_t, hipops.chain(*ch2) if ch2 else None,
                            out_is_i8=i8, strides=(st, st), padding=(pd, pd))
     if i8:
         assert ref.min() >= -128 and ref.max() <= 127, "case must be representable"
-        eq(nhwc_to_nchw(out, oc, oh, ow), ref, "conv2d_i8")
+        eq(act_to_nchw(out, n, oc, oh, ow), ref, "conv2d_i8")
     else:
         torch.cuda.synchronize()
         eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32")
+
+
+@pytest.mark.parametrize("cfg", range(7))
+@pytest.mark.parametrize("case", [(3, 96, 11, 13, 100, 3, 1, 1, True), (2, 256, 9, 9, 72, 1, 2, 0, False),
+                                  (1, 64, 8, 8, 40, 3, 2, 1, True)],
+                         ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%d" % c[:8])
+def test_conv_wave_kernel_every_configuration(case, cfg, dev):
+    """All tile / K-split configurations of the wavefront-private kernel, int8 and int32 output, with a residual."""
+    n, ic, h, w, oc, k, st, pd, bias = case
+    cid = "wavecfg-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768) if bias else None
+    ch1, ch2 = [("cvm_right_shift", 8, 11)], [("relu",), ("cvm_right_shift", 8, 1)]
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1)
+    r = synth.tensor(cid, "r", conv.shape, -127, 127)
+    ref8 = run_chain(oracle.elemwise("elemwise_add", run_chain(conv, ch1), r), ch2)
+    xp, wp, rp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev)), hipops.pack_act_i8(T(r, dev))
+    os.environ["CVM_HIP_CONV"] = "wave"
+    os.environ["CVM_HIP_WAVECFG"] = str(cfg)
+    try:
+        out8 = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1), rp,
+                                hipops.chain(*ch2), True, (st, st), (pd, pd))
+        out32 = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, None, None, None, False,
+                                 (st, st), (pd, pd))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_CONV", None)
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+    eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), ref8, "wave cfg %d int8" % cfg)
+    eq(out32.cpu().numpy(), conv, "wave cfg %d int32" % cfg)
 
 
 @pytest.mark.parametrize("case", [(2, 32, 19, 17, 3, 1, 1), (1, 96, 16, 16, 3, 2, 1), (1, 5, 9, 9, 3, 1, 0), (1, 256, 8, 8, 5, 1, 2)],
@@ -119,11 +164,11 @@ def test_depthwise_conv2d_i8(case, dev):
     b = synth.tensor(cid, "b", (c,), -3000, 3000)
     stages = [("relu",), ("cvm_right_shift", 8, 10)]
     ref = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), c), stages)
-    xp = hipops.pack_nhwc_i8(T(x, dev))
+    xp = hipops.pack_act_i8(T(x, dev))
     wp = hipops.pack_depthwise_weights(T(wt, dev))
-    out = hipops.depthwise_conv2d_i8(xp, c, h, w, wp, k, k, T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
-    eq(nhwc_to_nchw(out, c, ref.shape[2], ref.shape[3]), ref, "depthwise int8")
-    out32 = hipops.depthwise_conv2d_i8(xp, c, h, w, wp, k, k, T(b, dev), None, False, (st, st), (pd, pd))
+    out = hipops.depthwise_conv2d_i8(xp, n, c, h, w, wp, k, k, T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
+    eq(act_to_nchw(out, n, c, ref.shape[2], ref.shape[3]), ref, "depthwise int8")
+    out32 = hipops.depthwise_conv2d_i8(xp, n, c, h, w, wp, k, k, T(b, dev), None, False, (st, st), (pd, pd))
     torch.cuda.synchronize()
     eq(out32.cpu().numpy(), oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), c), "depthwise int32")
 
@@ -134,9 +179,9 @@ def test_add_i8(c, dev):
     b = synth.tensor("fadd-%d" % c, "b", (2, c, 5, 7), -127, 127)
     stages = [("relu",), ("cvm_right_shift", 8, 1)]
     ref = run_chain(oracle.elemwise("elemwise_add", a, b), stages)
-    ap, bp = hipops.pack_nhwc_i8(T(a, dev)), hipops.pack_nhwc_i8(T(b, dev))
-    eq(nhwc_to_nchw(hipops.add_i8(ap, bp, c, 5, 7, hipops.chain(*stages), True), c, 5, 7), ref, "add int8")
-    out = hipops.add_i8(ap, bp, c, 5, 7, None, False)
+    ap, bp = hipops.pack_act_i8(T(a, dev)), hipops.pack_act_i8(T(b, dev))
+    eq(act_to_nchw(hipops.add_i8(ap, bp, 2, c, 5, 7, hipops.chain(*stages), True), 2, c, 5, 7), ref, "add int8")
+    out = hipops.add_i8(ap, bp, 2, c, 5, 7, None, False)
     torch.cuda.synchronize()
     eq(out.cpu().numpy(), oracle.elemwise("elemwise_add", a, b), "add int32")
 
@@ -148,33 +193,33 @@ def test_max_pool2d_i8(case, dev):
     x = synth.tensor("fpool-%s" % (case,), "x", (n, c, h, w), -128, 127)
     ref = oracle.max_pool2d(x, (k, k), (st, st), (pd, pd), ceil)
     oh, ow = ref.shape[2:]
-    out = hipops.max_pool2d_i8(hipops.pack_nhwc_i8(T(x, dev)), c, h, w, (k, k), (st, st), (pd, pd), oh, ow)
-    eq(nhwc_to_nchw(out, c, oh, ow), ref, "max_pool int8")
+    out = hipops.max_pool2d_i8(hipops.pack_act_i8(T(x, dev)), n, c, h, w, (k, k), (st, st), (pd, pd), oh, ow)
+    eq(act_to_nchw(out, n, c, oh, ow), ref, "max_pool int8")
 
 
 @pytest.mark.parametrize("c", [10, 64, 2048])
 def test_sum_hw_i8(c, dev):
     x = synth.tensor("fsum-%d" % c, "x", (3, c, 7, 7), -127, 127)
     ref = oracle.reduce("sum", x, (2, 3), False, False)
-    xp = hipops.pack_nhwc_i8(T(x, dev))
-    out = hipops.sum_hw_i8(xp, c, 49, None, False)
+    xp = hipops.pack_act_i8(T(x, dev))
+    out = hipops.sum_hw_i8(xp, 3, c, 49, None, False)
     torch.cuda.synchronize()
     eq(out.cpu().numpy(), ref, "sum int32")
     stages = [("cvm_right_shift", 8, 6)]
-    out8 = hipops.sum_hw_i8(xp, c, 49, hipops.chain(*stages), True)
-    eq(nhwc_to_nchw(out8, c, 1, 1)[:, :, 0, 0], run_chain(ref, stages), "sum int8")
+    out8 = hipops.sum_hw_i8(xp, 3, c, 49, hipops.chain(*stages), True)
+    eq(act_to_nchw(out8, 3, c, 1, 1)[:, :, 0, 0], run_chain(ref, stages), "sum int8")
 
 
 def test_bad_arguments_are_refused(dev):
-    x = hipops.pack_nhwc_i8(T(np.zeros((1, 16, 4, 4), np.int32), dev))
+    x = hipops.pack_act_i8(T(np.zeros((1, 16, 4, 4), np.int32), dev))
     w = hipops.pack_weights(T(np.zeros((16, 16, 3, 3), np.int32), dev))
     from cvm_runtime_amd import CvmHipError
     with pytest.raises(CvmHipError):
-        hipops.conv2d_i8(x, 16, 4, 4, w, 16, 3, 3, dilation=(2, 2))      # dilated 3x3 window exceeds the 4x4 input
+        hipops.conv2d_i8(x, 1, 16, 4, 4, w, 16, 3, 3, dilation=(2, 2))      # dilated 3x3 window exceeds the 4x4 input
     bad = hipops.Chain()
     bad.count = 5
     with pytest.raises(CvmHipError):
-        hipops.conv2d_i8(x, 16, 4, 4, w, 16, 3, 3, chain1=bad, padding=(1, 1))
+        hipops.conv2d_i8(x, 1, 16, 4, 4, w, 16, 3, 3, chain1=bad, padding=(1, 1))
 
 
 @pytest.mark.parametrize("name", ["resnet20", "resnet50", "vgg16", "ssd"])
