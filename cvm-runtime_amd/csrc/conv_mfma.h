@@ -9,6 +9,30 @@ namespace cvmhip {
 
 enum { OUT_I32_NCHW = 0, OUT_I8_ACT = 1 };
 
+// Division of n < 2^31 by a fixed divisor in three instructions (multiply-high,
+// add, shift): q = (mulhi(n, m) + n) >> l with l = ceil(log2 d),
+// m = floor(2^32 * (2^l - d) / d) + 1.  The kernels decode pixel indices with it;
+// a wavefront that runs alone on its SIMD pays full latency for every
+// instruction, so the ~40-instruction generic division matters.
+struct FastDiv {
+  uint32_t m;
+  int32_t l;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.l = 0;
+  while ((1u << f.l) < d) ++f.l;
+  f.m = (uint32_t)((((uint64_t)1 << 32) * (((uint64_t)1 << f.l) - d)) / d + 1);
+  return f;
+}
+__host__ __device__ inline uint32_t fastdiv(uint32_t n, FastDiv f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (__umulhi(n, f.m) + n) >> f.l;
+#else
+  return (uint32_t)((((uint64_t)n * f.m) >> 32) + n) >> f.l;
+#endif
+}
+
 struct ConvGeom {
   int N, H, W, Cp;         // input: int8 activations in the layout above, channels padded to Cp
   int C;                   // true channel count (0 = unknown, only used to count algorithmic work)
@@ -17,6 +41,7 @@ struct ConvGeom {
   int taps, K, Kp;         // filled by conv_igemm: KH*KW, taps*Cp, K rounded up to 64
   int64_t P;               // filled by conv_igemm: N*OH*OW
   int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
+  FastDiv div_ohw, div_ow, div_ct, div_kw;  // filled by conv_igemm: division by OH*OW, OW, Cp/32 and KW
 };
 
 // What happens to an accumulator before it is stored:

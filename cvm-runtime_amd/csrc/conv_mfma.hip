@@ -215,9 +215,9 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     const int64_t p = px0 + ((wave + 4 * i) / CH32) * 32 + lrow;
     row_ok[i] = p < g.P;
     const int pp = row_ok[i] ? (int)p : 0;
-    const int n = pp / OHW;
+    const int n = (int)fastdiv((unsigned)pp, g.div_ohw);
     const int rem = pp - n * OHW;
-    const int oh = rem / g.OW, ow = rem - oh * g.OW;
+    const int oh = (int)fastdiv((unsigned)rem, g.div_ow), ow = rem - oh * g.OW;
     img_pix[i] = n * g.H * g.W;
     ih0[i] = oh * g.SH - g.PH;
     iw0[i] = ow * g.SW - g.PW;
@@ -363,7 +363,7 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     for (int j = 0; j < WN; ++j) {
       const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
       if (p >= g.P) continue;
-      const int n = (int)p / OHW;
+      const int n = (int)fastdiv((unsigned)p, g.div_ohw);
       const int rem = (int)p - n * OHW;
       int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
 #pragma unroll
@@ -395,18 +395,26 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 }
 
 // ---------------------------------------------------------------- wavefront-private kernel
-// Layers whose grid is small (few pixels, deep K) are bound by the latency of
-// the global -> LDS -> barrier chain of the tiled kernel above, not by MFMA
-// rate.  This kernel has no LDS and no barrier in its K loop: every wavefront
-// streams its own operands straight from memory into MFMA registers (filter and
-// pixel-blocked activations are both stored in fragment order, so a load is
-// 16 bytes per lane and, for a 1x1 convolution, 1 KiB contiguous per wavefront)
-// and keeps two batches of D chunks (32 bytes of K each) in flight.  The NW
-// wavefronts of a workgroup split the K range KSPLIT ways and the pixel axis
-// NW/KSPLIT ways; partial sums meet in LDS once, after the loop.
-// Requires Cp % 32 == 0 (pixel-blocked input; a chunk never straddles two filter
-// taps) and, when the convolution pads, at most 32 taps (per-lane validity mask).
-template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, bool NOPAD>
+// Layers whose grid is small (few pixels, deep K) are bound by latency, not by
+// MFMA rate: with one wavefront per SIMD every instruction pays its full
+// pipeline latency and every K step of the tiled kernel pays a global -> LDS ->
+// barrier round trip.  This kernel has no LDS and no barrier in its K loop:
+// every wavefront streams its own operands straight from memory into MFMA
+// registers (filter and pixel-blocked activations are both stored in fragment
+// order, so a load is 16 bytes per lane and, for a 1x1 convolution, 1 KiB
+// contiguous per wavefront) and keeps two batches of D chunks (32 bytes of K
+// each) in flight.  The NW wavefronts of a workgroup split the K range KSPLIT
+// ways and the pixel axis NW/KSPLIT ways; partial sums meet in LDS once, after
+// the loop.  Requires Cp % 32 == 0 (pixel-blocked input; a chunk never
+// straddles two filter taps).
+//   MODE WAVE_IDENT  1x1, stride 1, no padding: the operand of output pixel block
+//                    t is input block t, addresses are base + chunk * 1 KiB
+//        WAVE_NOPAD  no padding: every tap of a valid output pixel is inside the image
+//        WAVE_PAD    padding: per-lane row / column validity masks (KH, KW <= 32),
+//                    out-of-image granules are read from a zero granule
+enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2 };
+
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE>
 __global__ void __launch_bounds__(NW * 64, MINW)
 k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
             const ConvGeom g, const Epilogue ep) {
@@ -431,35 +439,45 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
   const int oc_tiles = (g.OC + BM - 1) / BM;
-  const int oc0 = (pid % oc_tiles) * BM;
-  const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
+  const int ptile = pid / oc_tiles;
+  const int oc0 = (pid - ptile * oc_tiles) * BM;
+  const int px0 = ptile * BN;              // P < 2^31 is checked on the host
   const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
+  const int P = (int)g.P;
 
-  // per-lane pixel: linear index of the first input pixel of its receptive field,
-  // and which taps fall inside the image
-  int base_p[TN];
-  unsigned vmask[TN];
+  // ---- per-lane operand addressing
+  const int8_t* xb[TN];                    // WAVE_IDENT: block base + lane * 16
+  int rowbase[TN];                         // otherwise: linear index of the first input pixel of the receptive field
+  unsigned rowmask[TN], colmask[TN];       // WAVE_PAD: filter rows / columns inside the image
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int64_t p = px0 + (pw_ * TN + j) * 32 + lrow;
-    const bool ok = p < g.P;
-    const int pp = ok ? (int)p : 0;
-    const int n = pp / OHW;
-    const int rem = pp - n * OHW;
-    const int oh = rem / g.OW, ow = rem - oh * g.OW;
-    const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
-    base_p[j] = (n * g.H + ih0) * g.W + iw0;
-    unsigned m = 0;
-    if (!NOPAD) {
-      int rr = 0, ss = 0;
-      for (int t = 0; t < g.taps; ++t) {
-        const int ih = ih0 + rr * g.DH, iw = iw0 + ss * g.DW;
-        m |= (ok && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W ? 1u : 0u) << t;
-        if (++ss == g.KW) { ss = 0; ++rr; }
+    if (MODE == WAVE_IDENT) {
+      int t = (px0 >> 5) + pw_ * TN + j;
+      const int last = (P - 1) >> 5;
+      t = t < last ? t : last;             // blocks past the tensor re-read its last block; their pixels are never stored
+      xb[j] = xp + (int64_t)t * ctiles * 1024 + lane * 16;
+      rowbase[j] = 0; rowmask[j] = 0; colmask[j] = 0;
+    } else {
+      const int p = px0 + (pw_ * TN + j) * 32 + lrow;
+      const bool ok = p < P;
+      const unsigned pp = ok ? (unsigned)p : 0u;
+      const int n = (int)fastdiv(pp, g.div_ohw);
+      const int rem = (int)pp - n * OHW;
+      const int oh = (int)fastdiv((unsigned)rem, g.div_ow);
+      const int ow = rem - oh * g.OW;
+      const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
+      rowbase[j] = (n * g.H + ih0) * g.W + iw0;
+      xb[j] = xp;
+      unsigned rm = 0, cm = 0;
+      if (MODE == WAVE_PAD) {
+        for (int t = 0; t < g.KH; ++t) rm |= ((unsigned)(ih0 + t * g.DH) < (unsigned)g.H ? 1u : 0u) << t;
+        for (int t = 0; t < g.KW; ++t) cm |= ((unsigned)(iw0 + t * g.DW) < (unsigned)g.W ? 1u : 0u) << t;
+        rm = ok ? rm : 0u;
       }
+      rowmask[j] = rm;
+      colmask[j] = cm;
     }
-    vmask[j] = m;
   }
 
   // K range of this wavefront, in chunks of 32 bytes; chunks past the true K are never visited
@@ -470,14 +488,19 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int c_end = c_begin + per < nlive ? c_begin + per : nlive;
   const int niter = (per + D - 1) / D;
   int cur = c_begin;
-  int tap = (cur * 32) / g.Cp;
-  int ch = cur * 32 - tap * g.Cp;
-  int r = tap / g.KW, s = tap - r * g.KW;
+  int tap = 0, ch = 0, r = 0, s = 0;
+  if (MODE != WAVE_IDENT) {
+    tap = (int)fastdiv((unsigned)cur, g.div_ct);
+    ch = (cur - tap * ctiles) * 32;
+    r = (int)fastdiv((unsigned)tap, g.div_kw);
+    s = tap - r * g.KW;
+  }
 
   const int8_t* wa[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + i) * (nch + 1)) * 1024 + lane * 16;
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
+  const int lconst = lgrp * 512;
 
   // bias of the groups this wavefront finalises, fetched before the K loop
   int gi[NU], gj[NU], gq[NU];
@@ -488,50 +511,78 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
     gi[m] = u / (TN * 4);
     gj[m] = (u >> 2) % TN;
     gq[m] = u & 3;
-    bias_v[m] = bias4(ep, g.OC, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
+    bias_v[m] = KSPLIT == 1 ? zero4() : bias4(ep, g.OC, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
   }
 
+  // without a K split the accumulators themselves start at the bias
   v16i acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i) {
+    v16i b;
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int q = 0; q < 4; ++q) {
+      const int4 bv = KSPLIT == 1 ? bias4(ep, g.OC, oc0 + i * 32 + q * 8 + lgrp * 4) : zero4();
+      b[q * 4] = bv.x; b[q * 4 + 1] = bv.y; b[q * 4 + 2] = bv.z; b[q * 4 + 3] = bv.w;
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    for (int j = 0; j < TN; ++j) acc[i][j] = b;
+  }
 
   // one batch = D chunks of both operands, one SSA value (see k_conv_igemm)
   typedef int regs_t __attribute__((ext_vector_type(4 * (TM + TN) * D)));
+  auto put = [](regs_t& R, int b, const int4 v) __attribute__((always_inline)) {
+    R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
+  };
   auto fetch = [&]() __attribute__((always_inline)) -> regs_t {
     regs_t R;
+    if (MODE == WAVE_IDENT && cur + D <= c_end) {
+      // whole batch inside the range: one pointer per operand block, chunks at constant offsets
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int8_t* pa = wa[i] + (int64_t)cur * 1024;
+#pragma unroll
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(pa + d * 1024));
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int8_t* pb = xb[j] + (int64_t)cur * 1024;
+#pragma unroll
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(pb + d * 1024));
+      }
+      cur += D;
+      return R;
+    }
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const bool live = cur < c_end;
       // a chunk past the end multiplies the all-zero filter chunk with a valid activation address
       const int chunk = live ? cur : nch;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int4 v = *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024);
-        const int b = (d * (TM + TN) + i) * 4;
-        R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
-      }
-      const int soff = live ? (r * g.DH) * g.W + s * g.DW : 0;  // in pixels
-      const int coff = live ? (ch >> 5) * 1024 : 0;
+      for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024));
+      if (MODE == WAVE_IDENT) {
+        const int cb = live ? cur : c_begin < nlive ? c_begin : 0;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int pin = base_p[j] + soff;
-        const int8_t* src = xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + coff + lgrp * 512 + (pin & 31) * 16);
-        if (!NOPAD) src = (live && ((vmask[j] >> tap) & 1u)) ? src : zero;
-        const int4 v = *reinterpret_cast<const int4*>(src);
-        const int b = (d * (TM + TN) + TM + j) * 4;
-        R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
+        for (int j = 0; j < TN; ++j) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb * 1024));
+      } else {
+        const int soff = live ? (r * g.DH) * g.W + s * g.DW : 0;  // in pixels
+        const int coff = (live ? (ch >> 5) * 1024 : 0) + lconst;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int pin = rowbase[j] + soff;
+          const int8_t* src = xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + ((pin & 31) << 4) + coff);
+          if (MODE == WAVE_PAD) src = (live && (((rowmask[j] >> r) & (colmask[j] >> s)) & 1u)) ? src : zero;
+          put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(src));
+        }
       }
       if (live) {
         ++cur;
-        ch += 32;
-        if (ch >= g.Cp) {
-          ch = 0;
-          ++tap;
-          if (++s == g.KW) { s = 0; ++r; }
+        if (MODE != WAVE_IDENT) {
+          ch += 32;
+          if (ch >= g.Cp) {
+            ch = 0;
+            ++tap;
+            if (++s == g.KW) { s = 0; ++r; }
+          }
         }
       }
     }
@@ -618,10 +669,10 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   if (OUT == OUT_I32_NCHW) {
 #pragma unroll
     for (int m = 0; m < NU; ++m) {
-      const int64_t p = px0 + (pw_ * TN + gj[m]) * 32 + lrow;
-      if (p >= g.P) continue;
-      const int n = (int)p / OHW;
-      const int rem = (int)p - n * OHW;
+      const int p = px0 + (pw_ * TN + gj[m]) * 32 + lrow;
+      if (p >= P) continue;
+      const int n = (int)fastdiv((unsigned)p, g.div_ohw);
+      const int rem = p - n * OHW;
       const int oc = oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4;
       int32_t* y32 = reinterpret_cast<int32_t*>(out) + ((int64_t)n * g.OC + oc) * OHW + rem;
 #pragma unroll
@@ -840,22 +891,27 @@ static void launch_out(int wm, int wn, int gran, bool wide, unsigned grid, hipSt
 }
 
 // ---- wavefront-private kernel: configurations and choice
-struct WaveCfg { int tm, tn, ksplit, nw; };
+struct WaveCfg { int tm, tn, ksplit, nw, blocks_per_cu; };
 static const WaveCfg kWaveCfgs[] = {
-    {2, 2, 1, 4}, {2, 2, 2, 4}, {2, 2, 4, 4}, {2, 2, 8, 8}, {1, 2, 4, 4}, {1, 2, 8, 8}, {1, 2, 1, 4},
+    // tile rows x cols of 32, K split, wavefronts, resident workgroups per CU (registers and LDS)
+    {2, 2, 8, 8, 1}, {2, 2, 4, 4, 2}, {2, 2, 2, 4, 2}, {2, 2, 1, 4, 2},
+    {1, 2, 8, 8, 2}, {1, 2, 4, 4, 2}, {1, 2, 1, 4, 2},
 };
 constexpr int kNumWaveCfgs = sizeof(kWaveCfgs) / sizeof(kWaveCfgs[0]);
 
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT>
+static void launch_wave_mode(int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+                             const ConvGeom& g, const Epilogue& ep) {
+  if (mode == WAVE_IDENT) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_IDENT><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+  else if (mode == WAVE_NOPAD) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_NOPAD><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+  else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_PAD><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+}
+
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW>
-static void launch_wave_cfg(bool i8, bool nopad, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+static void launch_wave_cfg(int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                             const ConvGeom& g, const Epilogue& ep) {
-  if (i8) {
-    if (nopad) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I8_ACT, true><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
-    else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I8_ACT, false><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
-  } else {
-    if (nopad) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I32_NCHW, true><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
-    else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT_I32_NCHW, false><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
-  }
+  if (ep.out_mode == OUT_I8_ACT) launch_wave_mode<TM, TN, KSPLIT, NW, D, MINW, OUT_I8_ACT>(mode, grid, s, xp, wp, out, g, ep);
+  else launch_wave_mode<TM, TN, KSPLIT, NW, D, MINW, OUT_I32_NCHW>(mode, grid, s, xp, wp, out, g, ep);
 }
 
 static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
@@ -863,34 +919,34 @@ static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
   return (int64_t)((g.OC + bm - 1) / bm) * ((g.P + bn - 1) / bn);
 }
 
-// The smallest K split of the largest tile that puts about 1.5 wavefronts on
-// every SIMD of the chip; a wavefront must keep at least two chunks of K.
+// A wavefront that runs alone pays full latency for every instruction and every
+// load, so the aim is one round of workgroups with as little serial K per
+// wavefront as possible: the deepest K split (at least two chunks per wavefront)
+// of the largest tile whose grid is resident at once.  Returns -1 when even the
+// unsplit grid needs more than two rounds; the tiled kernel serves those.
 static int choose_wave_cfg(const ConvGeom& g) {
   const int nlive = g.K / 32;
-  int best = 0;
-  int64_t best_waves = 0;
-  for (int i = 0; i < kNumWaveCfgs; ++i) {
+  const int first = g.OC > 32 ? 0 : 4;
+  const int last = g.OC > 32 ? 4 : kNumWaveCfgs;
+  for (int i = first; i < last; ++i) {
     const WaveCfg& c = kWaveCfgs[i];
     if (c.ksplit > 1 && nlive < 2 * c.ksplit) continue;
-    const int64_t waves = wave_cfg_blocks(c, g) * c.nw;
-    if (waves >= 1536) return i;
-    if (waves > best_waves) { best_waves = waves; best = i; }
+    const int64_t capacity = 256 * (int64_t)c.blocks_per_cu * (c.ksplit == 1 ? 2 : 1);
+    if (wave_cfg_blocks(c, g) <= capacity) return i;
   }
-  return best;
+  return -1;
 }
 
-static void launch_wave(int cfg, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                         const ConvGeom& g, const Epilogue& ep) {
-  const bool i8 = ep.out_mode == OUT_I8_ACT;
-  const bool nopad = g.PH == 0 && g.PW == 0;
   switch (cfg) {
-    case 0: launch_wave_cfg<2, 2, 1, 4, 2, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    case 1: launch_wave_cfg<2, 2, 2, 4, 4, 1>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    case 2: launch_wave_cfg<2, 2, 4, 4, 4, 1>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    case 3: launch_wave_cfg<2, 2, 8, 8, 2, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    case 4: launch_wave_cfg<1, 2, 4, 4, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    case 5: launch_wave_cfg<1, 2, 8, 8, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
-    default: launch_wave_cfg<1, 2, 1, 4, 4, 2>(i8, nopad, grid, s, xp, wp, out, g, ep); break;
+    case 0: launch_wave_cfg<2, 2, 8, 8, 2, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 1: launch_wave_cfg<2, 2, 4, 4, 2, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 2: launch_wave_cfg<2, 2, 2, 4, 2, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 3: launch_wave_cfg<2, 2, 1, 4, 2, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 4: launch_wave_cfg<1, 2, 8, 8, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 5: launch_wave_cfg<1, 2, 4, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    default: launch_wave_cfg<1, 2, 1, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
   }
 }
 
@@ -926,21 +982,28 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
     wm = forced[0] - '0';
     wn = forced[2] - '0';
   }
-  // kernel choice: "wave" (no LDS in the K loop) when the layout allows it, else the LDS-tiled kernel;
-  // test and tuning hooks: CVM_HIP_CONV=lds forces the tiled kernel, CVM_HIP_WAVECFG=<index> a configuration
+  g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
+  g.div_ow = make_fastdiv((uint32_t)g.OW);
+  g.div_ct = make_fastdiv((uint32_t)(g.Cp >= 32 ? g.Cp / 32 : 1));
+  g.div_kw = make_fastdiv((uint32_t)g.KW);
+  // kernel choice: the wavefront-private kernel when the layout allows it and its grid fits the chip,
+  // else the LDS-tiled kernel.  Test and tuning hooks (read per call): CVM_HIP_CONV=lds|wave forces
+  // one of them, CVM_HIP_WAVECFG=<index> a configuration.
   const char* conv_kind = getenv("CVM_HIP_CONV");
   const char* wave_forced = getenv("CVM_HIP_WAVECFG");
-  const bool wave_ok = (g.Cp % 32) == 0 && ((g.PH == 0 && g.PW == 0) || g.taps <= 32);
-  bool use_wave = wave_ok;
-  if (conv_kind && conv_kind[0] == 'l') use_wave = false;
-  if (conv_kind && conv_kind[0] == 'w') use_wave = wave_ok;
-  if (use_wave) {
-    int cfg = choose_wave_cfg(g);
-    if (wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
+  const bool nopad = g.PH == 0 && g.PW == 0;
+  const bool wave_ok = (g.Cp % 32) == 0 && (nopad || (g.KH <= 32 && g.KW <= 32));
+  int cfg = wave_ok ? choose_wave_cfg(g) : -1;
+  if (conv_kind && conv_kind[0] == 'l') cfg = -1;
+  if (wave_ok && conv_kind && conv_kind[0] == 'w' && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
+  if (wave_ok && cfg >= 0 && wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
+  if (cfg >= 0) {
+    const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                         ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
     KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
-    launch_wave(cfg, (unsigned)wnb, s, xp, wp, out, g, ep);
+    launch_wave(cfg, mode, (unsigned)wnb, s, xp, wp, out, g, ep);
     return check_launch("conv_wave");
   }
   const int64_t nb = blocks(64 * wm, 64 * wn);
