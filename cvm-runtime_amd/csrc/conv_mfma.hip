@@ -63,27 +63,14 @@ __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
     if ((s1 | ad | s2) == 0) {
 #pragma unroll
       for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], lo, hi);
+    } else if (s1 == 0) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = wadd(clamp3(v[e], lo, hi), ad) >> s2;
     } else {
 #pragma unroll
       for (int e = 0; e < N; ++e) v[e] = wadd(clamp3(v[e], lo, hi) >> s1, ad) >> s2;
     }
   }
-}
-
-// bias of 4 consecutive output channels starting at oc (zero past OC or without bias)
-__device__ __forceinline__ int4 bias4(const Epilogue& ep, int OC, int oc) {
-  int4 bv = zero4();
-  if (ep.bias) {
-    if (ep.bias_vec && oc + 3 < OC) {
-      bv = *reinterpret_cast<const int4*>(ep.bias + oc);
-    } else {
-      if (oc < OC) bv.x = ep.bias[oc];
-      if (oc + 1 < OC) bv.y = ep.bias[oc + 1];
-      if (oc + 2 < OC) bv.z = ep.bias[oc + 2];
-      if (oc + 3 < OC) bv.w = ep.bias[oc + 3];
-    }
-  }
-  return bv;
 }
 
 // low bytes of four values -> one dword
@@ -93,44 +80,146 @@ __device__ __forceinline__ uint32_t pack_bytes(int32_t a, int32_t b, int32_t c, 
   return __builtin_amdgcn_perm(hi2, lo2, 0x05040100u);
 }
 
-// residual of 4 consecutive channels of pixel p (clamped to valid memory)
-__device__ __forceinline__ uint32_t residual4(const Epilogue& ep, int64_t P, int64_t p, int oc) {
-  return *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ep.out_cp ? oc : 0, ep.out_cp));
+// a's lanes 32..63 <-> b's lanes 0..31
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void half_swap(uint32_t& a, uint32_t& b) {
+  const v2u r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r.x;
+  b = r.y;
 }
 
-// The int8 output tile sits in LDS as sOut[pixel][OPITCH] (channels contiguous);
-// NT threads move it to the output tensor in 16-byte granules, 32 consecutive
-// pixels per half wavefront (512 contiguous bytes of a pixel-blocked tensor).
-template <int BM, int BN, int NT>
-__device__ __forceinline__ void store_tile_i8(const int8_t* sOut, int opitch, void* out, const ConvGeom& g, const Epilogue& ep,
-                                              int oc0, int64_t px0, int tid) {
-  constexpr int CH = BM / 16;
-  int8_t* y8 = reinterpret_cast<int8_t*>(out);
+// the bias of the workgroup's BM output channels, staged in LDS by the first BM threads
+template <int BM>
+__device__ __forceinline__ void stage_bias(int* sBias, const Epilogue& ep, int OC, int oc0, int tid) {
+  if (tid < BM) sBias[tid] = (ep.bias && oc0 + tid < OC) ? ep.bias[oc0 + tid] : 0;
+}
+
+// keeps only the bytes of d[0..N-1] whose channel (first + 4k + byte) is below OC:
+// padding channels of the output tensor stay zero whatever the chain maps 0 to
+template <int N>
+__device__ __forceinline__ void mask_channels(uint32_t (&d)[N], int first, int OC) {
+  if (first + 4 * N > OC) {
 #pragma unroll
-  for (int id = tid; id < BN * CH; id += NT) {
-    const int rr = id & 31;
-    const int c16 = (id >> 5) % CH;
-    const int pl = ((id >> 5) / CH) * 32 + rr;
-    const int64_t p = px0 + pl;
-    const int oc = oc0 + c16 * 16;
-    if (p >= g.P || oc >= ep.out_cp) continue;
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(sOut + pl * opitch + c16 * 16);
-    uint32_t d[4] = {src[0], src[1], src[2], src[3]};
-    if (oc + 16 > g.OC) {
-      // padding channels of the tensor stay zero whatever the chain maps 0 to
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int keep = g.OC - (oc + 4 * k);
-        d[k] = keep >= 4 ? d[k] : (keep <= 0 ? 0u : d[k] & ((1u << (8 * keep)) - 1u));
-      }
+    for (int k = 0; k < N; ++k) {
+      const int keep = OC - (first + 4 * k);
+      d[k] = keep >= 4 ? d[k] : (keep <= 0 ? 0u : d[k] & ((1u << (8 * keep)) - 1u));
     }
-    int8_t* dst = y8 + act_offset(p, oc, ep.out_cp);
-    if (ep.out_cp >= 16) {
-      *reinterpret_cast<int4*>(dst) = make_int4(d[0], d[1], d[2], d[3]);
+  }
+}
+
+// Epilogue shared by both kernels.  A wavefront holds NG groups of 4 values; group
+// u (counted from u0, which is a multiple of NG) belongs to the 32x32 MFMA tile
+// t = u / 4 of the wavefront's TM x TN tiles (t = i * TN + j) and is the 4
+// consecutive channels q*8 + (lane/32)*4 .. +3, q = u % 4, of pixel lane % 32.
+//   v = chain(acc + bias);  if (residual) v = chain2(v + residual);  store
+// For a pixel-blocked int8 tensor two half-wave swaps turn the 4 packed dwords of a
+// tile into 16 consecutive channels per lane, so the wavefront reads the
+// residual and writes the result as one contiguous KiB per tile.
+template <int TN, int NG, int OUT>
+__device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
+                                              int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep) {
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int P = (int)g.P;
+  const int ocp = ep.out_cp;
+  const bool blocked = act_blocked(ocp);
+  // group m: tile (gi, gj), channel quarter gq; ch = first channel inside the workgroup's BM channels
+  int gj[NG], ch[NG];
+#pragma unroll
+  for (int m = 0; m < NG; ++m) {
+    const int u = u0 + m;
+    const int t = u >> 2;
+    gj[m] = t % TN;
+    ch[m] = ch_wave + (t / TN) * 32 + (u & 3) * 8 + lgrp * 4;
+    const int4 bv = *reinterpret_cast<const int4*>(sBias + ch[m]);
+    val[m * 4] = wadd(val[m * 4], bv.x); val[m * 4 + 1] = wadd(val[m * 4 + 1], bv.y);
+    val[m * 4 + 2] = wadd(val[m * 4 + 2], bv.z); val[m * 4 + 3] = wadd(val[m * 4 + 3], bv.w);
+  }
+  // byte offset of the KiB block (pixel block, 32 channels) that tile of group m belongs to
+  auto block_off = [&](int m) {
+    const int pblk = (px_wave >> 5) + gj[m];
+    const int cblk = (oc0 + (ch[m] - lgrp * 4)) >> 5;
+    return ((int64_t)pblk * (ocp >> 5) + cblk) * 1024;
+  };
+  const bool whole = blocked && (NG % 4 == 0);   // whole tiles: 16 bytes per lane
+  const bool halves = blocked && NG == 2;         // half a tile (q pair): 8 bytes per lane
+
+  if (ep.residual) {
+    uint32_t rp[NG];
+    if (whole) {
+#pragma unroll
+      for (int t = 0; t < NG / 4; ++t) {
+        // the block exists (all 32 pixel rows of it are allocated) unless it lies past the tensor
+        const bool tile_ok = (px_wave + gj[t * 4] * 32) < P && (oc0 + ch[t * 4] - lgrp * 4) < ocp;
+        const int4 r4 = tile_ok ? *reinterpret_cast<const int4*>(ep.residual + block_off(t * 4) + lane * 16) : zero4();
+        uint32_t a = r4.x, b = r4.y, c = r4.z, d = r4.w;
+        half_swap(a, b);
+        half_swap(c, d);
+        rp[t * 4] = a; rp[t * 4 + 1] = c; rp[t * 4 + 2] = b; rp[t * 4 + 3] = d;
+      }
     } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (oc + k * 4 < ep.out_cp) reinterpret_cast<uint32_t*>(dst)[k] = d[k];
+      for (int m = 0; m < NG; ++m) {
+        const int p = px_wave + gj[m] * 32 + lrow;
+        const int oc = oc0 + ch[m];
+        rp[m] = *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ocp ? oc : 0, ocp));
+      }
+    }
+    run_chain(ep.chain, val);
+#pragma unroll
+    for (int e = 0; e < NG * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
+    run_chain(ep.chain2, val);
+  } else {
+    run_chain(ep.chain, val);
+  }
+
+  if (OUT == OUT_I32_NCHW) {
+    const int OHW = g.OH * g.OW;
+#pragma unroll
+    for (int m = 0; m < NG; ++m) {
+      const int p = px_wave + gj[m] * 32 + lrow;
+      if (p >= P) continue;
+      const int n = (int)fastdiv((unsigned)p, g.div_ohw);
+      const int rem = p - n * OHW;
+      const int oc = oc0 + ch[m];
+      int32_t* y32 = reinterpret_cast<int32_t*>(out) + ((int64_t)n * g.OC + oc) * OHW + rem;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (oc + e < g.OC) y32[(int64_t)e * OHW] = val[m * 4 + e];
+    }
+    return;
+  }
+  int8_t* y8 = reinterpret_cast<int8_t*>(out);
+  uint32_t pk[NG];
+#pragma unroll
+  for (int m = 0; m < NG; ++m) pk[m] = pack_bytes(val[m * 4], val[m * 4 + 1], val[m * 4 + 2], val[m * 4 + 3]);
+  if (whole) {
+#pragma unroll
+    for (int t = 0; t < NG / 4; ++t) {
+      uint32_t a = pk[t * 4], b = pk[t * 4 + 1], c = pk[t * 4 + 2], d = pk[t * 4 + 3];
+      half_swap(a, c);   // lower half wave: channels 0..15 of the tile, upper: 16..31
+      half_swap(b, d);
+      uint32_t w[4] = {a, c, b, d};
+      const int first = oc0 + ch_wave + ((u0 >> 2) + t) / TN * 32 + lgrp * 16;
+      mask_channels(w, first, g.OC);
+      const int p = px_wave + gj[t * 4] * 32 + lrow;
+      if (p < P && first < ocp) *reinterpret_cast<int4*>(y8 + block_off(t * 4) + lane * 16) = make_int4(w[0], w[1], w[2], w[3]);
+    }
+  } else if (halves) {
+    uint32_t a = pk[0], b = pk[1];
+    half_swap(a, b);     // lower half wave: channels 0..7 of the 16-channel granule, upper: 8..15
+    uint32_t w[2] = {a, b};
+    const int first = oc0 + ch[0] - lgrp * 4 + lgrp * 8;
+    mask_channels(w, first, g.OC);
+    const int p = px_wave + gj[0] * 32 + lrow;
+    if (p < P && first < ocp) *reinterpret_cast<uint2*>(y8 + act_offset(p, first, ocp)) = make_uint2(w[0], w[1]);
+  } else {
+#pragma unroll
+    for (int m = 0; m < NG; ++m) {
+      uint32_t w[1] = {pk[m]};
+      const int first = oc0 + ch[m];
+      mask_channels(w, first, g.OC);
+      const int p = px_wave + gj[m] * 32 + lrow;
+      if (p < P && first < ocp) *reinterpret_cast<uint32_t*>(y8 + act_offset(p, first, ocp)) = w[0];
     }
   }
 }
@@ -178,8 +267,6 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   constexpr int CH32 = KS / 32;      // 32-byte chunks of K per step
   constexpr int NA = BM * KS / 4096; // 16-byte granules per thread and K step, filter
   constexpr int NB = BN * KS / 4096; //   ... activations
-  constexpr int OPITCH = BM + 4;     // pitch of the int8 output tile (odd number of dwords)
-  static_assert(BN * OPITCH <= 2 * (BM + BN) * KS, "output tile must fit the staging area");
   // two buffers of each operand in fragment order: granule index = ((tile32*CH32 + chunk)*64 + lane)
   __shared__ __attribute__((aligned(16))) int8_t smem[2 * (BM + BN) * KS];
   int8_t* sA = smem;
@@ -233,20 +320,16 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   int kbyte = 0;
 
   // Accumulator element e of lane l in a 32x32 tile is row (e/4)*8 + (l/32)*4 + e%4
-  // (output channel), column l%32 (pixel).  Accumulators start at the bias of
-  // their channel, so the epilogue has no bias pass.
+  // (output channel), column l%32 (pixel).
+  __shared__ __attribute__((aligned(16))) int sBias[BM];
+  stage_bias<BM>(sBias, ep, g.OC, oc0, tid);   // visible after the first barrier of the K loop
   v16i acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    v16i b;
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int4 bv = bias4(ep, g.OC, oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4);
-      b[q * 4] = bv.x; b[q * 4 + 1] = bv.y; b[q * 4 + 2] = bv.z; b[q * 4 + 3] = bv.w;
-    }
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
-    for (int j = 0; j < WN; ++j) acc[i][j] = b;
-  }
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   // One K step of operands held in registers as a single SSA vector value
   // (granules 0..NA-1 filter, NA..NA+NB-1 activations); two of them are in flight.
@@ -332,7 +415,7 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     __syncthreads();
   }
 
-  // ---- epilogue: v = chain(acc); if (residual) v = chain2(v + residual)
+  // ---- epilogue
   int32_t val[WM * WN * 16];
 #pragma unroll
   for (int i = 0; i < WM; ++i)
@@ -340,58 +423,7 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) val[(i * WN + j) * 16 + e] = acc[i][j][e];
-  if (ep.residual) {
-    // one dword = the residual of 4 consecutive channels; loads are issued before the first chain runs
-    uint32_t rp[WM * WN * 4];
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          rp[(i * WN + j) * 4 + q] = residual4(ep, g.P, px0 + (wn * WN + j) * 32 + lrow, oc0 + (wm * WM + i) * 32 + q * 8 + lgrp * 4);
-    run_chain(ep.chain, val);
-#pragma unroll
-    for (int e = 0; e < WM * WN * 16; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
-    run_chain(ep.chain2, val);
-  } else {
-    run_chain(ep.chain, val);
-  }
-
-  if (OUT == OUT_I32_NCHW) {
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int64_t p = px0 + (wn * WN + j) * 32 + lrow;
-      if (p >= g.P) continue;
-      const int n = (int)fastdiv((unsigned)p, g.div_ohw);
-      const int rem = (int)p - n * OHW;
-      int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * g.OC * OHW + rem;
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int oc = oc0 + (wm * WM + i) * 32 + (e >> 2) * 8 + lgrp * 4 + (e & 3);
-          if (oc < g.OC) y32[(int64_t)oc * OHW] = val[(i * WN + j) * 16 + e];
-        }
-    }
-  } else {
-    // int8: the tile goes through LDS (the staging area is free after the last
-    // barrier of the K loop) so that global stores are 16 contiguous bytes per thread
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int pl = (wn * WN + j) * 32 + lrow;
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int ol = (wm * WM + i) * 32 + q * 8 + lgrp * 4;
-          const int b = (i * WN + j) * 16 + q * 4;
-          *reinterpret_cast<uint32_t*>(&smem[pl * OPITCH + ol]) = pack_bytes(val[b], val[b + 1], val[b + 2], val[b + 3]);
-        }
-    }
-    __syncthreads();
-    store_tile_i8<BM, BN, 256>(smem, OPITCH, out, g, ep, oc0, px0, tid);
-  }
+  finish_groups<WN, WM * WN * 4, OUT>(val, 0, sBias, wm * WM * 32, oc0, (int)px0 + wn * WN * 32, lane, out, g, ep);
 }
 
 // ---------------------------------------------------------------- wavefront-private kernel
@@ -424,10 +456,9 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   constexpr int BN = WPIX * PS;           // pixels per workgroup
   constexpr int U = TM * TN * 4;          // groups of 4 accumulator registers (4 consecutive channels) per wavefront
   constexpr int NU = U / KSPLIT;          // groups one wavefront finalises
-  constexpr int OPITCH = BM + 4;
   static_assert(NW % KSPLIT == 0 && U % KSPLIT == 0, "split must divide the work");
   __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
-  __shared__ __attribute__((aligned(16))) int8_t sOut[OUT == OUT_I8_ACT ? BN * OPITCH : 16];
+  __shared__ __attribute__((aligned(16))) int sBias[BM];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -502,31 +533,15 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   const int lconst = lgrp * 512;
 
-  // bias of the groups this wavefront finalises, fetched before the K loop
-  int gi[NU], gj[NU], gq[NU];
-  int4 bias_v[NU];
-#pragma unroll
-  for (int m = 0; m < NU; ++m) {
-    const int u = KSPLIT == 1 ? m : kw_ + KSPLIT * m;
-    gi[m] = u / (TN * 4);
-    gj[m] = (u >> 2) % TN;
-    gq[m] = u & 3;
-    bias_v[m] = KSPLIT == 1 ? zero4() : bias4(ep, g.OC, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
-  }
+  stage_bias<BM>(sBias, ep, g.OC, oc0, tid);
 
-  // without a K split the accumulators themselves start at the bias
   v16i acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    v16i b;
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int4 bv = KSPLIT == 1 ? bias4(ep, g.OC, oc0 + i * 32 + q * 8 + lgrp * 4) : zero4();
-      b[q * 4] = bv.x; b[q * 4 + 1] = bv.y; b[q * 4 + 2] = bv.z; b[q * 4 + 3] = bv.w;
-    }
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = b;
-  }
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   // one batch = D chunks of both operands, one SSA value (see k_conv_igemm)
   typedef int regs_t __attribute__((ext_vector_type(4 * (TM + TN) * D)));
@@ -619,7 +634,9 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
     consume(R1);
   }
 
-  // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS
+  // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
+  // wavefront kw_ then finalises the groups kw_*NU .. kw_*NU + NU-1 of the tile set
+  int32_t val[NU * 4];
   if (KSPLIT > 1) {
     int* mine = sPart + wave * U * 256;
 #pragma unroll
@@ -631,64 +648,26 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
           *reinterpret_cast<int4*>(mine + (((i * TN + j) * 4 + q) * 64 + lane) * 4) =
               make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
     __syncthreads();
-  }
-
-  // ---- finalise: wavefront kw_ owns the groups u = kw_ + KSPLIT * m of its tile
-  int32_t val[NU * 4];
 #pragma unroll
-  for (int m = 0; m < NU; ++m) {
-    int4 sum = bias_v[m];
-    if (KSPLIT == 1) {
-      // u == m is a compile-time constant here: plain register reads
-      const v16i& a = acc[m / (TN * 4)][(m >> 2) % TN];
-      const int q = (m & 3) * 4;
-      sum.x = wadd(sum.x, a[q]); sum.y = wadd(sum.y, a[q + 1]); sum.z = wadd(sum.z, a[q + 2]); sum.w = wadd(sum.w, a[q + 3]);
-    } else {
-      const int u = kw_ + KSPLIT * m;
+    for (int m = 0; m < NU; ++m) {
+      int4 sum = zero4();
 #pragma unroll
       for (int k = 0; k < KSPLIT; ++k) {
-        const int4 v = *reinterpret_cast<const int4*>(sPart + (((pw_ * KSPLIT + k) * U + u) * 64 + lane) * 4);
+        const int4 v = *reinterpret_cast<const int4*>(sPart + (((pw_ * KSPLIT + k) * U + kw_ * NU + m) * 64 + lane) * 4);
         sum.x = wadd(sum.x, v.x); sum.y = wadd(sum.y, v.y); sum.z = wadd(sum.z, v.z); sum.w = wadd(sum.w, v.w);
       }
-    }
-    val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
-  }
-  if (ep.residual) {
-    uint32_t rp[NU];
-#pragma unroll
-    for (int m = 0; m < NU; ++m)
-      rp[m] = residual4(ep, g.P, px0 + (pw_ * TN + gj[m]) * 32 + lrow, oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4);
-    run_chain(ep.chain, val);
-#pragma unroll
-    for (int e = 0; e < NU * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
-    run_chain(ep.chain2, val);
-  } else {
-    run_chain(ep.chain, val);
-  }
-
-  if (OUT == OUT_I32_NCHW) {
-#pragma unroll
-    for (int m = 0; m < NU; ++m) {
-      const int p = px0 + (pw_ * TN + gj[m]) * 32 + lrow;
-      if (p >= P) continue;
-      const int n = (int)fastdiv((unsigned)p, g.div_ohw);
-      const int rem = p - n * OHW;
-      const int oc = oc0 + gi[m] * 32 + gq[m] * 8 + lgrp * 4;
-      int32_t* y32 = reinterpret_cast<int32_t*>(out) + ((int64_t)n * g.OC + oc) * OHW + rem;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (oc + e < g.OC) y32[(int64_t)e * OHW] = val[m * 4 + e];
+      val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
     }
   } else {
+    __syncthreads();   // bias staged
 #pragma unroll
-    for (int m = 0; m < NU; ++m) {
-      const int pl = (pw_ * TN + gj[m]) * 32 + lrow;
-      const int ol = gi[m] * 32 + gq[m] * 8 + lgrp * 4;
-      *reinterpret_cast<uint32_t*>(&sOut[pl * OPITCH + ol]) = pack_bytes(val[m * 4], val[m * 4 + 1], val[m * 4 + 2], val[m * 4 + 3]);
-    }
-    __syncthreads();
-    store_tile_i8<BM, BN, NW * 64>(sOut, OPITCH, out, g, ep, oc0, px0, tid);
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) val[((i * TN + j) * 16 + e) % (NU * 4)] = acc[i][j][e];
   }
+  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, out, g, ep);
 }
 
 constexpr int KSTEP = 64;  // granularity K is padded to

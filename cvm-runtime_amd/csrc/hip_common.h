@@ -114,7 +114,7 @@ __device__ __forceinline__ int32_t apply_rshift(const RShift& r, int32_t t) {
 //     v = (clamp(v, lo, hi) >> s1) + add) >> s2          (add wraps)
 //   relu            : clamp to [0, INT32_MAX]
 //   clip / cvm_clip : clamp to [lo, hi]
-//   cvm_right_shift : regime "saturate"  clamp to the pre-shifted bounds, s1 = b-1, add = 1, s2 = 1
+//   cvm_right_shift : regime "saturate"  clamp to the pre-shifted bounds, s1 = 0, add = 2^(b-1), s2 = b
 //                     (the rounding shift is monotonic and maps the bounds to -max / max, so
 //                      clamping first equals the reference's compare-then-shift)
 //                     regime "p + b >= 32"  no clamp, s1 = b-1, add = 1, s2 = 1
@@ -168,7 +168,11 @@ inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
       else if (r.mode == 1) { d.s1 = 31; }
       else {
         d.s1 = r.sh; d.add = 1; d.s2 = 1;
-        if (r.mode == 3) { d.lo = r.x_min; d.hi = r.x_max; }
+        if (r.mode == 3) {
+          // after the clamp v + 2^(b-1) cannot overflow, and ((v >> (b-1)) + 1) >> 1 == (v + 2^(b-1)) >> b
+          d.lo = r.x_min; d.hi = r.x_max;
+          d.s1 = 0; d.add = (int32_t)1 << r.sh; d.s2 = r.sh + 1;
+        }
       }
     } else {
       return false;
