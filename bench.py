@@ -126,11 +126,24 @@ def main():
     api_s = (time.perf_counter() - t0) / n_api
     model.close()
 
-    conv = kt.get("k_conv_igemm", {"launches": 0, "ms": 0.0, "work": 0.0})
+    # The two implicit-GEMM kernels (same arithmetic, chosen per layer); the roofline object is about the
+    # one that takes more of the step.  An event pair makes a launch look longer than it is.  Every launch
+    # of a step is timed and the un-instrumented step is GPU-bound with its kernels back to back, so the
+    # cost of one pair is (sum of all pair times - un-instrumented step time) / launches; it is taken off
+    # every launch.  The rocprofv3 kernel trace under profiles/ measures the same durations directly.
+    n_timed = sum(v["launches"] for v in kt.values())
+    pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall * 1e6) / max(n_timed, 1))
+    pair_us = {"empty_us": pair_cost_us}
+    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm")}
+    dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
+    conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
     launches = max(conv["launches"], 1)
     ops_per_launch = conv["work"] / launches
-    avg_s = conv["ms"] / 1e3 / launches
-    achieved = ops_per_launch / avg_s / 1e12 if avg_s > 0 else 0.0
+    raw_avg_s = conv["ms"] / 1e3 / launches
+    avg_s = max(raw_avg_s - pair_us["empty_us"] * 1e-6, 1e-9)
+    achieved = ops_per_launch / avg_s / 1e12
+    all_ops = sum(v["work"] for v in convs.values())
+    all_s = sum(v["ms"] / 1e3 - v["launches"] * pair_us["empty_us"] * 1e-6 for v in convs.values())
     step_s = wall / args.steps
     line = {
         "metric": "images/sec int8 ResNet-50 (224x224), one MI355X, input resident in HBM",
@@ -153,10 +166,14 @@ def main():
                    "output_checksum": int(np.bitwise_xor.reduce(out.view(np.uint32)))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_I8_TOPS, "unit": "TOP/s",
                      "frac": achieved / PEAK_I8_TOPS, "traffic": None,
-                     "kernel": "k_conv_igemm", "launches_per_step": conv["launches"] / args.steps,
-                     "avg_launch_us": avg_s * 1e6, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
-                     "kernel_ms_per_step": conv["ms"] / args.steps,
-                     "other_kernels_ms_per_step": {k: v["ms"] / args.steps for k, v in kt.items() if k != "k_conv_igemm"}},
+                     "kernel": dom, "launches_per_step": conv["launches"] / args.steps,
+                     "avg_launch_us": avg_s * 1e6, "avg_launch_us_with_event_pair": raw_avg_s * 1e6,
+                     "event_pair_cost_us": pair_cost_us, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
+                     "kernel_ms_per_step": avg_s * 1e3 * conv["launches"] / args.steps,
+                     "all_conv_dense_launches": {"achieved_tops": all_ops / max(all_s, 1e-9) / 1e12,
+                                                 "launches_per_step": sum(v["launches"] for v in convs.values()) / args.steps,
+                                                 "ms_per_step": all_s * 1e3 / args.steps},
+                     "other_kernels_ms_per_step": {k: v["ms"] / args.steps for k, v in kt.items() if k != dom}},
     }
     if not args.no_cpu_baseline:
         g1, h1 = graphgen.resnet50(1)

@@ -981,7 +981,7 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
                          ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
-    KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+    KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
     launch_wave(cfg, mode, (unsigned)wnb, s, xp, wp, out, g, ep);
     return check_launch("conv_wave");
   }

@@ -283,6 +283,7 @@ int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int o
   const int cp = pad_channels(c);
   const int64_t total = act_bytes(n, cp) / 4;
   hipStream_t s = as_stream(stream);
+  KernelTimer timer("k_sum_hw_i8", (double)n * c * hw + (double)n * c, s);  // bytes in + out
   k_sum_hw_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
                                                    hw, ch);
   return check_launch("sum_hw_i8");
