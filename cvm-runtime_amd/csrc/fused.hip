@@ -74,22 +74,71 @@ k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t 
   }
 }
 
+// max_pool2d for Cp >= 16: one thread per 16 channels of one output pixel (16-byte loads and stores)
+__global__ void __launch_bounds__(256)
+k_max_pool_i8x16(const int8_t* __restrict__ x, int8_t* __restrict__ y, int64_t total, int64_t npix_out, int cp, int h,
+                 int w, int oh, int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    int64_t t;
+    int c0;
+    act_decode(i * 4, cp, &t, &c0);
+    if (t >= npix_out) continue;
+    const int q = (int)(t % ow);
+    t /= ow;
+    const int p = (int)(t % oh);
+    const int64_t n = t / oh;
+    int32_t m[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) m[e] = -128;
+    for (int r = 0; r < kh; ++r) {
+      const int ih = p * sh + r - ph;
+      if (ih < 0 || ih >= h) continue;
+      for (int s = 0; s < kw; ++s) {
+        const int iw = q * sw + s - pw;
+        if (iw < 0 || iw >= w) continue;
+        const int4 v = *reinterpret_cast<const int4*>(x + act_offset((n * h + ih) * w + iw, c0, cp));
+        const uint32_t d[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int32_t b = byte_of(d[e >> 2], e & 3);
+          m[e] = b > m[e] ? b : m[e];
+        }
+      }
+    }
+    *reinterpret_cast<int4*>(y + i * 16) = make_int4(pack4(m[0], m[1], m[2], m[3]), pack4(m[4], m[5], m[6], m[7]),
+                                                     pack4(m[8], m[9], m[10], m[11]), pack4(m[12], m[13], m[14], m[15]));
+  }
+}
+
 // out[n][c] = chain(sum_hw x[n][hw][c]); the result is a tensor of n "pixels"
+// Eight consecutive lanes share one output dword (4 channels of one image): each
+// sums every eighth pixel, a butterfly over the 8 lanes adds the parts.
 __global__ void __launch_bounds__(256)
 k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i8, int64_t total, int nimg, int c, int cp,
             int hw, DevChain chain) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+  const int64_t stride = ((int64_t)gridDim.x * blockDim.x) >> 3;
+  const int part = threadIdx.x & 7;
+  // all 8 lanes of a group run the same number of iterations (total is rounded up by the launch)
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 3; i < total; i += stride) {
     int64_t n;
     int c0;
     act_decode(i, cp, &n, &c0);
-    if (n >= nimg) continue;
     int32_t acc[4] = {0, 0, 0, 0};
-    for (int t = 0; t < hw; ++t) {
-      const uint32_t v = x[act_offset(n * hw + t, c0, cp) >> 2];
+    if (n < nimg) {
+      for (int t = part; t < hw; t += 8) {
+        const uint32_t v = x[act_offset(n * hw + t, c0, cp) >> 2];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e);
+        for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e);
+      }
     }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[e] += __shfl_xor(acc[e], 1, 64);
+      acc[e] += __shfl_xor(acc[e], 2, 64);
+      acc[e] += __shfl_xor(acc[e], 4, 64);
+    }
+    if (part != 0 || n >= nimg) continue;
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc[e] = apply_chain(chain, acc[e]);
     if (out_is_i8) {
@@ -268,9 +317,16 @@ int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, i
   const int64_t total = act_bytes(npix, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_max_pool_i8", (double)n * c * ((double)h * w + (double)oh * ow), s);
-  k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
-                                                            reinterpret_cast<uint32_t*>(yp), total, npix, cp, h, w, oh, ow,
-                                                            kh, kw, stride_h, stride_w, pad_h, pad_w);
+  if (cp >= 16) {
+    if (((uintptr_t)xp | (uintptr_t)yp) & 15) return arg_error("max_pool2d_i8 alignment");
+    k_max_pool_i8x16<<<grid_for(total / 4, 256, 1 << 16), 256, 0, s>>>(
+        reinterpret_cast<const int8_t*>(xp), reinterpret_cast<int8_t*>(yp), total / 4, npix, cp, h, w, oh, ow, kh, kw,
+        stride_h, stride_w, pad_h, pad_w);
+  } else {
+    k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
+                                                              reinterpret_cast<uint32_t*>(yp), total, npix, cp, h, w, oh, ow,
+                                                              kh, kw, stride_h, stride_w, pad_h, pad_w);
+  }
   return check_launch("max_pool2d_i8");
 }
 
@@ -284,7 +340,7 @@ int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int o
   const int64_t total = act_bytes(n, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_sum_hw_i8", (double)n * c * hw + (double)n * c, s);  // bytes in + out
-  k_sum_hw_i8<<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
+  k_sum_hw_i8<<<grid_for(total * 8, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
                                                    hw, ch);
   return check_launch("sum_hw_i8");
 }
