@@ -179,4 +179,51 @@ int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms) {
   return CVMHIP_OK;
 }
 
+int cvmhip_kernel_timing_active(void) { return g_timing ? 1 : 0; }
+
+int cvmhip_capture_begin(void* stream) {
+  HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+  return CVMHIP_OK;
+}
+
+int cvmhip_capture_end(void* stream, void** graph_exec) {
+  if (!graph_exec) return arg_error("capture_end");
+  hipGraph_t graph = nullptr;
+  HIP_TRY(hipStreamEndCapture(as_stream(stream), &graph), "hipStreamEndCapture");
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    set_error("hipGraphInstantiate: %s", hipGetErrorString(e));
+    return CVMHIP_ERR_RUNTIME;
+  }
+  *graph_exec = exec;
+  return CVMHIP_OK;
+}
+
+// An event recorded on `from` and waited for on `to`: inside a capture this is
+// how a second stream joins the graph (and how it is joined back).
+int cvmhip_stream_fork(void* from, void* to) {
+  hipEvent_t ev;
+  HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate");
+  hipError_t e = hipEventRecord(ev, as_stream(from));
+  if (e == hipSuccess) e = hipStreamWaitEvent(as_stream(to), ev, 0);
+  hipEventDestroy(ev);   // released once the work that references it has been captured or completed
+  if (e != hipSuccess) {
+    set_error("stream fork: %s", hipGetErrorString(e));
+    return CVMHIP_ERR_RUNTIME;
+  }
+  return CVMHIP_OK;
+}
+
+int cvmhip_graph_launch(void* graph_exec, void* stream) {
+  HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream)), "hipGraphLaunch");
+  return CVMHIP_OK;
+}
+
+int cvmhip_graph_destroy(void* graph_exec) {
+  if (graph_exec) HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy");
+  return CVMHIP_OK;
+}
+
 }  // extern "C"

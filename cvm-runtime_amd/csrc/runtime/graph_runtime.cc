@@ -441,6 +441,7 @@ HipGraphRuntime::HipGraphRuntime(const std::string& graph_json, int device_id, b
 }
 
 void HipGraphRuntime::Release() {
+  if (graph_exec_) { cvmhip_graph_destroy(graph_exec_); graph_exec_ = nullptr; }
   plan_.clear();
   execs_.clear();  // releases per-node device state before the stream goes away
   if (i8_slab_) { cvmhip_free(i8_slab_); i8_slab_ = nullptr; }
@@ -604,12 +605,59 @@ void HipGraphRuntime::LoadParams(const std::string& blob) {
 }
 
 // ---------------------------------------------------------------- execution
-void HipGraphRuntime::Run() {
+void HipGraphRuntime::Launch() {
   if (fused_) {
     for (PlanStep& st : plan_) RunStep(st);
   } else {
     for (Exec& ex : execs_) ex.kernel->run(ex.call);
   }
+}
+
+// The launches of a run never change (shapes, pointers and attributes are
+// fixed at load time), so after one eager run they are captured into an
+// executable graph and replayed with a single submission.  Per-kernel timing
+// needs the eager path (its event pairs must not end up inside a graph);
+// CVM_HIP_GRAPH=0 keeps it for good.
+void HipGraphRuntime::Run() {
+  if (graph_state_ == 0) {
+    const char* env = std::getenv("CVM_HIP_GRAPH");
+    graph_state_ = (env && std::string(env) == "0") ? -1 : 1;
+  }
+  if (graph_state_ < 0 || cvmhip_kernel_timing_active()) {
+    Launch();
+    return;
+  }
+  if (graph_state_ == 1) {  // first run: eager (operators may finish lazy set-up)
+    Launch();
+    graph_state_ = 2;
+    return;
+  }
+  if (graph_state_ == 2) {
+    HipCheck(cvmhip_stream_sync(stream_), "capture");
+    if (cvmhip_capture_begin(stream_) == CVMHIP_OK) {
+      bool ok = true;
+      try {
+        Launch();
+      } catch (...) {
+        ok = false;
+      }
+      void* exec = nullptr;
+      if (cvmhip_capture_end(stream_, &exec) == CVMHIP_OK && ok && exec) {
+        graph_exec_ = exec;
+        graph_state_ = 3;
+      } else {
+        if (exec) cvmhip_graph_destroy(exec);
+        graph_state_ = -1;  // not capturable: stay eager
+        Launch();
+        return;
+      }
+    } else {
+      graph_state_ = -1;
+      Launch();
+      return;
+    }
+  }
+  HipCheck(cvmhip_graph_launch(graph_exec_, stream_), "graph launch");
 }
 
 std::map<std::string, double> HipGraphRuntime::ProfileRun() {

@@ -112,7 +112,8 @@ class HipGraphRuntime {
   void LoadParams(const std::string& blob);
   // `data` tensor from host memory: int32 values, already widened
   void SetData(const int32_t* host, const Shape& shape);
-  void Run();
+  void Run();      // replays the captured graph once it exists
+  void Launch();   // issues every launch of a run on the stream, one by one
   void CopyOutputTo(int index, int32_t* host);  // synchronises the stream
 
   // device-resident variants used to time Run() alone
@@ -176,6 +177,8 @@ class HipGraphRuntime {
   struct Exec { uint32_t nid; const OpKernel* kernel; OpCall call; };
   std::vector<Exec> execs_;
   bool params_loaded_ = false;
+  void* graph_exec_ = nullptr;
+  int graph_state_ = 0;  // 0 undecided, -1 eager for good, 1 before the first run, 2 ready to capture, 3 captured
 
   // ---- fused executor: int8 NHWC activations + folded requantisation chains
   void BuildPlan();
