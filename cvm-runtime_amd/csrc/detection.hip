@@ -85,6 +85,25 @@ __device__ __forceinline__ int64_t iou100(const int32_t* r1, const int32_t* r2) 
   return overlap / uni;
 }
 
+// iou100(r1, r2) >= thr without the 64-bit division when the products are small
+// enough to compare exactly: floor(100*o/u) >= t  <=>  100*o >= t*u  for u > 0.
+__device__ __forceinline__ bool iou_at_least(const int32_t* r1, const int32_t* r2, int thr) {
+  const int64_t a1 = (int64_t)wsub(r1[2], r1[0]) * wsub(r1[3], r1[1]);
+  const int64_t a2 = (int64_t)wsub(r2[2], r2[0]) * wsub(r2[3], r2[1]);
+  const int64_t sum_area = (int64_t)((uint64_t)a1 + (uint64_t)a2);
+  const int32_t xr = r1[2] < r2[2] ? r1[2] : r2[2], xl = r1[0] > r2[0] ? r1[0] : r2[0];
+  const int32_t yb = r1[3] < r2[3] ? r1[3] : r2[3], yt = r1[1] > r2[1] ? r1[1] : r2[1];
+  int32_t w = wsub(xr, xl), h = wsub(yb, yt);
+  if (w < 0) w = 0;
+  if (h < 0) h = 0;
+  const int64_t overlap = (int64_t)h * w;
+  const int64_t uni = sum_area - overlap;
+  const int64_t small = (int64_t)1 << 40;
+  if (sum_area > 0 && sum_area < small && overlap < small && uni > 0 && thr > 0 && thr < (1 << 20))
+    return overlap * 100 >= (int64_t)thr * uni;
+  return iou100(r1, r2) >= thr;
+}
+
 __device__ __forceinline__ int clamp_vc(int vc, int n) { return vc > n ? n : (vc < 0 ? 0 : vc); }
 
 // The reference returns from the whole call at the first batch without valid
@@ -99,37 +118,65 @@ __device__ __forceinline__ int batch_state(const int32_t* valid_count, int b, in
 // Rank of row i among the first vc rows under (score descending, index
 // ascending) -- the order std::stable_sort gives (nms.cc:89-91).
 // Also gathers the row into its sorted slot.
+constexpr int RANK_JT = 1024;  // candidate rows one workgroup compares its 256 rows against
+
+__global__ void __launch_bounds__(256) k_zero32(int32_t* __restrict__ p, int64_t count) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) p[i] = 0;
+}
+
+// rank[i] += number of rows j of this workgroup's chunk that sort before row i.
+// The chunks of all workgroups add up with integer atomics, so the result does
+// not depend on their order.
 __global__ void __launch_bounds__(256)
-k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ order,
-           int32_t* __restrict__ sorted, int n, int k, int score_index, int64_t ws_stride) {
-  __shared__ int32_t tile[256];
+k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
+           int n, int k, int score_index) {
+  __shared__ __attribute__((aligned(16))) int32_t tile[RANK_JT];
+  const int b = blockIdx.z;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  const int base = blockIdx.y * RANK_JT;
+  if (blockIdx.x * 256 >= vc || base >= vc) return;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int32_t* xb = x + (int64_t)b * n * k;
+  const int32_t si = i < vc ? xb[(int64_t)i * k + score_index] : 0;
+#pragma unroll
+  for (int t = 0; t < RANK_JT / 256; ++t) {
+    const int j = base + t * 256 + threadIdx.x;
+    tile[t * 256 + threadIdx.x] = j < vc ? xb[(int64_t)j * k + score_index] : INT32_MIN;
+  }
+  __syncthreads();
+  const int lim = vc - base < RANK_JT ? vc - base : RANK_JT;
+  int r = 0;
+  for (int t = 0; t < lim; t += 4) {  // entries past vc hold INT32_MIN and an index above every row: they lose both tests
+    const int4 s4 = *reinterpret_cast<const int4*>(&tile[t]);
+    const int j = base + t;
+    r += (s4.x > si) || (s4.x == si && j < i);
+    r += (s4.y > si) || (s4.y == si && j + 1 < i);
+    r += (s4.z > si) || (s4.z == si && j + 2 < i);
+    r += (s4.w > si) || (s4.w == si && j + 3 < i);
+  }
+  if (i < vc && r) atomicAdd(&rank[(int64_t)b * n + i], r);
+}
+
+// row i moves to its sorted slot
+__global__ void __launch_bounds__(256)
+k_nms_scatter(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, const int32_t* __restrict__ rank,
+              int32_t* __restrict__ order, int32_t* __restrict__ sorted, int n, int k, int64_t ws_stride) {
   const int b = blockIdx.y;
   if (batch_state(valid_count, b, n) != 0) return;
   const int vc = clamp_vc(valid_count[b], n);
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (blockIdx.x * 256 >= vc) return;
+  if (i >= vc) return;
   const int32_t* xb = x + (int64_t)b * n * k;
-  const int32_t si = i < vc ? xb[(int64_t)i * k + score_index] : 0;
-  int rank = 0;
-  for (int base = 0; base < vc; base += 256) {
-    const int j = base + threadIdx.x;
-    __syncthreads();
-    tile[threadIdx.x] = j < vc ? xb[(int64_t)j * k + score_index] : INT32_MIN;
-    __syncthreads();
-    const int lim = vc - base < 256 ? vc - base : 256;
-    for (int t = 0; t < lim; ++t) {
-      const int32_t sj = tile[t];
-      rank += (sj > si) || (sj == si && base + t < i);
-    }
-  }
-  if (i < vc) {
-    order[b * ws_stride + rank] = i;
-    int32_t* dst = sorted + b * ws_stride * k + (int64_t)rank * k;
-    for (int c = 0; c < k; ++c) dst[c] = xb[(int64_t)i * k + c];
-  }
+  const int r = rank[(int64_t)b * n + i];
+  order[b * ws_stride + r] = i;
+  int32_t* dst = sorted + b * ws_stride * k + (int64_t)r * k;
+  for (int c = 0; c < k; ++c) dst[c] = xb[(int64_t)i * k + c];
 }
 
 constexpr int NMS_THREADS = 1024;
+constexpr int NMS_LDS_ROWS = 2048, NMS_LDS_K = 6;  // rows x columns of the LDS copy in k_nms_select (48 KiB)
 
 // One workgroup per batch walks the sorted rows in order.  Row i is emitted if
 // it survived and has id >= 0; a surviving row then suppresses, in parallel,
@@ -189,9 +236,24 @@ k_nms_select(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, i
     __syncthreads();
   }
 
+  // The greedy walk is a chain of dependent steps, each a barrier plus a few
+  // reads: when the candidate rows fit (top_k bounds them in practice) they and
+  // the removal flags are staged in LDS, whose latency is a tenth of HBM's.
+  __shared__ int32_t s_rows[NMS_LDS_ROWS * NMS_LDS_K];
+  __shared__ int32_t s_rem[NMS_LDS_ROWS];
+  __shared__ int32_t s_nn[NMS_LDS_ROWS + 1];
+  if (keep <= NMS_LDS_ROWS && k <= NMS_LDS_K) {
+    for (int i = tid; i < keep * k; i += NMS_THREADS) s_rows[i] = srt[i];
+    for (int i = tid; i < keep; i += NMS_THREADS) s_rem[i] = 0;
+    for (int i = tid; i <= keep; i += NMS_THREADS) s_nn[i] = nn[i];
+    srt = s_rows;
+    rem = s_rem;
+    nn = s_nn;
+  }
+
   int yi = 0;
   for (int i = 0; i < keep; ++i) {
-    __syncthreads();  // removals from the previous row are visible
+    __syncthreads();  // removals from the previous row (and the staging above) are visible
     if (rem[i]) continue;
     const int32_t* r1 = srt + (int64_t)i * k;
     if (r1[0] >= 0) {
@@ -204,7 +266,7 @@ k_nms_select(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, i
       if (rem[j]) continue;
       const int32_t* r2 = srt + (int64_t)j * k;
       if (force_suppress || id_index < 0 || id1 == r2[id_index])
-        if (iou100(r1 + coord_start, r2 + coord_start) >= iou_threshold) rem[j] = 1;
+        if (iou_at_least(r1 + coord_start, r2 + coord_start, iou_threshold)) rem[j] = 1;
     }
   }
   // max_output_size keeps the first `max_output_size` emitted rows (nms.cc:126-137)
@@ -241,9 +303,9 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
   return check_launch("get_valid_counts.scatter");
 }
 
-// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k]
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n]
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
-  return (size_t)batches * ((size_t)n * (3 + (size_t)k) + 1) * sizeof(int32_t);
+  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 1) * sizeof(int32_t);
 }
 
 int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
@@ -262,9 +324,15 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
   int32_t* nextneg = order + (size_t)batches * n;
   int32_t* removed = nextneg + (size_t)batches * (n + 1);
   int32_t* sorted = removed + (size_t)batches * n;
-  dim3 grid((n + 255) / 256, batches);
-  k_nms_rank<<<grid, 256, 0, s>>>(x, valid_count, order, sorted, n, k, score_index, (int64_t)n);
+  int32_t* rank = sorted + (size_t)batches * n * k;
+  k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
+  dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
+  k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, n, k, score_index);
   int rc = check_launch("nms.rank");
+  if (rc) return rc;
+  dim3 grid((n + 255) / 256, batches);
+  k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, n, k, (int64_t)n);
+  rc = check_launch("nms.scatter");
   if (rc) return rc;
   k_nms_select<<<batches, NMS_THREADS, 0, s>>>(x, valid_count, y, order, sorted, nextneg, removed, n, k,
                                                max_output_size, iou_threshold, topk, coord_start, id_index,
