@@ -205,11 +205,16 @@ int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, 
 /* ---- fused int8 path.  No counterpart in the reference: it runs every node as
  * its own int32 kernel.  Inside a verified graph every conv2d/dense operand is
  * proven to fit 8 bits (src/top/nn/convolution.cc:153-158, src/top/nn/nn.cc:26-31),
- * so the graph executor keeps such activations as int8 NHWC (channels padded to
- * cvmhip_pad_channels(c)) between layers and folds the requantisation chain
- * that follows a producer -- any sequence of relu / cvm_right_shift / cvm_clip /
- * clip -- into the producer's epilogue.  Results are bit-identical to running
- * the nodes one by one. */
+ * so the graph executor keeps such activations as int8 between layers and folds
+ * the requantisation chain that follows a producer -- any sequence of relu /
+ * cvm_right_shift / cvm_clip / clip -- into the producer's epilogue.  Results
+ * are bit-identical to running the nodes one by one.
+ * int8 activation layout ("act" below): channels padded to cp =
+ * cvmhip_pad_channels(c) = 4, 8, 16 or a multiple of 32.  cp <= 16: NHWC.
+ * Otherwise blocks of 32 consecutive pixels (linear index over n, h, w) x 32
+ * channels, each stored as the 1 KiB operand fragment of v_mfma_i32_32x32x32_i8:
+ *   offset(p, c) = ((p/32)*(cp/32) + c/32)*1024 + ((c/16)%2)*512 + (p%32)*16 + c%16
+ * A buffer for npix pixels has cvmhip_packed_act_bytes(npix, c) bytes, 16-byte aligned. */
 enum { CVMHIP_STAGE_RELU = 1, CVMHIP_STAGE_RSHIFT = 2, CVMHIP_STAGE_CLIP = 3 };
 typedef struct {
   int32_t kind;        /* CVMHIP_STAGE_* */
@@ -223,31 +228,31 @@ typedef struct {
 } cvmhip_chain;
 
 int cvmhip_pad_channels(int channels);
-/* int32 NCHW <-> int8 NHWC (narrowing is static_cast<int8_t>) */
+/* int32 NCHW <-> int8 act layout (narrowing is static_cast<int8_t>) */
 int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream);
 int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void* stream);
-/* conv2d / dense on int8 NHWC input with packed filter (cvmhip_pack_weights):
+/* conv2d / dense on int8 act input with packed filter (cvmhip_pack_weights):
  *   v = chain(acc + bias);  if (residual) v = chain2(v + residual);
- * out is int8 NHWC when out_is_i8, else int32 NCHW.  residual is int8 NHWC with
- * the output's geometry, or NULL. */
+ * out is int8 act layout when out_is_i8, else int32 NCHW.  residual is an int8 act
+ * tensor with the output's geometry, or NULL. */
 int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                      const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
                      int n, int ic, int h, int wd, int oc, int kh, int kw,
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
-/* depthwise conv2d (groups == channels == out channels) on int8 NHWC, filter packed by
+/* depthwise conv2d (groups == channels == out channels) on int8 act tensors, filter packed by
  * cvmhip_pack_depthwise_weights into [kh*kw][cp] int8 */
 size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw);
 int cvmhip_pack_depthwise_weights(const int32_t* w, void* wp, int c, int kh, int kw, void* stream);
 int cvmhip_depthwise_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                                void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
                                int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
-/* out = chain(a + b) on int8 NHWC tensors of identical geometry */
+/* out = chain(a + b) on int8 act tensors of identical geometry */
 int cvmhip_add_i8(const void* a, const void* b, const cvmhip_chain* chain, void* out, int out_is_i8,
                   int n, int c, int hw, void* stream);
-/* max_pool2d on int8 NHWC (padding counts as the smallest value, as INT32_MIN does) */
+/* max_pool2d on int8 act tensors (padding counts as the smallest value, as INT32_MIN does) */
 int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, int oh, int ow,
                          int kh, int kw, int stride_h, int stride_w, int pad_h, int pad_w, void* stream);
-/* out[n][c] = chain(sum over h,w of x[n][h][w][c]); out int8 [n][cp] or int32 [n][c] */
+/* out[n][c] = chain(sum over h,w of x[n][h][w][c]); out int8 act tensor of n pixels, or int32 [n][c] */
 int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int out_is_i8,
                      int n, int c, int hw, void* stream);
 
