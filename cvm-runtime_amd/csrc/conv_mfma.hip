@@ -532,6 +532,11 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + i) * (nch + 1)) * 1024 + lane * 16;
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   const int lconst = lgrp * 512;
+  const int8_t* tapptr[TN];                // per-lane operand address of the current filter tap
+  int okv[TN];                             // 0: the lane reads the zero granule for this tap
+  bool need_tap = true;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) { tapptr[j] = zero; okv[j] = 0; }
 
   stage_bias<BM>(sBias, ep, g.OC, oc0, tid);
 
@@ -579,15 +584,23 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
         for (int j = 0; j < TN; ++j) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb * 1024));
       } else {
-        const int soff = live ? (r * g.DH) * g.W + s * g.DW : 0;  // in pixels
-        const int coff = (live ? (ch >> 5) * 1024 : 0) + lconst;
+        // the address of a pixel is computed once per filter tap; the Cp/32 chunks of
+        // the tap differ by a multiple of 1 KiB (not applied to lanes that read zeros)
+        if (live && need_tap) {
+          const int soff = (r * g.DH) * g.W + s * g.DW;  // in pixels
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int pin = rowbase[j] + soff;
-          const int8_t* src = xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + ((pin & 31) << 4) + coff);
-          if (MODE == WAVE_PAD) src = (live && (((rowmask[j] >> r) & (colmask[j] >> s)) & 1u)) ? src : zero;
-          put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(src));
+          for (int j = 0; j < TN; ++j) {
+            const int pin = rowbase[j] + soff;
+            const bool ok = MODE != WAVE_PAD || ((((rowmask[j] >> r) & (colmask[j] >> s)) & 1u) != 0);
+            tapptr[j] = ok ? xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + ((pin & 31) << 4) + lconst) : zero;
+            okv[j] = ok ? 1 : 0;
+          }
+          need_tap = false;
         }
+        const int coff = live ? (ch >> 5) * 1024 : 0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(tapptr[j] + (okv[j] ? coff : 0)));
       }
       if (live) {
         ++cur;
@@ -597,6 +610,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
             ch = 0;
             ++tap;
             if (++s == g.KW) { s = 0; ++r; }
+            need_tap = true;
           }
         }
       }
@@ -901,8 +915,8 @@ static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
 // A wavefront that runs alone pays full latency for every instruction and every
 // load, so the aim is one round of workgroups with as little serial K per
 // wavefront as possible: the deepest K split (at least two chunks per wavefront)
-// of the largest tile whose grid is resident at once.  Returns -1 when even the
-// unsplit grid needs more than two rounds; the tiled kernel serves those.
+// of the largest tile whose grid is resident at once.  Larger grids run unsplit
+// in several rounds (the wavefronts of a workgroup then share the filter through L1).
 static int choose_wave_cfg(const ConvGeom& g) {
   const int nlive = g.K / 32;
   const int first = g.OC > 32 ? 0 : 4;
@@ -910,10 +924,10 @@ static int choose_wave_cfg(const ConvGeom& g) {
   for (int i = first; i < last; ++i) {
     const WaveCfg& c = kWaveCfgs[i];
     if (c.ksplit > 1 && nlive < 2 * c.ksplit) continue;
-    const int64_t capacity = 256 * (int64_t)c.blocks_per_cu * (c.ksplit == 1 ? 2 : 1);
-    if (wave_cfg_blocks(c, g) <= capacity) return i;
+    const int64_t capacity = 256 * (int64_t)c.blocks_per_cu;
+    if (c.ksplit == 1 || wave_cfg_blocks(c, g) <= capacity) return i;
   }
-  return -1;
+  return last - 1;
 }
 
 static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
