@@ -919,6 +919,9 @@ static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
 // in several rounds (the wavefronts of a workgroup then share the filter through L1).
 static int choose_wave_cfg(const ConvGeom& g) {
   const int nlive = g.K / 32;
+  // very few pixels, deep K (fully connected layers, the last stage): even the deepest split of
+  // the 64-channel tile leaves SIMDs without a wavefront, so halve the tile instead
+  if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < 128) return 4;
   const int first = g.OC > 32 ? 0 : 4;
   const int last = g.OC > 32 ? 4 : kNumWaveCfgs;
   for (int i = first; i < last; ++i) {
