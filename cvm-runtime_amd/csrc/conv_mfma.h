@@ -42,6 +42,7 @@ struct ConvGeom {
   int64_t P;               // filled by conv_igemm: N*OH*OW
   int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
   FastDiv div_ohw, div_ow, div_ct, div_kw;  // filled by conv_igemm: division by OH*OW, OW, Cp/32 and KW
+  int row_bytes;           // > 0: row-window input (see stem_* below): bytes of K per filter row, 16 or 32
 };
 
 // What happens to an accumulator before it is stored:
@@ -90,6 +91,25 @@ __host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c
 
 int pad_channels(int c);
 size_t packed_act_bytes(int64_t npix, int c);
+
+// ---- row-window form of a convolution over a few input channels (the RGB stem).
+// The input is stored as int8 [N][Hp][Wp][4], already padded with zeros, so the
+// KW taps x 4 channel bytes of one filter row are contiguous in memory; they are
+// read as one window of row_bytes = 16 or 32 bytes and K is ordered
+// k = kh*row_bytes + kw*4 + c.  No tap is ever outside the stored tensor, so the
+// kernel needs neither masks nor per-tap address arithmetic.
+struct StemGeom {
+  int hp, wp;        // stored (padded) height and width
+  int row_bytes;     // 16 or 32
+  int k, kp;         // KH*row_bytes, rounded up to 64
+  size_t bytes;      // size of the stored input
+};
+bool stem_eligible(int c, int kh, int kw, int dil_h, int dil_w);
+StemGeom stem_geom(int n, int h, int w, int kh, int kw, int sh, int sw, int ph, int pw);
+size_t packed_stem_weight_bytes(int oc, int kp);
+int pack_stem_input(const int32_t* x, int8_t* xs, int n, int c, int h, int w, int kh, int kw, int sh, int sw, int ph,
+                    int pw, hipStream_t s);
+int pack_stem_weights(const int32_t* w, int8_t* wp, int oc, int c, int kh, int kw, hipStream_t s);
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp);
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw);
 

@@ -442,9 +442,11 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 //   MODE WAVE_IDENT  1x1, stride 1, no padding: the operand of output pixel block
 //                    t is input block t, addresses are base + chunk * 1 KiB
 //        WAVE_NOPAD  no padding: every tap of a valid output pixel is inside the image
+//        WAVE_ROWS   row-window input of a few-channel convolution (conv_mfma.h: StemGeom):
+//                    a chunk is 32 bytes of one or two filter rows, always inside the stored tensor
 //        WAVE_PAD    padding: per-lane row / column validity masks (KH, KW <= 32),
 //                    out-of-image granules are read from a zero granule
-enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2 };
+enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE>
 __global__ void __launch_bounds__(NW * 64, MINW)
@@ -499,6 +501,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       const int ow = rem - oh * g.OW;
       const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
       rowbase[j] = (n * g.H + ih0) * g.W + iw0;
+      if (MODE == WAVE_ROWS) rowbase[j] *= 4;   // byte offset of the window of filter row 0 (g.H, g.W: stored size, no padding left)
       xb[j] = xp;
       unsigned rm = 0, cm = 0;
       if (MODE == WAVE_PAD) {
@@ -513,14 +516,14 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 
   // K range of this wavefront, in chunks of 32 bytes; chunks past the true K are never visited
   const int nch = g.Kp >> 5;
-  const int nlive = g.K >> 5;
+  const int nlive = (g.K + 31) >> 5;
   const int per = (nlive + KSPLIT - 1) / KSPLIT;
   const int c_begin = kw_ * per;
   const int c_end = c_begin + per < nlive ? c_begin + per : nlive;
   const int niter = (per + D - 1) / D;
   int cur = c_begin;
   int tap = 0, ch = 0, r = 0, s = 0;
-  if (MODE != WAVE_IDENT) {
+  if (MODE != WAVE_IDENT && MODE != WAVE_ROWS) {
     tap = (int)fastdiv((unsigned)cur, g.div_ct);
     ch = (cur - tap * ctiles) * 32;
     r = (int)fastdiv((unsigned)tap, g.div_kw);
@@ -583,6 +586,13 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
         const int cb = live ? cur : c_begin < nlive ? c_begin : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb * 1024));
+      } else if (MODE == WAVE_ROWS) {
+        // 16-byte unit k16 of K: filter row k16 / (row_bytes/16), part k16 % (row_bytes/16) of its window
+        const int k16 = (live ? cur : 0) * 2 + lgrp;
+        const int sh16 = g.row_bytes >> 5;   // 0 or 1
+        const int off = (k16 >> sh16) * (g.W * 4) + (k16 & sh16) * 16;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xp + (rowbase[j] + off)));
       } else {
         // the address of a pixel is computed once per filter tap; the Cp/32 chunks of
         // the tap differ by a multiple of 1 KiB (not applied to lanes that read zeros)
@@ -604,7 +614,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       }
       if (live) {
         ++cur;
-        if (MODE != WAVE_IDENT) {
+        if (MODE != WAVE_IDENT && MODE != WAVE_ROWS) {
           ch += 32;
           if (ch >= g.Cp) {
             ch = 0;
@@ -717,8 +727,9 @@ __global__ void __launch_bounds__(256) k_pack_act(const int32_t* __restrict__ x,
 // lane l holds row (l & 31), bytes (l >> 5)*16 .. +15 of the chunk.  Each tile
 // has nch + 1 chunks; the last one is all zero (a K range that ends early reads
 // it instead of branching).  Layout: [OCp/32][nch + 1][64][16].
+// row_bytes > 0 selects the row-window K order k = kh*row_bytes + kw*4 + c (conv_mfma.h: StemGeom).
 __global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict__ w, int8_t* __restrict__ wp, int64_t total,
-                                                      int oc, int ic, int taps, int cp, int nch) {
+                                                      int oc, int ic, int taps, int cp, int nch, int row_bytes, int kw_taps) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
     const int d = (int)(i & 3);
@@ -728,7 +739,12 @@ __global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict_
     const int64_t tile = t / (nch + 1);
     const int64_t o = tile * 32 + (lane & 31);
     const int k = chunk * 32 + (lane >> 5) * 16 + d * 4;
-    const int tap = k / cp, c = k - tap * cp;
+    int tap = k / cp, c = k - tap * cp;
+    if (row_bytes > 0) {
+      const int r = k / row_bytes, s4 = (k - r * row_bytes) >> 2;   // filter row, tap inside the window
+      tap = s4 < kw_taps ? r * kw_taps + s4 : taps;                  // window bytes past the last tap multiply by zero
+      c = 0;
+    }
     uint32_t pack = 0;
     if (o < oc && tap < taps && chunk < nch) {
 #pragma unroll
@@ -738,6 +754,28 @@ __global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict_
       }
     }
     reinterpret_cast<uint32_t*>(wp)[i] = pack;
+  }
+}
+
+// int32 NCHW -> row-window input int8 [N][hp][wp][4], zero outside the image (conv_mfma.h: StemGeom)
+__global__ void __launch_bounds__(256) k_pack_stem(const int32_t* __restrict__ x, uint32_t* __restrict__ xs, int64_t total,
+                                                   int nimg, int c, int h, int w, int hp, int wp, int ph, int pw) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int q = (int)(i % wp);
+    const int64_t t = i / wp;
+    const int p = (int)(t % hp);
+    const int64_t n = t / hp;
+    const int ih = p - ph, iw = q - pw;
+    uint32_t pack = 0;
+    if (n < nimg && ih >= 0 && ih < h && iw >= 0 && iw < w) {   // the slack behind the last image is cleared
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int32_t v = j < c ? x[((n * c + j) * h + ih) * w + iw] : 0;
+        pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
+      }
+    }
+    xs[i] = pack;
   }
 }
 
@@ -851,9 +889,50 @@ int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, h
   weight_dims(oc, ic, kh, kw, &ocp, &kp);
   const int nch = kp / 32;
   const int64_t total = (int64_t)(ocp / 32) * (nch + 1) * 256;  // dwords
-  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, ic, kh * kw, pad_channels(ic), nch);
+  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, ic, kh * kw, pad_channels(ic), nch, 0, kw);
   return check_launch("pack_weights");
 }
+
+bool stem_eligible(int c, int kh, int kw, int dil_h, int dil_w) {
+  return c >= 1 && c <= 4 && kw * 4 <= 32 && kh >= 1 && dil_h == 1 && dil_w == 1;
+}
+
+StemGeom stem_geom(int n, int h, int w, int kh, int kw, int sh, int sw, int ph, int pw) {
+  StemGeom sg;
+  sg.row_bytes = kw * 4 <= 16 ? 16 : 32;
+  sg.k = kh * sg.row_bytes;
+  sg.kp = (sg.k + KSTEP - 1) / KSTEP * KSTEP;
+  const int oh = (h + 2 * ph - kh) / sh + 1, ow = (w + 2 * pw - kw) / sw + 1;
+  // rows and columns the windows of the last output pixel reach (K is rounded up to whole 32-byte chunks)
+  const int max_row = (((sg.k + 31) / 32) * 2 - 1) / (sg.row_bytes / 16);
+  const int need_h = (oh - 1) * sh + max_row + 1, need_w = (ow - 1) * sw + sg.row_bytes / 4;
+  sg.hp = need_h > h + 2 * ph ? need_h : h + 2 * ph;
+  sg.wp = need_w > w + 2 * pw ? need_w : w + 2 * pw;
+  sg.bytes = ((size_t)n * sg.hp * sg.wp * 4 + 64 + 255) / 256 * 256;   // 64: the last window may run past the last row
+  return sg;
+}
+
+int pack_stem_input(const int32_t* x, int8_t* xs, int n, int c, int h, int w, int kh, int kw, int sh, int sw, int ph,
+                    int pw, hipStream_t s) {
+  const StemGeom sg = stem_geom(n, h, w, kh, kw, sh, sw, ph, pw);
+  const int64_t total = (int64_t)sg.bytes / 4;   // the slack behind the last row is cleared too
+  KernelTimer timer("k_pack_stem", (double)n * c * h * w * 5.0, s);
+  k_pack_stem<<<grid_for(total, 256), 256, 0, s>>>(x, reinterpret_cast<uint32_t*>(xs), total, n, c, h, w, sg.hp, sg.wp, ph, pw);
+  return check_launch("pack_stem");
+}
+
+int pack_stem_weights(const int32_t* w, int8_t* wp, int oc, int c, int kh, int kw, hipStream_t s) {
+  const int rb = kw * 4 <= 16 ? 16 : 32;
+  const int kp = (kh * rb + KSTEP - 1) / KSTEP * KSTEP;
+  const int ocp = (oc + 127) / 128 * 128;
+  const int nch = kp / 32;
+  const int64_t total = (int64_t)(ocp / 32) * (nch + 1) * 256;  // dwords
+  k_pack_weights<<<grid_for(total, 256), 256, 0, s>>>(w, wp, total, oc, c, kh * kw, 4, nch, rb, kw);
+  return check_launch("pack_stem_weights");
+}
+
+size_t packed_stem_weight_bytes(int oc, int kp) { return (size_t)((oc + 127) / 128 * 128 / 32) * (kp / 32 + 1) * 1024 + 8192; }
+
 
 template <int WM, int WN, int OUT>
 static void launch_tile(int gran, bool wide, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
@@ -897,6 +976,7 @@ static void launch_wave_mode(int mode, unsigned grid, hipStream_t s, const int8_
                              const ConvGeom& g, const Epilogue& ep) {
   if (mode == WAVE_IDENT) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_IDENT><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
   else if (mode == WAVE_NOPAD) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_NOPAD><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
+  else if (mode == WAVE_ROWS) k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_ROWS><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
   else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_PAD><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
 }
 
@@ -952,13 +1032,15 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
       g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
     return arg_error("conv geometry");
   if (g.Cp != 4 && g.Cp != 8 && g.Cp != 16 && (g.Cp % 32) != 0) return arg_error("conv channel padding");
+  if (g.row_bytes != 0 && (g.Cp != 4 || (g.row_bytes != 16 && g.row_bytes != 32) || g.PH != 0 || g.PW != 0 || g.KW * 4 > g.row_bytes))
+    return arg_error("conv row-window geometry");
   if (((uintptr_t)xp | (uintptr_t)wp) & 15) return arg_error("conv operand alignment");
   if ((ep0.out_mode == OUT_I8_ACT || ep0.residual) && ep0.out_cp != pad_channels(g.OC))
     return arg_error("conv int8 output layout");
   if (((uintptr_t)out | (uintptr_t)ep0.residual) & 3) return arg_error("conv output alignment");
   if (ep0.out_mode == OUT_I8_ACT && ep0.out_cp >= 16 && ((uintptr_t)out & 15)) return arg_error("conv output alignment");
   g.taps = g.KH * g.KW;
-  g.K = g.taps * g.Cp;
+  g.K = g.row_bytes ? g.KH * g.row_bytes : g.taps * g.Cp;
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
   if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
@@ -988,14 +1070,16 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   const char* conv_kind = getenv("CVM_HIP_CONV");
   const char* wave_forced = getenv("CVM_HIP_WAVECFG");
   const bool nopad = g.PH == 0 && g.PW == 0;
-  const bool wave_ok = (g.Cp % 32) == 0 && (nopad || (g.KH <= 32 && g.KW <= 32));
+  const bool rows = g.row_bytes != 0;
+  const bool wave_ok = rows || ((g.Cp % 32) == 0 && (nopad || (g.KH <= 32 && g.KW <= 32)));
   int cfg = wave_ok ? choose_wave_cfg(g) : -1;
-  if (conv_kind && conv_kind[0] == 'l') cfg = -1;
+  if (conv_kind && conv_kind[0] == 'l' && !rows) cfg = -1;
   if (wave_ok && conv_kind && conv_kind[0] == 'w' && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
   if (cfg >= 0) {
-    const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
-                         ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
+    const int mode = rows ? WAVE_ROWS
+                          : (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                                ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
     KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);

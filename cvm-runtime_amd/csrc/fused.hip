@@ -252,6 +252,57 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                     as_stream(stream));
 }
 
+// ---- row-window convolution over at most 4 input channels (the RGB stem of a network)
+int cvmhip_stem_eligible(int c, int kh, int kw, int dil_h, int dil_w) { return stem_eligible(c, kh, kw, dil_h, dil_w) ? 1 : 0; }
+
+size_t cvmhip_stem_input_bytes(int n, int h, int w, int kh, int kw, int stride_h, int stride_w, int pad_h, int pad_w) {
+  if (n < 1 || h < 1 || w < 1 || kh < 1 || kw < 1 || kw > 8 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0 ||
+      h + 2 * pad_h < kh || w + 2 * pad_w < kw)
+    return 0;
+  return stem_geom(n, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w).bytes;
+}
+
+int cvmhip_pack_stem_input(const int32_t* x, void* xs, int n, int c, int h, int w, int kh, int kw,
+                           int stride_h, int stride_w, int pad_h, int pad_w, void* stream) {
+  if (!x || !xs || ((uintptr_t)xs & 15) || !stem_eligible(c, kh, kw, 1, 1) ||
+      cvmhip_stem_input_bytes(n, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w) == 0)
+    return arg_error("pack_stem_input");
+  return pack_stem_input(x, reinterpret_cast<int8_t*>(xs), n, c, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w, as_stream(stream));
+}
+
+size_t cvmhip_packed_stem_weight_bytes(int oc, int kh, int kw) {
+  if (oc < 1 || kh < 1 || kw < 1 || kw > 8) return 0;
+  const int rb = kw * 4 <= 16 ? 16 : 32;
+  return packed_stem_weight_bytes(oc, (kh * rb + 63) / 64 * 64);
+}
+
+int cvmhip_pack_stem_weights(const int32_t* w, void* wp, int oc, int c, int kh, int kw, void* stream) {
+  if (!w || !wp || oc < 1 || !stem_eligible(c, kh, kw, 1, 1)) return arg_error("pack_stem_weights");
+  return pack_stem_weights(w, reinterpret_cast<int8_t*>(wp), oc, c, kh, kw, as_stream(stream));
+}
+
+int cvmhip_conv2d_stem_i8(const void* xs, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          void* out, int out_is_i8, int n, int c, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, void* stream) {
+  if (!xs || !wp || !out || oc < 1 || !stem_eligible(c, kh, kw, 1, 1) ||
+      cvmhip_stem_input_bytes(n, h, wd, kh, kw, stride_h, stride_w, pad_h, pad_w) == 0)
+    return arg_error("conv2d_stem_i8");
+  const StemGeom sg = stem_geom(n, h, wd, kh, kw, stride_h, stride_w, pad_h, pad_w);
+  ConvGeom g = {};
+  g.N = n; g.H = sg.hp; g.W = sg.wp; g.Cp = 4; g.C = c;
+  g.OC = oc;
+  g.OH = (h + 2 * pad_h - kh) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - kw) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = 0; g.PW = 0; g.DH = 1; g.DW = 1;
+  g.row_bytes = sg.row_bytes;
+  Epilogue ep = {};
+  ep.bias = bias;
+  if (!make_chain(chain, &ep.chain)) return arg_error("conv2d_stem_i8 chain");
+  ep.out_mode = out_is_i8 ? OUT_I8_ACT : OUT_I32_NCHW;
+  ep.out_cp = pad_channels(oc);
+  return conv_igemm(reinterpret_cast<const int8_t*>(xs), reinterpret_cast<const int8_t*>(wp), out, g, ep, as_stream(stream));
+}
+
 size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw) {
   return ((size_t)pad_channels(c) * kh * kw + 255) / 256 * 256;
 }

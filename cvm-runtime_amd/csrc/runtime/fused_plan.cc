@@ -250,7 +250,35 @@ void HipGraphRuntime::BuildPlan() {
         st.oc = (int)shape_[we][0];
         ok = shape_[we].size() == 2 && shape_[we][1] == (int64_t)st.c * st.kh * st.kw;
       }
-      if (ok) {
+      // A few-channel input that only exists as int32 (the image itself) goes through the
+      // row-window form: packed once into a zero-padded int8 tensor, convolved without masks.
+      const bool stem = ok && op == "conv2d" && st.kind == PlanStep::CONV && !has_i8[src] && has_i32[src] &&
+                        cvmhip_stem_eligible(st.c, st.kh, st.kw, st.dh, st.dw) &&
+                        cvmhip_stem_input_bytes(st.n, st.h, st.w, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw) > 0;
+      if (stem) {
+        auto in = std::make_shared<DeviceBuffer>();
+        Check(cvmhip_alloc(&in->ptr, cvmhip_stem_input_bytes(st.n, st.h, st.w, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw)),
+              "row-window input buffer");
+        auto buf = std::make_shared<DeviceBuffer>();
+        Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_stem_weight_bytes(st.oc, st.kh, st.kw)), "filter buffer");
+        Check(cvmhip_pack_stem_weights(entry_ptr_[we], buf->ptr, st.oc, st.c, st.kh, st.kw, stream_), "filter pack");
+        PlanStep pk = st;
+        pk.kind = PlanStep::STEMPACK;
+        pk.label = "pack_stem_input";
+        pk.src = pk.dst = src;
+        pk.aux = in;
+        plan.push_back(pk);
+        st.stem = true;
+        st.aux = in;
+        st.weights = buf;
+        st.src = src;
+        st.src2 = kNone;
+        Bound b;
+        const uint32_t out = follow_chain(out0, &st.chain, &b);
+        finish_output(&st, out, b);
+        plan.push_back(st);
+        done = true;
+      } else if (ok) {
         need_i8(src);
         auto buf = std::make_shared<DeviceBuffer>();
         if (st.kind == PlanStep::CONV) {
@@ -282,7 +310,7 @@ void HipGraphRuntime::BuildPlan() {
         for (int swap = 0; swap < 2 && !folded; ++swap) {
           const uint32_t x = swap ? be : ae, r = swap ? ae : be;
           const int ps = producer_step[x], pr = producer_step[r];
-          if (ps < 0 || pr < 0 || pr >= ps) continue;
+          if (ps < 0 || pr < 0 || pr >= ps || plan[ps].stem) continue;
           PlanStep& cs = plan[ps];
           if (cs.kind != PlanStep::CONV || cs.dst != x || !cs.out_i8 || cs.src2 != kNone) continue;
           if (uses[x].size() != 1 || is_head[x]) continue;
@@ -439,8 +467,18 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
     case PlanStep::UNPACK:
       Check(cvmhip_unpack_nhwc_i8(i8_ptr_[st.src], entry_ptr_[st.dst], st.n, st.c, st.h, stream_), "unpack");
       break;
+    case PlanStep::STEMPACK:
+      Check(cvmhip_pack_stem_input(entry_ptr_[st.src], static_cast<DeviceBuffer*>(st.aux.get())->ptr, st.n, st.c, st.h, st.w,
+                                   st.kh, st.kw, st.sh, st.sw, st.ph, st.pw, stream_), "pack_stem_input");
+      break;
     case PlanStep::CONV: {
       void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      if (st.stem) {
+        Check(cvmhip_conv2d_stem_i8(static_cast<DeviceBuffer*>(st.aux.get())->ptr, static_cast<DeviceBuffer*>(st.weights.get())->ptr,
+                                    st.bias, &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw,
+                                    st.sh, st.sw, st.ph, st.pw, stream_), "conv2d_stem_i8");
+        break;
+      }
       const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
       Check(cvmhip_conv2d_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res,
                              &st.chain2, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh,

@@ -90,7 +90,7 @@ struct Node {
 
 // One launch of the fused executor (fused_plan.cc).
 struct PlanStep {
-  enum Kind { NODE, PACK, UNPACK, CONV, DWCONV, ADD, POOL, SUM } kind = NODE;
+  enum Kind { NODE, PACK, UNPACK, STEMPACK, CONV, DWCONV, ADD, POOL, SUM } kind = NODE;
   std::string label;            // operator name for the time table
   size_t exec_index = 0;        // NODE: index into execs_
   uint32_t src = 0, src2 = 0, dst = 0;  // entry ids (src2: residual / second addend; UINT32_MAX = none)
@@ -98,6 +98,8 @@ struct PlanStep {
   cvmhip_chain chain{}, chain2{};
   const int32_t* bias = nullptr;
   std::shared_ptr<void> weights;  // packed filter (device)
+  std::shared_ptr<void> aux;      // row-window copy of the input (device), see cvmhip_pack_stem_input
+  bool stem = false;              // CONV through the row-window form
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;
 };
 

@@ -422,3 +422,26 @@ def sum_hw_i8(xp, n, c, hw, chain1=None, out_is_i8=False):
     check(lib().cvmhip_sum_hw_i8(_vp(xp), ctypes.byref(chain1) if chain1 else None, _vp(out), int(out_is_i8),
                                  n, c, hw, _stream()))
     return out
+
+
+def conv2d_stem_i8(x, w, bias=None, chain1=None, out_is_i8=True, strides=(1, 1), padding=(0, 0)):
+    """conv2d over <= 4 input channels in row-window form; x and w are int32 NCHW / OIHW device tensors."""
+    L = lib()
+    n, c, h, wd = x.shape
+    oc, _, kh, kw = w.shape
+    L.cvmhip_stem_input_bytes.restype = ctypes.c_size_t
+    L.cvmhip_packed_stem_weight_bytes.restype = ctypes.c_size_t
+    assert L.cvmhip_stem_eligible(c, kh, kw, 1, 1)
+    xs = _workspace(L.cvmhip_stem_input_bytes(n, h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1]), x.device)
+    wp = _workspace(L.cvmhip_packed_stem_weight_bytes(oc, kh, kw), x.device)
+    check(L.cvmhip_pack_stem_input(_ptr(x), _vp(xs), n, c, h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1], _stream()))
+    check(L.cvmhip_pack_stem_weights(_ptr(w), _vp(wp), oc, c, kh, kw, _stream()))
+    oh, ow = conv_out_hw(h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1], 1, 1)
+    if out_is_i8:
+        out = _act_buffer(n * oh * ow, oc, x.device)
+    else:
+        out = torch.empty((n, oc, oh, ow), dtype=torch.int32, device=x.device)
+    check(L.cvmhip_conv2d_stem_i8(_vp(xs), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None, _vp(out),
+                                  int(out_is_i8), n, c, h, wd, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                  _stream()))
+    return out

@@ -239,6 +239,19 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                      const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
                      int n, int ic, int h, int wd, int oc, int kh, int kw,
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* conv2d over at most 4 input channels with kw <= 8, dilation 1 (the RGB stem of a network), in
+ * row-window form: the input is packed once per inference into int8 [n][hp][wp][4], zero padded, so
+ * that the kw taps x 4 channel bytes of a filter row are one contiguous window and no tap lies
+ * outside the stored tensor; K is ordered (kh, window byte).  Same arithmetic as cvmhip_conv2d_i8. */
+int cvmhip_stem_eligible(int c, int kh, int kw, int dil_h, int dil_w);
+size_t cvmhip_stem_input_bytes(int n, int h, int w, int kh, int kw, int stride_h, int stride_w, int pad_h, int pad_w);
+int cvmhip_pack_stem_input(const int32_t* x, void* xs, int n, int c, int h, int w, int kh, int kw,
+                           int stride_h, int stride_w, int pad_h, int pad_w, void* stream);
+size_t cvmhip_packed_stem_weight_bytes(int oc, int kh, int kw);
+int cvmhip_pack_stem_weights(const int32_t* w, void* wp, int oc, int c, int kh, int kw, void* stream);
+int cvmhip_conv2d_stem_i8(const void* xs, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          void* out, int out_is_i8, int n, int c, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, void* stream);
 /* depthwise conv2d (groups == channels == out channels) on int8 act tensors, filter packed by
  * cvmhip_pack_depthwise_weights into [kh*kw][cp] int8 */
 size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw);

@@ -123,6 +123,34 @@ def test_conv2d_i8(case, conv_kernel, dev):
         eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32")
 
 
+STEM_CASES = [
+    # n, c, h, w, oc, kh, kw, stride, pad
+    (2, 3, 32, 32, 64, 7, 7, 2, 3),      # ResNet stem shape, shrunk
+    (1, 3, 20, 24, 16, 3, 3, 1, 1),      # VGG / CIFAR stem: 16-byte windows, two filter rows per chunk
+    (3, 1, 9, 11, 40, 5, 3, 1, 0),       # one channel, no padding, odd sizes
+    (2, 4, 12, 12, 70, 3, 8, 1, 4),      # four channels, the widest window
+    (1, 3, 13, 13, 32, 1, 1, 2, 0),      # 1x1, strided
+    (2, 2, 8, 30, 24, 4, 2, 3, 1),       # stride 3, asymmetric filter
+]
+
+
+@pytest.mark.parametrize("case", STEM_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%dx%ds%dp%d" % c)
+def test_conv2d_stem_i8(case, dev):
+    """Row-window convolution of the few-channel input layer against the oracle's conv2d + chain."""
+    n, c, h, w, oc, kh, kw, st, pd = case
+    cid = "stem-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, c, kh, kw), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1)
+    stages = [("relu",), ("cvm_right_shift", 8, 9)]
+    out32 = hipops.conv2d_stem_i8(T(x, dev), T(wt, dev), T(b, dev), None, False, (st, st), (pd, pd))
+    torch.cuda.synchronize()
+    eq(out32.cpu().numpy(), conv, "stem int32")
+    out8 = hipops.conv2d_stem_i8(T(x, dev), T(wt, dev), T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
+    eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), run_chain(conv, stages), "stem int8")
+
+
 @pytest.mark.parametrize("cfg", range(7))
 @pytest.mark.parametrize("case", [(3, 96, 11, 13, 100, 3, 1, 1, True), (2, 256, 9, 9, 72, 1, 2, 0, False),
                                   (1, 64, 8, 8, 40, 3, 2, 1, True)],
