@@ -115,3 +115,31 @@ def test_argmax_and_detection_postprocess(dev):
     logits = og.run_graph(js, graphgen.load_params(pb), x)[0].ravel()
     # the reference compares the logits as int8 (src/core/model.cc:193)
     assert out[0] == int(np.argmax(logits.astype(np.int8)))
+
+
+def test_graph_replay_equals_eager_on_every_replay(dev):
+    """After its first run a model replays a captured graph.  Every replay -- with fresh inputs, other
+    GPU work and synchronisations in between -- must equal the eager, launch-by-launch result."""
+    import os
+    import torch
+    g, heads = graphgen.resnet50(2, width=16, size=64, classes=50, config_id="replay-r50")
+    js, pb = g.build(heads)
+    xs = [synth.tensor("replay", "data%d" % i, (2, 3, 64, 64), -127, 127).astype(np.int8) for i in range(6)]
+    os.environ["CVM_HIP_GRAPH"] = "0"
+    try:
+        eager = runtime.HipModel(js, pb)
+        want = [eager.inference(x.tobytes()) for x in xs]
+        eager.close()
+    finally:
+        os.environ.pop("CVM_HIP_GRAPH", None)
+    m = runtime.HipModel(js, pb)
+    scratch = torch.zeros(1 << 20, device=dev)
+    for rnd in range(2):
+        for i, x in enumerate(xs):        # run 1 is eager, run 2 captures, the rest replay
+            got = m.inference(x.tobytes())
+            assert got == want[i], "replay %d of round %d differs from the eager result" % (i, rnd)
+            scratch.add_(1.0)             # unrelated eager work between replays
+            torch.cuda.synchronize()
+    m.close()
+    ref = og.run_graph(js, graphgen.load_params(pb), xs[3].astype(np.int32))
+    assert np.array_equal(np.frombuffer(want[3], np.int32), np.concatenate([r.ravel() for r in ref]))
