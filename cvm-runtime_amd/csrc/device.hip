@@ -201,21 +201,6 @@ int cvmhip_capture_end(void* stream, void** graph_exec) {
   return CVMHIP_OK;
 }
 
-// An event recorded on `from` and waited for on `to`: inside a capture this is
-// how a second stream joins the graph (and how it is joined back).
-int cvmhip_stream_fork(void* from, void* to) {
-  hipEvent_t ev;
-  HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate");
-  hipError_t e = hipEventRecord(ev, as_stream(from));
-  if (e == hipSuccess) e = hipStreamWaitEvent(as_stream(to), ev, 0);
-  hipEventDestroy(ev);   // released once the work that references it has been captured or completed
-  if (e != hipSuccess) {
-    set_error("stream fork: %s", hipGetErrorString(e));
-    return CVMHIP_ERR_RUNTIME;
-  }
-  return CVMHIP_OK;
-}
-
 int cvmhip_graph_launch(void* graph_exec, void* stream) {
   HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream)), "hipGraphLaunch");
   return CVMHIP_OK;

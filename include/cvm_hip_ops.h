@@ -178,13 +178,10 @@ int cvmhip_kernel_timing_active(void);   /* 1 between begin and end */
 
 /* ---- stream capture: the launches issued on `stream` between begin and end
  * become one executable graph that replays them with a single submission
- * (hipStreamBeginCapture / hipGraphInstantiate / hipGraphLaunch).  A second
- * stream joins a capture with cvmhip_stream_fork (its later work depends on
- * what `from` has captured so far) and must be joined back before end.
+ * (hipStreamBeginCapture / hipGraphInstantiate / hipGraphLaunch).
  * No counterpart in the reference: its GPU runtime launches node by node. */
 int cvmhip_capture_begin(void* stream);
 int cvmhip_capture_end(void* stream, void** graph_exec);
-int cvmhip_stream_fork(void* from, void* to);   /* `to` waits for everything issued on `from` so far */
 int cvmhip_graph_launch(void* graph_exec, void* stream);
 int cvmhip_graph_destroy(void* graph_exec);
 
