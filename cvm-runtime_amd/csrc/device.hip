@@ -79,6 +79,34 @@ int cvmhip_memset32(void* ptr, int32_t value, size_t count, void* stream) {
   return check_launch("memset32");
 }
 
+int cvmhip_host_alloc(void** ptr, size_t bytes) {
+  if (!ptr) return arg_error("host_alloc");
+  HIP_TRY(hipHostMalloc(ptr, bytes ? bytes : 256, hipHostMallocDefault), "hipHostMalloc");
+  return CVMHIP_OK;
+}
+
+int cvmhip_host_free(void* ptr) {
+  if (ptr) HIP_TRY(hipHostFree(ptr), "hipHostFree");
+  return CVMHIP_OK;
+}
+
+// int8 -> int32 with the input clamp of the graph runtime (graph_runtime.cc:345-352)
+__global__ void __launch_bounds__(256) k_widen_clamp(const int8_t* __restrict__ src, int32_t* __restrict__ dst, int64_t count,
+                                                     int32_t range) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+    const int32_t v = src[i];
+    dst[i] = v > range ? range : (v < -range ? -range : v);
+  }
+}
+
+int cvmhip_widen_clamp_i8(const void* src, int32_t* dst, int64_t count, int32_t range, void* stream) {
+  if (!src || !dst || count < 0 || range < 0) return arg_error("widen_clamp_i8");
+  if (count == 0) return CVMHIP_OK;
+  k_widen_clamp<<<grid_for(count, 256), 256, 0, as_stream(stream)>>>(reinterpret_cast<const int8_t*>(src), dst, count, range);
+  return check_launch("widen_clamp_i8");
+}
+
 int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
   if (bytes == 0) return CVMHIP_OK;
   HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)), "copy_h2d");

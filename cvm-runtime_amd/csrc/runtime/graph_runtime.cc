@@ -445,6 +445,8 @@ void HipGraphRuntime::Release() {
   plan_.clear();
   execs_.clear();  // releases per-node device state before the stream goes away
   if (i8_slab_) { cvmhip_free(i8_slab_); i8_slab_ = nullptr; }
+  if (in_stage_dev_) { cvmhip_free(in_stage_dev_); in_stage_dev_ = nullptr; }
+  if (in_stage_host_) { cvmhip_host_free(in_stage_host_); in_stage_host_ = nullptr; }
   if (stream_) cvmhip_stream_sync(stream_);
   if (workspace_) cvmhip_free(workspace_);
   if (slab_) cvmhip_free(slab_);
@@ -484,6 +486,31 @@ void HipGraphRuntime::SetInput(uint32_t input_index, const int32_t* data32, cons
   }
   HipCheck(cvmhip_copy_h2d(entry_ptr_[eid], staged.data(), static_cast<size_t>(size) * 4, stream_), "copy input to device");
   HipCheck(cvmhip_stream_sync(stream_), "copy input to device");  // `staged` dies here
+}
+
+// `data` given as int8 bytes: staged through pinned memory, widened and clamped on the device.
+// Same result as SetData on the widened values; a quarter of the bytes cross the bus and the
+// host does one memcpy.
+void HipGraphRuntime::SetDataI8(const int8_t* host, const Shape& shape) {
+  const int idx = GetInputIndex("data");
+  const uint32_t nid = input_nodes_[idx];
+  CVM_VERIFY(nodes_[nid].is_data()) << "set input must named `data`";
+  const uint32_t eid = entry_id(nid, 0);
+  const Shape& expected = shape_[eid];
+  CVM_VERIFY(shape.size() == expected.size()) << "Loaded data shape ndim " << shape.size() << " not matched " << expected.size();
+  for (size_t i = 0; i < shape.size(); ++i)
+    CVM_VERIFY(shape[i] == expected[i]) << "Loaded data shape at index " << i << " with value " << shape[i] << ", Expected " << expected[i];
+  const size_t size = static_cast<size_t>(shape_size(shape));
+  const int prec = precision_[eid];
+  const int32_t range = static_cast<int32_t>((static_cast<uint32_t>(1) << (prec - 1)) - 1);
+  if (!in_stage_host_) {
+    HipCheck(cvmhip_host_alloc(&in_stage_host_, size), "input staging buffer");
+    HipCheck(cvmhip_alloc(&in_stage_dev_, size), "input staging buffer");
+  }
+  HipCheck(cvmhip_stream_sync(stream_), "copy input to device");  // the previous copy out of the staging buffer is done
+  std::memcpy(in_stage_host_, host, size);
+  HipCheck(cvmhip_copy_h2d(in_stage_dev_, in_stage_host_, size, stream_), "copy input to device");
+  HipCheck(cvmhip_widen_clamp_i8(in_stage_dev_, entry_ptr_[eid], static_cast<int64_t>(size), range, stream_), "widen input");
 }
 
 void HipGraphRuntime::SetData(const int32_t* host, const Shape& shape) {

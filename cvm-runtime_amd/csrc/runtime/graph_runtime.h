@@ -114,6 +114,7 @@ class HipGraphRuntime {
   void LoadParams(const std::string& blob);
   // `data` tensor from host memory: int32 values, already widened
   void SetData(const int32_t* host, const Shape& shape);
+  void SetDataI8(const int8_t* host, const Shape& shape);   // the same for an input given as int8 bytes
   void Run();      // replays the captured graph once it exists
   void Launch();   // issues every launch of a run on the stream, one by one
   void CopyOutputTo(int index, int32_t* host);  // synchronises the stream
@@ -175,6 +176,8 @@ class HipGraphRuntime {
   void* workspace_ = nullptr;  // shared operator scratch
   size_t workspace_bytes_ = 0;
   void* stream_ = nullptr;
+  void* in_stage_host_ = nullptr;  // pinned staging copy of an int8 input
+  void* in_stage_dev_ = nullptr;   // its device copy before widening
   std::vector<int32_t*> entry_ptr_;
   struct Exec { uint32_t nid; const OpKernel* kernel; OpCall call; };
   std::vector<Exec> execs_;

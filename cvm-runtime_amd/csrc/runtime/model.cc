@@ -51,14 +51,11 @@ int HipModel::GetOutputLength() const {
 // model.cc:154-169 + 284-291
 void HipModel::SetInput(const void* input, int size) {
   CVM_VERIFY(GetInputLength() == size);
-  std::vector<int32_t> wide(static_cast<size_t>(in_size_));
   if (input_bytes_ == 4) {
-    std::memcpy(wide.data(), input, wide.size() * 4);
+    rt_->SetData(static_cast<const int32_t*>(input), in_shape_);
   } else {
-    const int8_t* p = static_cast<const int8_t*>(input);
-    for (int64_t i = 0; i < in_size_; ++i) wide[i] = p[i];
+    rt_->SetDataI8(static_cast<const int8_t*>(input), in_shape_);   // widened on the device
   }
-  rt_->SetData(wide.data(), in_shape_);
 }
 
 void HipModel::GetOutput(char* mem) {

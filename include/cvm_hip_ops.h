@@ -156,6 +156,11 @@ int cvmhip_set_device(int device_id);
 int cvmhip_alloc(void** ptr, size_t bytes);
 int cvmhip_free(void* ptr);
 int cvmhip_memset32(void* ptr, int32_t value, size_t count, void* stream);
+int cvmhip_host_alloc(void** ptr, size_t bytes);   /* pinned host memory for staging copies */
+int cvmhip_host_free(void* ptr);
+/* int8 bytes already on the device -> the int32 `data` tensor, clamped to [-range, range]: the input
+ * path of CvmRuntime::SetInput (src/runtime/graph_runtime.cc:317-397) without widening on the host */
+int cvmhip_widen_clamp_i8(const void* src, int32_t* dst, int64_t count, int32_t range, void* stream);
 int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream);
 int cvmhip_copy_d2h(void* dst, const void* src, size_t bytes, void* stream);
 int cvmhip_copy_d2d(void* dst, const void* src, size_t bytes, void* stream);

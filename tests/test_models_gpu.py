@@ -143,3 +143,16 @@ def test_graph_replay_equals_eager_on_every_replay(dev):
     m.close()
     ref = og.run_graph(js, graphgen.load_params(pb), xs[3].astype(np.int32))
     assert np.array_equal(np.frombuffer(want[3], np.int32), np.concatenate([r.ravel() for r in ref]))
+
+
+def test_int8_input_is_clamped_like_the_reference(dev):
+    """CvmRuntime::SetInput clamps `data` to +-(2^(p-1)-1) (graph_runtime.cc:345-352): the byte -128 runs as -127."""
+    g, heads = graphgen.conv_op_graph(n=1, c=64, h=8, w=8, oc=64)
+    js, pb = g.build(heads)
+    x = synth.tensor("clamp", "data", (1, 64, 8, 8), -128, 127)
+    x[0, :, 0, 0] = -128
+    m = runtime.HipModel(js, pb)
+    out = np.frombuffer(m.inference(x.astype(np.int8).tobytes()), np.int8).astype(np.int32)
+    m.close()
+    ref = og.run_graph(js, graphgen.load_params(pb), np.clip(x, -127, 127))
+    assert np.array_equal(out, ref[0].ravel())
