@@ -159,57 +159,102 @@ k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_coun
   if (i < vc && r) atomicAdd(&rank[(int64_t)b * n + i], r);
 }
 
-// row i moves to its sorted slot
+// Row i moves to its sorted slot; rows ranked at or past top_k are then overwritten with -1 in the input
+// tensor (nms.cc:92-96).  Every output row starts as -1: k_nms_select writes the kept rows over the front.
 __global__ void __launch_bounds__(256)
-k_nms_scatter(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, const int32_t* __restrict__ rank,
-              int32_t* __restrict__ order, int32_t* __restrict__ sorted, int n, int k, int64_t ws_stride) {
+k_nms_scatter(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, const int32_t* __restrict__ rank,
+              int32_t* __restrict__ order, int32_t* __restrict__ sorted, int32_t* __restrict__ y, int n, int k,
+              int topk, int64_t ws_stride) {
   const int b = blockIdx.y;
-  if (batch_state(valid_count, b, n) != 0) return;
-  const int vc = clamp_vc(valid_count[b], n);
+  const int state = batch_state(valid_count, b, n);
+  if (state == 2) return;
   const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  int32_t* yrow = y + ((int64_t)b * n + i) * k;
+  for (int c = 0; c < k; ++c) yrow[c] = -1;
+  if (state == 1) return;
+  const int vc = clamp_vc(valid_count[b], n);
   if (i >= vc) return;
-  const int32_t* xb = x + (int64_t)b * n * k;
+  int32_t* xrow = x + ((int64_t)b * n + i) * k;
   const int r = rank[(int64_t)b * n + i];
   order[b * ws_stride + r] = i;
   int32_t* dst = sorted + b * ws_stride * k + (int64_t)r * k;
-  for (int c = 0; c < k; ++c) dst[c] = xb[(int64_t)i * k + c];
+  for (int c = 0; c < k; ++c) dst[c] = xrow[c];
+  if (topk > 0 && r >= topk)
+    for (int c = 0; c < k; ++c) xrow[c] = -1;
+}
+
+constexpr int NMS_BM_ROWS = 512, NMS_BM_WORDS = 16;  // rows of the suppression bit matrix and its words per row
+
+// Suppression bit matrix for the first `keep` sorted rows, when they are few enough: bit j of row i says
+// that row i, if it survives, removes row j (j > i, matching id unless forced, overlap at the threshold).
+// One wavefront per (row, 64 candidates); the ballot is the two mask words.
+__global__ void __launch_bounds__(256)
+k_nms_mask(const int32_t* __restrict__ valid_count, const int32_t* __restrict__ sorted, uint32_t* __restrict__ mask,
+           int n, int k, int iou_threshold, int topk, int coord_start, int id_index, int force_suppress,
+           int64_t ws_stride) {
+  const int b = blockIdx.z;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  const int keep = (topk >= 0 && topk < vc) ? topk : vc;
+  if (keep > NMS_BM_ROWS) return;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (i >= keep) return;
+  const int j = blockIdx.y * 64 + lane;
+  const int32_t* srt = sorted + b * ws_stride * k;
+  bool hit = false;
+  if (j > i && j < keep) {
+    const int32_t* r1 = srt + (int64_t)i * k;
+    const int32_t* r2 = srt + (int64_t)j * k;
+    if (force_suppress || id_index < 0 || r1[id_index] == r2[id_index])
+      hit = iou_at_least(r1 + coord_start, r2 + coord_start, iou_threshold);
+  }
+  const unsigned long long bits = __ballot(hit);
+  if (lane == 0) {
+    uint32_t* m = mask + ((int64_t)b * NMS_BM_ROWS + i) * NMS_BM_WORDS + blockIdx.y * 2;
+    m[0] = (uint32_t)bits;
+    m[1] = (uint32_t)(bits >> 32);
+  }
 }
 
 constexpr int NMS_THREADS = 1024;
-constexpr int NMS_LDS_ROWS = 2048, NMS_LDS_K = 6;  // rows x columns of the LDS copy in k_nms_select (48 KiB)
+constexpr int NMS_LDS_ROWS = 1024, NMS_LDS_K = 6;  // rows x columns of the LDS copy in k_nms_select (24 KiB)
 
 // One workgroup per batch walks the sorted rows in order.  Row i is emitted if
 // it survived and has id >= 0; a surviving row then suppresses, in parallel,
 // the rows after it up to (not including) the first row with a negative id.
 __global__ void __launch_bounds__(NMS_THREADS)
-k_nms_select(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ y,
-             const int32_t* __restrict__ order, const int32_t* __restrict__ sorted, int32_t* __restrict__ nextneg,
-             int32_t* __restrict__ removed, int n, int k, int max_output_size, int iou_threshold, int topk,
-             int coord_start, int id_index, int force_suppress, int64_t ws_stride) {
+k_nms_select(const int32_t* __restrict__ valid_count, int32_t* __restrict__ y,
+             const int32_t* __restrict__ sorted, int32_t* __restrict__ nextneg,
+             int32_t* __restrict__ removed, const uint32_t* __restrict__ mask, int n, int k, int max_output_size,
+             int iou_threshold, int topk, int coord_start, int id_index, int force_suppress, int64_t ws_stride) {
   __shared__ int s_wmin[NMS_THREADS / 64];
   __shared__ int s_carry;
   const int b = blockIdx.x, tid = threadIdx.x;
   const int state = batch_state(valid_count, b, n);
   if (state == 2) return;
+  if (state == 1) return;  // k_nms_scatter has already filled the output with -1
   int32_t* yb = y + (int64_t)b * n * k;
-  if (state == 1) {
-    for (int64_t i = tid; i < (int64_t)n * k; i += NMS_THREADS) yb[i] = -1;
-    return;
-  }
   const int vc = clamp_vc(valid_count[b], n);
-  int32_t* xb = x + (int64_t)b * n * k;
-  const int32_t* ord = order + b * ws_stride;
   const int32_t* srt = sorted + b * ws_stride * k;
   int32_t* nn = nextneg + b * (ws_stride + 1);
   int32_t* rem = removed + b * ws_stride;
   const int keep = (topk >= 0 && topk < vc) ? topk : vc;
 
-  // rows past top_k are overwritten with -1 in the input tensor (nms.cc:92-96)
-  if (topk > 0 && topk < vc)
-    for (int64_t i = tid; i < (int64_t)(vc - topk) * k; i += NMS_THREADS) {
-      const int r = topk + (int)(i / k);
-      xb[(int64_t)ord[r] * k + (i % k)] = -1;
-    }
+  // The greedy walk is a chain of dependent steps: when the candidate rows fit (top_k bounds them in
+  // practice) they, the cut points and the removal flags live in LDS, whose latency is a tenth of HBM's.
+  __shared__ int32_t s_rows[NMS_LDS_ROWS * NMS_LDS_K];
+  __shared__ int32_t s_nn[NMS_LDS_ROWS + 1];
+  __shared__ uint32_t s_mask[NMS_BM_ROWS * NMS_BM_WORDS];  // the loop path keeps its removal flags here instead
+  static_assert(NMS_BM_ROWS * NMS_BM_WORDS >= NMS_LDS_ROWS, "removal flags share the bit matrix's storage");
+  const bool staged = keep <= NMS_LDS_ROWS && k <= NMS_LDS_K;
+  if (staged) {
+    for (int i = tid; i < keep * k; i += NMS_THREADS) s_rows[i] = srt[i];
+    srt = s_rows;
+    rem = reinterpret_cast<int32_t*>(s_mask);
+    nn = s_nn;
+    __syncthreads();
+  }
 
   // nn[j] = smallest j' >= j with a negative id (keep if none): suffix minimum,
   // computed chunk by chunk from the back.
@@ -236,22 +281,73 @@ k_nms_select(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, i
     __syncthreads();
   }
 
-  // The greedy walk is a chain of dependent steps, each a barrier plus a few
-  // reads: when the candidate rows fit (top_k bounds them in practice) they and
-  // the removal flags are staged in LDS, whose latency is a tenth of HBM's.
-  __shared__ int32_t s_rows[NMS_LDS_ROWS * NMS_LDS_K];
-  __shared__ int32_t s_rem[NMS_LDS_ROWS];
-  __shared__ int32_t s_nn[NMS_LDS_ROWS + 1];
-  if (keep <= NMS_LDS_ROWS && k <= NMS_LDS_K) {
-    for (int i = tid; i < keep * k; i += NMS_THREADS) s_rows[i] = srt[i];
-    for (int i = tid; i < keep; i += NMS_THREADS) s_rem[i] = 0;
-    for (int i = tid; i <= keep; i += NMS_THREADS) s_nn[i] = nn[i];
-    srt = s_rows;
-    rem = s_rem;
-    nn = s_nn;
-  }
-
   int yi = 0;
+  // With few enough rows k_nms_mask has tested every pair up front, and the walk only has to find the set
+  // of removed rows: a row is removed by rows before it only, so whether it acts is known when the walk
+  // reaches it.  One wavefront holds the set in registers (lane l: bits 32l..32l+31, repeated every 16
+  // lanes) and ORs in the matrix row of each row that is still there, cut at the first later row with a
+  // negative id.  The rows emitted are then the surviving ones whose id is not negative, in order.  Same
+  // decisions as the loop below.
+  __shared__ uint32_t s_pos[NMS_BM_WORDS], s_emit[NMS_BM_WORDS];
+  __shared__ int s_before[NMS_BM_WORDS], s_yi;
+  if (staged && keep <= NMS_BM_ROWS) {
+    const uint32_t* mb = mask + (int64_t)b * NMS_BM_ROWS * NMS_BM_WORDS;
+    for (int t = tid; t < keep * NMS_BM_WORDS; t += NMS_THREADS) {
+      const int live = s_nn[(t / NMS_BM_WORDS) + 1] - (t % NMS_BM_WORDS) * 32;  // bits of this word below the cut
+      s_mask[t] = mb[t] & (live >= 32 ? 0xffffffffu : live <= 0 ? 0u : (1u << live) - 1u);
+    }
+    if (tid < NMS_BM_ROWS) {
+      const unsigned long long pos = __ballot(tid < keep && s_rows[tid * k] >= 0);
+      if ((tid & 63) == 0) {
+        s_pos[tid >> 5] = (uint32_t)pos;
+        s_pos[(tid >> 5) + 1] = (uint32_t)(pos >> 32);
+      }
+    }
+    __syncthreads();
+    if (tid < 64) {
+      const int l16 = tid & (NMS_BM_WORDS - 1);
+      uint32_t remw = 0, cur[4], nxt[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) cur[u] = s_mask[u * NMS_BM_WORDS + l16];
+      for (int i = 0; i < keep; i += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {  // the next four matrix rows are on their way while these four are decided
+          const int r = i + 4 + u < NMS_BM_ROWS ? i + 4 + u : NMS_BM_ROWS - 1;
+          nxt[u] = s_mask[r * NMS_BM_WORDS + l16];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int r = i + u;
+          const uint32_t word = (uint32_t)__builtin_amdgcn_readlane((int)remw, r >> 5);
+          if (r < keep && !((word >> (r & 31)) & 1u)) remw |= cur[u];
+          cur[u] = nxt[u];
+        }
+      }
+      const int live = keep - l16 * 32;
+      const uint32_t e = ~remw & s_pos[l16] & (live >= 32 ? 0xffffffffu : live <= 0 ? 0u : (1u << live) - 1u);
+      const int c = __popc(e);
+      int p = c;  // inclusive prefix over the 16 words
+      for (int d = 1; d < NMS_BM_WORDS; d <<= 1) {
+        const int o = __shfl_up(p, d, NMS_BM_WORDS);
+        if (l16 >= d) p += o;
+      }
+      if (tid < NMS_BM_WORDS) { s_emit[tid] = e; s_before[tid] = p - c; }
+      if (tid == NMS_BM_WORDS - 1) s_yi = p;
+    }
+    __syncthreads();
+    yi = s_yi;
+    // max_output_size keeps the first `max_output_size` emitted rows (nms.cc:126-137)
+    if (max_output_size > 0 && yi > max_output_size) yi = max_output_size;
+    if (tid < NMS_BM_ROWS) {
+      const uint32_t e = s_emit[tid >> 5];
+      if ((e >> (tid & 31)) & 1u) {
+        const int at = s_before[tid >> 5] + __popc(e & ((1u << (tid & 31)) - 1u));
+        if (at < yi)
+          for (int c = 0; c < k; ++c) yb[(int64_t)at * k + c] = s_rows[tid * k + c];
+      }
+    }
+    return;
+  }
   for (int i = 0; i < keep; ++i) {
     __syncthreads();  // removals from the previous row (and the staging above) are visible
     if (rem[i]) continue;
@@ -303,9 +399,9 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
   return check_launch("get_valid_counts.scatter");
 }
 
-// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n]
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
-  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 1) * sizeof(int32_t);
+  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 1 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS) * sizeof(int32_t);
 }
 
 int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
@@ -313,7 +409,8 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
                                int iou_threshold, int topk, int coord_start,
                                int score_index, int id_index, int force_suppress,
                                void* workspace, size_t workspace_bytes, void* stream) {
-  if (!x || !valid_count || !y || batches < 1 || n < 1 || k < 2 || batches > 65535) return arg_error("non_max_suppression");
+  if (!x || !valid_count || !y || x == y || batches < 1 || n < 1 || k < 2 || batches > 65535)
+    return arg_error("non_max_suppression");
   if (iou_threshold <= 0) return arg_error("non_max_suppression.iou_threshold must be positive");
   if (coord_start < 0 || coord_start + 4 > k || score_index < 0 || score_index >= k || id_index >= k)
     return arg_error("non_max_suppression indices");
@@ -331,10 +428,20 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
   int rc = check_launch("nms.rank");
   if (rc) return rc;
   dim3 grid((n + 255) / 256, batches);
-  k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, n, k, (int64_t)n);
+  k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, y, n, k, topk, (int64_t)n);
   rc = check_launch("nms.scatter");
   if (rc) return rc;
-  k_nms_select<<<batches, NMS_THREADS, 0, s>>>(x, valid_count, y, order, sorted, nextneg, removed, n, k,
+  uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
+  int rows = n < NMS_BM_ROWS ? n : NMS_BM_ROWS;  // upper bound of the rows the walk can see, when the matrix is used
+  if (topk >= 0 && topk < rows) rows = topk;
+  if (rows > 0 && k <= NMS_LDS_K) {
+    dim3 mgrid((rows + 3) / 4, (rows + 63) / 64, batches);
+    k_nms_mask<<<mgrid, 256, 0, s>>>(valid_count, sorted, mask, n, k, iou_threshold, topk, coord_start, id_index,
+                                     force_suppress, (int64_t)n);
+    rc = check_launch("nms.mask");
+    if (rc) return rc;
+  }
+  k_nms_select<<<batches, NMS_THREADS, 0, s>>>(valid_count, y, sorted, nextneg, removed, mask, n, k,
                                                max_output_size, iou_threshold, topk, coord_start, id_index,
                                                force_suppress, (int64_t)n);
   return check_launch("nms.select");

@@ -271,6 +271,10 @@ NMS_CASES = [
     (1, 2000, -1, 45, -1, 100, False, 128),
     (2, 50, 0, 45, 0, -1, False, 64),          # top_k == 0 keeps nothing
     (1, 1, 0, 45, -1, -1, False, 64),
+    (1, 4000, -1, 45, -1, -1, False, 256),     # more candidate rows than the kernel stages on chip
+    (1, 3000, -1, 45, 512, -1, False, 128),    # the largest top_k that takes the bit-matrix walk
+    (2, 3000, -1, 45, 513, 200, False, 128),   # one more: the row-by-row walk
+    (2, 700, 0, 45, 65, -1, True, 48),         # top_k straddling a 64-row ballot
 ]
 
 
