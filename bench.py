@@ -20,6 +20,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
+# HBM bytes per k_conv_wave launch of the batch-16 workload, from the FETCH_SIZE and WRITE_SIZE counter
+# passes summarised in profiles/k_conv_wave_resnet50_b16_traffic.txt (a counter pass cannot run inside
+# this program, so the figure is carried here; it is reported only for the workload it was measured on)
+TRAFFIC_BYTES_PER_LAUNCH = {("k_conv_wave", 16): 12.91e6}
 
 
 def cpu_baseline(js1, pb1, budget_s=20.0):
@@ -48,7 +52,7 @@ def cpu_baseline(js1, pb1, budget_s=20.0):
             L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out)
             n += 1
             dt = time.perf_counter() - t0
-            if dt > budget_s or n >= 64:
+            if dt > budget_s or n >= 1000:
                 break
         L.CVMAPIFreeModel(net)
         kind = "reference"
@@ -60,7 +64,7 @@ def cpu_baseline(js1, pb1, budget_s=20.0):
             og.run_graph(js1, params, x)
             n += 1
             dt = time.perf_counter() - t0
-            if dt > budget_s or n >= 64:
+            if dt > budget_s or n >= 1000:
                 break
         kind = "port"
     return {"value": n / dt, "unit": "images/s", "cores": cores, "kind": kind,
@@ -74,6 +78,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also launch a plain copy kernel of known size (256 MiB read + 256 MiB written, 5 times): "
+                         "under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counter reading gives the scale of the counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on exactly one GPU (got --gpus %d); the path shards by batch "
@@ -126,6 +133,14 @@ def main():
     api_s = (time.perf_counter() - t0) / n_api
     model.close()
 
+    if args.traffic_calibration:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            pkg.check(L.cvmhip_copy_kernel(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()),
+                                           ctypes.c_size_t(a.numel()), None))
+        torch.cuda.synchronize()
+
     # The two implicit-GEMM kernels (same arithmetic, chosen per layer); the roofline object is about the
     # one that takes more of the step.  An event pair makes a launch look longer than it is.  Every launch
     # of a step is timed and the un-instrumented step is GPU-bound with its kernels back to back, so the
@@ -165,7 +180,8 @@ def main():
                    "images_per_s_through_CVMAPIInference": args.batch / api_s,
                    "output_checksum": int(np.bitwise_xor.reduce(out.view(np.uint32)))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_I8_TOPS, "unit": "TOP/s",
-                     "frac": achieved / PEAK_I8_TOPS, "traffic": None,
+                     "frac": achieved / PEAK_I8_TOPS,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((dom, args.batch)), "traffic_unit": "bytes per launch",
                      "kernel": dom, "launches_per_step": conv["launches"] / args.steps,
                      "avg_launch_us": avg_s * 1e6, "avg_launch_us_with_event_pair": raw_avg_s * 1e6,
                      "event_pair_cost_us": pair_cost_us, "algorithmic_gop_per_launch": ops_per_launch / 1e9,

@@ -107,6 +107,22 @@ int cvmhip_widen_clamp_i8(const void* src, int32_t* dst, int64_t count, int32_t 
   return check_launch("widen_clamp_i8");
 }
 
+// plain 16-bytes-per-lane copy
+__global__ void __launch_bounds__(256) k_copy16(const int4* __restrict__ src, int4* __restrict__ dst, int64_t count) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) dst[i] = src[i];
+}
+
+int cvmhip_copy_kernel(void* dst, const void* src, size_t bytes, void* stream) {
+  if (!dst || !src || (bytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15)) return arg_error("copy_kernel: 16-byte granules");
+  if (bytes == 0 || dst == src) return CVMHIP_OK;
+  const int64_t count = (int64_t)(bytes / 16);
+  int64_t blocks = (count + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  k_copy16<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(reinterpret_cast<const int4*>(src), reinterpret_cast<int4*>(dst), count);
+  return check_launch("copy_kernel");
+}
+
 int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
   if (bytes == 0) return CVMHIP_OK;
   HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)), "copy_h2d");

@@ -164,6 +164,9 @@ int cvmhip_widen_clamp_i8(const void* src, int32_t* dst, int64_t count, int32_t 
 int cvmhip_copy_h2d(void* dst, const void* src, size_t bytes, void* stream);
 int cvmhip_copy_d2h(void* dst, const void* src, size_t bytes, void* stream);
 int cvmhip_copy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+/* device-to-device copy done by a compute kernel (16-byte granules) instead of the copy engine: a launch of
+ * exactly known HBM traffic, 2*bytes, against which hardware traffic counters can be scaled */
+int cvmhip_copy_kernel(void* dst, const void* src, size_t bytes, void* stream);
 int cvmhip_stream_create(void** stream);
 int cvmhip_stream_destroy(void* stream);
 int cvmhip_stream_sync(void* stream);
