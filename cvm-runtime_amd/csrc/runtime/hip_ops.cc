@@ -93,8 +93,11 @@ OpKernel DenseKernel() {
       Check(cvmhip_conv2d_packed(c.in[0].data, static_cast<DeviceBuffer*>(c.state.get())->ptr, bias, c.out[0].data,
                                  m, kk, 1, 1, n, 1, 1, 1, 1, 0, 0, 1, 1, c.workspace, c.workspace_bytes, c.stream), "dense");
     } else {
-      // operand precision <= 8 is guaranteed by DensePrec for every accepted graph
-      Check(cvmhip_dense(c.in[0].data, c.in[1].data, bias, c.out[0].data, m, kk, n, 8, c.workspace, c.workspace_bytes,
+      // DensePrec guarantees operand precision <= 8 for every accepted graph; a single-operator call
+      // declares what its tensors hold, and wider operands take the exact int32 path
+      const int p0 = c.in[0].precision, p1 = c.in[1].precision;
+      const int bits = (p0 < 1 || p1 < 1) ? 32 : (p0 > p1 ? p0 : p1);
+      Check(cvmhip_dense(c.in[0].data, c.in[1].data, bias, c.out[0].data, m, kk, n, bits, c.workspace, c.workspace_bytes,
                          c.stream), "dense");
     }
   };

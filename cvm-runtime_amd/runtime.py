@@ -169,3 +169,46 @@ def list_ops():
     buf = ctypes.create_string_buffer(1 << 14)
     _ck(lib().CVMHIPListOps(buf, len(buf)), "CVMHIPListOps")
     return buf.value.decode().split()
+
+
+def run_op(op, attrs, inputs, out_init=0, execute=True):
+    """One registered operator on host arrays (CVMHIPRunOp): what the reference's
+    tests/test_op.cc does per case.  Outputs start filled with `out_init`.
+    Returns (status, failed_stage, outputs, message); with execute=False only
+    attribute parsing and shape inference run (no GPU) and outputs are empty
+    arrays of the inferred shapes."""
+    import numpy as np
+    L = lib()
+    ins = [np.ascontiguousarray(v, dtype=np.int32) for v in inputs]
+    n = len(ins)
+    shp = (ctypes.c_longlong * (6 * max(n, 1)))()
+    nd = (ctypes.c_int * max(n, 1))()
+    ptrs = (ctypes.POINTER(ctypes.c_int) * max(n, 1))()
+    for i, v in enumerate(ins):
+        nd[i] = v.ndim
+        for d, s in enumerate(v.shape):
+            shp[6 * i + d] = s
+        ptrs[i] = v.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+    max_out = 4
+    oshp = (ctypes.c_longlong * (6 * max_out))()
+    ond = (ctypes.c_int * max_out)()
+    nout = ctypes.c_int()
+    stage = ctypes.c_int(-1)
+    err = ctypes.create_string_buffer(4096)
+    aj = json.dumps(attrs).encode()
+    rc = L.CVMHIPRunOp(op.encode(), aj, n, shp, nd, ptrs, max_out, ctypes.byref(nout), oshp, ond, None, None,
+                       ctypes.byref(stage), err, 4096)
+    if rc != 0:
+        return rc, stage.value, [], err.value.decode(errors="replace")
+    shapes = [tuple(oshp[6 * i + d] for d in range(ond[i])) for i in range(nout.value)]
+    outs = [np.full(s, out_init, np.int32) for s in shapes]
+    if not execute:
+        return 0, -1, outs, ""
+    optrs = (ctypes.POINTER(ctypes.c_int) * max_out)()
+    cap = (ctypes.c_longlong * max_out)()
+    for i, o in enumerate(outs):
+        optrs[i] = o.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+        cap[i] = o.size
+    rc = L.CVMHIPRunOp(op.encode(), aj, n, shp, nd, ptrs, max_out, ctypes.byref(nout), oshp, ond, optrs, cap,
+                       ctypes.byref(stage), err, 4096)
+    return rc, (stage.value if rc else -1), outs, err.value.decode(errors="replace")

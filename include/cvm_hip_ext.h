@@ -33,6 +33,20 @@ int CVMHIPInferNode(const char* op, const char* attr_json, int n_in,
                     const long long* in_shapes, const int* in_ndims, const int* in_precs,
                     int* n_out, long long* out_shapes, int* out_ndims, int* out_precs,
                     char* err, int errlen);
+/* ONE registered operator on host tensors: the single-operator call that the reference's own operator
+ * test makes for each case directory (tests/test_op.cc:479-660: parse the attributes, FInferShape,
+ * allocate, copy in, call cvm.runtime.<dev>.<op> with its extra space, copy out).  int32 tensors, shapes
+ * as rows of 6 int64.  Outputs are first filled from the caller's buffers (some operators leave part of
+ * an output untouched), `out_capacity[i]` is the room of `out_data[i]` in elements.  With
+ * `out_data == NULL` only the attributes are parsed and the output shapes inferred (no device needed).
+ * `*failed_stage` tells what a non-zero status came from: 0 = attributes / shape inference (the failure
+ * a case directory announces in err.txt), 1 = execution.  Returns SUCCEED / ERROR_LOGIC / ERROR_RUNTIME
+ * with the message in err. */
+int CVMHIPRunOp(const char* op, const char* attr_json, int n_in,
+                const long long* in_shapes, const int* in_ndims, const int* const* in_data,
+                int max_out, int* n_out, long long* out_shapes, int* out_ndims,
+                int* const* out_data, const long long* out_capacity,
+                int* failed_stage, char* err, int errlen);
 /* Newline-separated names registered for the device: cvm.runtime.hip.<op> */
 int CVMHIPListOps(char* out, int capacity);
 

@@ -538,9 +538,9 @@ def ref_run_op(op, attrs, ins, outs, dev="cpu"):
     return rc, err.value.decode(errors="replace")
 
 
-def ref_infer(op, attrs, in_shapes, in_precs):
-    """Reference FInferShape + FInferPrecision for one node.
-    Returns (status, out_shapes, out_precs, message)."""
+def ref_infer(op, attrs, in_shapes, in_precs=None):
+    """Reference FInferShape + FInferPrecision for one node (shapes only when
+    `in_precs` is None).  Returns (status, out_shapes, out_precs, message)."""
     n = len(in_shapes)
     ins = (_RefTensor * max(n, 1))()
     for i, s in enumerate(in_shapes):
@@ -548,7 +548,7 @@ def ref_infer(op, attrs, in_shapes, in_precs):
         for d, v in enumerate(s):
             ins[i].shape[d] = v
     outs = (_RefTensor * 4)()
-    ip = (ctypes.c_int * max(n, 1))(*in_precs)
+    ip = (ctypes.c_int * max(n, 1))(*in_precs) if in_precs is not None else None
     op_ = (ctypes.c_int * 4)()
     nout = ctypes.c_int(0)
     err = ctypes.create_string_buffer(4096)

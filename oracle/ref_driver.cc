@@ -94,6 +94,7 @@ int ref_op_call(const char* dev, const char* op, const char* attr_json,
 // Runs attr parsing + FInferShape + FInferPrecision for one node.
 // in: shapes + precisions of inputs; out: shapes (filled) + precisions (filled).
 // *n_out receives the operator's output count.  Same status codes as above.
+// in_prec == NULL: attribute parsing and FInferShape only.
 int ref_op_infer(const char* op, const char* attr_json, int n_in,
                  const RefTensor* in, const int* in_prec, int max_out,
                  int* n_out, RefTensor* out, int* out_prec, char* err,
@@ -119,6 +120,7 @@ int ref_op_infer(const char* op, const char* attr_json, int n_in,
       for (int d = 0; d < (int)oshape[i].ndim() && d < 6; ++d) out[i].shape[d] = oshape[i][d];
       shapes.push_back(oshape[i]);
     }
+    if (in_prec == nullptr) return 0;  // shapes only, as tests/test_op.cc:522-556 does before it runs a case
     std::vector<int> ip(in_prec, in_prec + n_in), opv(nout, -1);
     auto fp = fprec.get(attrs.op, nullptr);
     if (fp == nullptr) return fail(err, errlen, "no FInferPrecision", 2);
