@@ -78,6 +78,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--suite", choices=("model", "ops"), default="model",
+                    help="model: the headline line (default); ops: one JSON line per bandwidth-bound operator at the "
+                         "shapes of the configurations, achieved GB/s against the 8 TB/s HBM peak")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain copy kernel of known size (256 MiB read + 256 MiB written, 5 times): "
                          "under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counter reading gives the scale of the counters")
@@ -93,6 +96,12 @@ def main():
     from cvm_runtime_amd import graphgen, runtime, synth
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     L = pkg.lib()
+
+    if args.suite == "ops":
+        from cvm_runtime_amd import bench_ops
+        for row in bench_ops.run(max(args.steps, 5)):
+            print(json.dumps(row))
+        return
 
     g, heads = graphgen.resnet50(args.batch)
     js, pb = g.build(heads)

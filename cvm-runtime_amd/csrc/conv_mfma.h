@@ -55,6 +55,11 @@ struct Epilogue {
   DevChain chain2;
   int out_mode;            // OUT_I32_NCHW or OUT_I8_ACT
   int out_cp;              // padded channel count of the int8 output / residual (>= OC)
+  // int32 output: element (n, oc, pixel) goes to out[n*o32_img + oc*o32_ch + pixel*o32_px].  All zero
+  // (the default) means NCHW, filled in by conv_igemm; {stride, 1, OC} writes NHWC rows of image n at
+  // out + n*stride, e.g. straight into its slice of a concatenated tensor.
+  int64_t o32_img;
+  int o32_ch, o32_px;
 };
 
 // ---- int8 activation layout.  Channels are padded to Cp = 4, 8, 16 or a

@@ -181,10 +181,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int n = (int)fastdiv((unsigned)p, g.div_ohw);
       const int rem = p - n * OHW;
       const int oc = oc0 + ch[m];
-      int32_t* y32 = reinterpret_cast<int32_t*>(out) + ((int64_t)n * g.OC + oc) * OHW + rem;
+      int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * ep.o32_img + (int64_t)oc * ep.o32_ch + (int64_t)rem * ep.o32_px;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (oc + e < g.OC) y32[(int64_t)e * OHW] = val[m * 4 + e];
+        if (oc + e < g.OC) y32[(int64_t)e * ep.o32_ch] = val[m * 4 + e];
     }
     return;
   }
@@ -1046,6 +1046,13 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
   Epilogue ep = ep_in;
   ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
+  if (ep.o32_img == 0 && ep.o32_ch == 0 && ep.o32_px == 0) {  // int32 output defaults to NCHW
+    ep.o32_img = (int64_t)g.OC * g.OH * g.OW;
+    ep.o32_ch = g.OH * g.OW;
+    ep.o32_px = 1;
+  } else if (ep.o32_ch < 1 || ep.o32_px < 1 || ep.o32_img < 0) {
+    return arg_error("conv int32 output strides");
+  }
   const bool wide = (g.Kp % 128) == 0;
   const int gran = g.Cp >= 16 ? 16 : g.Cp;
   // Tile choice: the largest tile that still yields >= 2 workgroups per CU;

@@ -226,10 +226,10 @@ int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void
   return unpack_activations(reinterpret_cast<const int8_t*>(xp), x, n, c, hw, as_stream(stream));
 }
 
-int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
-                     const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
-                     int n, int ic, int h, int wd, int oc, int kh, int kw,
-                     int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                         const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8, int64_t nhwc_image_stride,
+                         int n, int ic, int h, int wd, int oc, int kh, int kw,
+                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
   if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
   if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
       pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
@@ -248,8 +248,30 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
   ep.residual = reinterpret_cast<const int8_t*>(residual);
   ep.out_mode = out_is_i8 ? OUT_I8_ACT : OUT_I32_NCHW;
   ep.out_cp = pad_channels(oc);
+  if (nhwc_image_stride >= 0) {
+    if (out_is_i8 || nhwc_image_stride < (int64_t)g.OH * g.OW * oc) return arg_error("conv2d_i8_nhwc image stride");
+    ep.o32_img = nhwc_image_stride;
+    ep.o32_ch = 1;
+    ep.o32_px = oc;
+  }
   return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep,
                     as_stream(stream));
+}
+
+int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                     const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
+                     int n, int ic, int h, int wd, int oc, int kh, int kw,
+                     int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, out_is_i8, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
+                       pad_h, pad_w, dil_h, dil_w, stream);
+}
+
+int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          int32_t* out, int64_t image_stride, int n, int ic, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  if (image_stride < 0) return arg_error("conv2d_i8_nhwc image stride");
+  return conv2d_i8_any(xp, wp, bias, chain, nullptr, nullptr, out, 0, image_stride, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
+                       pad_h, pad_w, dil_h, dil_w, stream);
 }
 
 // ---- row-window convolution over at most 4 input channels (the RGB stem of a network)

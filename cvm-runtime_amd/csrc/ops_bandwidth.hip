@@ -547,7 +547,7 @@ int cvmhip_concatenate(const int32_t* const* inputs, const int64_t* const* ishap
     const int64_t xrow = ishapes[m][axis] * inner;
     if (start + xrow > yrow) return arg_error("concatenate.shape");
     const int64_t n = outer * xrow;
-    if (n > 0) {
+    if (n > 0 && inputs[m] != nullptr) {  // a null input: that slice of y is already in place
       k_copy2d<<<grid_for(n, 256), 256, 0, as_stream(stream)>>>(inputs[m], y + start, outer, xrow, xrow, yrow);
       int rc = check_launch("concatenate");
       if (rc) return rc;

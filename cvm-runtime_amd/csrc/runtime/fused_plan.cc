@@ -14,11 +14,15 @@
 //   * folds a residual elemwise_add (and its own chain) into the epilogue of
 //     the convolution that produces one of its addends,
 //   * turns flatten -> dense over a 4-D tensor into a convolution whose kernel
-//     covers the whole feature map.
+//     covers the whole feature map,
+//   * lets a convolution whose result only goes through transpose(0,2,3,1) ->
+//     reshape -> concatenate (a detection head) write its pixel-major rows
+//     straight into its slice of the concatenated tensor.
 // Every value a later node or the caller can observe is computed by the same
 // integer arithmetic as in node-by-node execution.
 #include <algorithm>
 #include <climits>
+#include <map>
 
 #include "graph_runtime.h"
 
@@ -125,6 +129,11 @@ void HipGraphRuntime::BuildPlan() {
   auto i8_capable_shape = [&](uint32_t eid) { return shape_[eid].size() == 4 || shape_[eid].size() == 2; };
   auto pix = [&](uint32_t eid) { return shape_[eid].size() == 4 ? (int)(shape_[eid][2] * shape_[eid][3]) : 1; };
 
+  // concatenate inputs that a producer has already written into the output tensor
+  std::vector<std::vector<bool>> in_place(nodes_.size());
+  std::map<uint32_t, std::shared_ptr<DeviceBuffer>> own_storage;
+  std::vector<std::vector<bool>> head_safe(ne);  // per concatenated entry: int8 range of each part written in place
+
   std::vector<PlanStep> plan;
   auto need_i32 = [&](uint32_t eid) {
     if (has_i32[eid]) return;
@@ -192,6 +201,73 @@ void HipGraphRuntime::BuildPlan() {
       has_i32[out] = true;
       safe[out] = FitsI8(b);
     }
+  };
+
+  // conv result `out` (N, C, H, W) -> transpose(0,2,3,1) -> reshape/flatten -> one input of a concatenate
+  // whose leading dimensions multiply to N: image n's H*W*C pixel-major values are one contiguous run of
+  // the concatenated tensor.  Marks the three nodes as done and points the step at that run.
+  auto fuse_head = [&](uint32_t out, PlanStep* st) {
+    const Shape& os = shape_[out];
+    if (os.size() != 4 || is_head[out] || uses[out].size() != 1) return false;
+    const uint32_t tn = uses[out][0];
+    const Node& t = nodes_[tn];
+    if (t.func_name != "transpose" || absorbed[tn] || t.attrs.t("axes") != Shape{0, 2, 3, 1}) return false;
+    const uint32_t te = entry_id(tn, 0);
+    if (is_head[te] || uses[te].size() != 1) return false;
+    const uint32_t rn = uses[te][0];
+    const Node& r = nodes_[rn];
+    if ((r.func_name != "reshape" && r.func_name != "flatten") || absorbed[rn]) return false;
+    const uint32_t re = entry_id(rn, 0);
+    if (is_head[re] || uses[re].size() != 1) return false;
+    const uint32_t cn = uses[re][0];
+    const Node& c = nodes_[cn];
+    if (c.func_name != "concatenate" || absorbed[cn]) return false;
+    const Shape& rs = shape_[re];
+    int64_t axis = c.attrs.i("axis");
+    if (axis < 0) axis += (int64_t)rs.size();
+    if (axis < 0 || axis >= (int64_t)rs.size()) return false;
+    int64_t outer = 1, inner = 1, before = 0;
+    for (int64_t d = 0; d < axis; ++d) outer *= rs[d];
+    for (size_t d = axis + 1; d < rs.size(); ++d) inner *= rs[d];
+    if (outer != os[0]) return false;
+    int at = -1;
+    for (size_t k = 0; k < c.inputs.size(); ++k) {
+      const uint32_t ie = entry_id(c.inputs[k]);
+      if (ie == re) {
+        if (at >= 0) return false;  // the same tensor twice: leave it to the copy kernels
+        at = (int)k;
+      } else if (at < 0) {
+        before += shape_[ie][axis];
+      }
+    }
+    if (at < 0) return false;
+    const uint32_t ce = entry_id(cn, 0);
+    // The slice is written long before the concatenate node's place in the order, while the graph's
+    // storage plan may still lend that storage to other tensors: the concatenated tensor moves to
+    // storage of its own, and every node that reads or writes it is pointed there.
+    if (!own_storage.count(ce)) {
+      auto buf = std::make_shared<DeviceBuffer>();
+      Check(cvmhip_alloc(&buf->ptr, static_cast<size_t>(shape_size(shape_[ce])) * 4), "concatenated tensor");
+      own_storage[ce] = buf;
+      entry_ptr_[ce] = static_cast<int32_t*>(buf->ptr);
+      for (Exec& e : execs_) {
+        const Node& en = nodes_[e.nid];
+        for (size_t k = 0; k < en.inputs.size(); ++k)
+          if (entry_id(en.inputs[k]) == ce) e.call.in[k].data = entry_ptr_[ce];
+        if (e.nid == cn) e.call.out[0].data = entry_ptr_[ce];
+      }
+    }
+    st->aux = own_storage[ce];
+    st->nhwc = true;
+    st->dst = ce;
+    st->dst_off = before * inner;
+    st->img_stride = shape_[ce][axis] * inner;
+    st->out_i8 = false;
+    st->label += "+head";
+    absorbed[tn] = absorbed[rn] = true;
+    if (in_place[cn].empty()) in_place[cn].assign(c.inputs.size(), false);
+    in_place[cn][at] = true;
+    return true;
   };
 
   for (uint32_t nid = 0; nid < nodes_.size(); ++nid) {
@@ -293,7 +369,8 @@ void HipGraphRuntime::BuildPlan() {
         st.src2 = kNone;
         Bound b;
         const uint32_t out = follow_chain(out0, &st.chain, &b);
-        finish_output(&st, out, b);
+        if (st.kind == PlanStep::CONV && fuse_head(out, &st)) head_safe[st.dst].push_back(FitsI8(b));
+        else finish_output(&st, out, b);
         plan.push_back(st);
         done = true;
       }
@@ -426,14 +503,25 @@ void HipGraphRuntime::BuildPlan() {
 
     if (done) continue;
     // ---- the node runs as its own int32 kernel
-    for (const NodeEntry& e : n.inputs) need_i32(entry_id(e));
-    PlanStep st;
-    st.kind = PlanStep::NODE;
-    st.label = op;
-    st.exec_index = ex;
-    plan.push_back(st);
-    bool all_safe = true;
-    for (const NodeEntry& e : n.inputs) all_safe = all_safe && safe[entry_id(e)];
+    const std::vector<bool>& placed = in_place[nid];  // concatenate only: inputs already written into the output
+    bool all_safe = true, any_left = placed.empty();
+    for (size_t k = 0; k < n.inputs.size(); ++k) {
+      if (!placed.empty() && placed[k]) {
+        execs_[ex].call.in[k].data = nullptr;  // the copy of this input is skipped (cvmhip_concatenate)
+        continue;
+      }
+      need_i32(entry_id(n.inputs[k]));
+      all_safe = all_safe && safe[entry_id(n.inputs[k])];
+      any_left = true;
+    }
+    for (bool ok8 : head_safe[out0]) all_safe = all_safe && ok8;
+    if (any_left) {
+      PlanStep st;
+      st.kind = PlanStep::NODE;
+      st.label = op;
+      st.exec_index = ex;
+      plan.push_back(st);
+    }
     for (uint32_t i = 0; i < n.num_outputs; ++i) {
       const uint32_t eid = entry_id(nid, i);
       has_i32[eid] = true;
@@ -477,6 +565,12 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
         Check(cvmhip_conv2d_stem_i8(static_cast<DeviceBuffer*>(st.aux.get())->ptr, static_cast<DeviceBuffer*>(st.weights.get())->ptr,
                                     st.bias, &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw,
                                     st.sh, st.sw, st.ph, st.pw, stream_), "conv2d_stem_i8");
+        break;
+      }
+      if (st.nhwc) {
+        Check(cvmhip_conv2d_i8_nhwc(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain,
+                                    entry_ptr_[st.dst] + st.dst_off, st.img_stride, st.n, st.c, st.h, st.w, st.oc, st.kh,
+                                    st.kw, st.sh, st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "conv2d_i8_nhwc");
         break;
       }
       const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];

@@ -377,6 +377,17 @@ def conv2d_i8(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=
     return out
 
 
+def conv2d_i8_nhwc(xp, n, ic, h, w, wp, oc, kh, kw, out, offset, image_stride, bias=None, chain1=None,
+                   strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """The convolution's int32 result written pixel-major into the flat int32 tensor `out`:
+    image i's OH*OW*OC values start at element offset + i*image_stride."""
+    check(lib().cvmhip_conv2d_i8_nhwc(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
+                                      ctypes.c_void_p(out.data_ptr() + 4 * offset), ctypes.c_int64(image_stride),
+                                      n, ic, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                      dilation[0], dilation[1], _stream()))
+    return out
+
+
 def pack_depthwise_weights(w):
     c, one, kh, kw = w.shape
     wp = _workspace(lib().cvmhip_packed_depthwise_bytes(c, kh, kw), w.device)
@@ -397,8 +408,10 @@ def depthwise_conv2d_i8(xp, n, c, h, w, wp, kh, kw, bias=None, chain1=None, out_
     return out
 
 
-def add_i8(a, b, n, c, h, w, chain1=None, out_is_i8=True):
-    if out_is_i8:
+def add_i8(a, b, n, c, h, w, chain1=None, out_is_i8=True, out=None):
+    if out is not None:
+        pass
+    elif out_is_i8:
         out = torch.zeros_like(a)
     else:
         out = torch.empty((n, c, h, w), dtype=torch.int32, device=a.device)
@@ -407,15 +420,18 @@ def add_i8(a, b, n, c, h, w, chain1=None, out_is_i8=True):
     return out
 
 
-def max_pool2d_i8(xp, n, c, h, w, pool_size, strides, padding, oh, ow):
-    out = _act_buffer(n * oh * ow, c, xp.device)
+def max_pool2d_i8(xp, n, c, h, w, pool_size, strides, padding, oh, ow, out=None):
+    if out is None:
+        out = _act_buffer(n * oh * ow, c, xp.device)
     check(lib().cvmhip_max_pool2d_i8(_vp(xp), _vp(out), n, c, h, w, oh, ow, pool_size[0], pool_size[1],
                                      strides[0], strides[1], padding[0], padding[1], _stream()))
     return out
 
 
-def sum_hw_i8(xp, n, c, hw, chain1=None, out_is_i8=False):
-    if out_is_i8:
+def sum_hw_i8(xp, n, c, hw, chain1=None, out_is_i8=False, out=None):
+    if out is not None:
+        pass
+    elif out_is_i8:
         out = _act_buffer(n, c, xp.device)
     else:
         out = torch.empty((n, c), dtype=torch.int32, device=xp.device)

@@ -106,6 +106,7 @@ int cvmhip_reduce(int op, const int32_t* x, const int64_t* xshape, int ndim,
  * cuda_where, cuda_flatten/reshape/expand_dims/squeeze (cuda_ops.h:156-235);
  * CPU ops.cc:567-989,1049-1075 and elemwise.cc:64-86. */
 int cvmhip_copy(const int32_t* x, int32_t* y, int64_t size, void* stream); /* flatten/reshape/expand_dims/squeeze */
+/* inputs[m] == NULL skips that input: its slice of y is taken to be in place already */
 int cvmhip_concatenate(const int32_t* const* inputs, const int64_t* const* ishapes, int ninputs,
                        int ndim, int axis, int32_t* y, const int64_t* yshape, void* stream);
 int cvmhip_transpose(const int32_t* x, const int64_t* xshape, int ndim,
@@ -244,6 +245,13 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                      const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
                      int n, int ic, int h, int wd, int oc, int kh, int kw,
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values
+ * are contiguous at out + n*image_stride (elements).  This is what conv2d -> transpose(0,2,3,1) ->
+ * reshape -> concatenate produces for a detection head (transpose: ops.cc:743-789, concatenate:
+ * ops.cc:567-602), written in one pass straight into the head's slice of the concatenated tensor. */
+int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          int32_t* out, int64_t image_stride, int n, int ic, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
 /* conv2d over at most 4 input channels with kw <= 8, dilation 1 (the RGB stem of a network), in
  * row-window form: the input is packed once per inference into int8 [n][hp][wp][4], zero padded, so
  * that the kw taps x 4 channel bytes of a filter row are one contiguous window and no tap lies

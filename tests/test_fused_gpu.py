@@ -123,6 +123,37 @@ def test_conv2d_i8(case, conv_kernel, dev):
         eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32")
 
 
+HEAD_CASES = [
+    # n, ic, h, w, oc, k, pad, elements before the slice, elements after it
+    (1, 64, 8, 8, 84, 3, 1, 0, 0),        # SSD class head: 4 anchors x 21 classes
+    (2, 128, 5, 7, 24, 3, 1, 11, 30),     # two images, a slice in the middle of each image's row
+    (3, 32, 4, 4, 126, 1, 0, 5, 0),       # 1x1 head, odd channel count past 96
+    (1, 512, 3, 3, 16, 3, 1, 7, 9),       # deep K, very few pixels
+]
+
+
+@pytest.mark.parametrize("case", HEAD_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%d" % c[:6])
+def test_conv2d_i8_writes_a_detection_head_in_place(case, conv_kernel, dev):
+    """conv2d -> chain -> transpose(0,2,3,1) -> reshape -> concatenate, done by one launch that writes
+    the pixel-major rows into the concatenated tensor; everything outside the slice stays untouched."""
+    n, ic, h, w, oc, k, pd, before, after = case
+    cid = "head-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    ch = [("cvm_right_shift", 8, 9), ("cvm_clip", 8)]
+    ref = run_chain(oracle.conv2d(x, wt, b, (1, 1), (pd, pd), (1, 1), 1), ch)
+    part = np.ascontiguousarray(ref.transpose(0, 2, 3, 1)).reshape(n, -1)
+    stride = before + part.shape[1] + after
+    want = np.full((n, stride), 77, np.int32)
+    want[:, before:before + part.shape[1]] = part
+    out = T(np.full((n, stride), 77, np.int32), dev)
+    hipops.conv2d_i8_nhwc(hipops.pack_act_i8(T(x, dev)), n, ic, h, w, hipops.pack_weights(T(wt, dev)), oc, k, k, out, before,
+                          stride, T(b, dev), hipops.chain(*ch), padding=(pd, pd))
+    torch.cuda.synchronize()
+    eq(out.cpu().numpy(), want, "conv2d_i8_nhwc")
+
+
 STEM_CASES = [
     # n, c, h, w, oc, kh, kw, stride, pad
     (2, 3, 32, 32, 64, 7, 7, 2, 3),      # ResNet stem shape, shrunk
@@ -276,5 +307,46 @@ def test_fused_executor_equals_node_by_node(name, dev):
             os.environ.pop("CVM_HIP_FUSE", None)
     assert outs["1"] == outs["0"]
     ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
+def test_detection_heads_written_in_place_with_other_concat_inputs(dev):
+    """Two heads of different feature maps plus an ordinary tensor meet in one concatenate, batch 2.
+    The heads are written into the concatenated tensor long before the concatenate node's place in
+    the order, with more layers computed in between that reuse freed storage; a second concatenate
+    takes a head tensor twice, which must stay with the copy kernels."""
+    g = graphgen.GraphBuilder("heads-mixed")
+    x = g.var("data", (2, 3, 24, 24), 8)
+    f1 = g.conv_relu_q(x, 32, 3, 2, 1)                       # 12x12
+    h1 = g.conv_relu_q(f1, 12, 3, 1, 1, relu=False)
+    p1 = g.reshape(g.transpose(h1, (0, 2, 3, 1)), (2, 12 * 12 * 3, 4))
+    f2 = g.conv_relu_q(g.conv_relu_q(f1, 64, 3, 2, 1), 64, 1)  # 6x6, storage of earlier tensors is free again here
+    h2 = g.conv_relu_q(f2, 20, 1, 1, 0, relu=False)
+    p2 = g.reshape(g.transpose(h2, (0, 2, 3, 1)), (2, 6 * 6 * 5, 4))
+    f3 = g.conv_relu_q(f2, 32, 3, 1, 1)
+    extra = g.reshape(g.conv_relu_q(f3, 8, 3, 1, 1, relu=False), (2, 6 * 6 * 2, 4))   # NCHW order: not a head
+    cat = g.concat([p1, extra, p2], 1)
+    h3 = g.conv_relu_q(f3, 8, 1, 1, 0, relu=False)
+    p3 = g.reshape(g.transpose(h3, (0, 2, 3, 1)), (2, 6 * 6 * 2, 4))
+    twice = g.concat([p3, p3], 1)
+    js, pb = g.build([g.concat([cat, twice], 1)])
+    xv = synth.tensor("heads-mixed", "data", (2, 3, 24, 24), -127, 127)
+    outs = {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_FUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(xv.astype(np.int8).tobytes())
+            if mode == "1":
+                labels = m.profile_ops()
+                again = m.inference(xv.astype(np.int8).tobytes())     # graph replay gives the same bytes
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FUSE", None)
+    assert "conv2d+head" in labels, labels
+    assert outs["1"] == outs["0"] == again
+    ref = og.run_graph(js, graphgen.load_params(pb), xv)
     got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
