@@ -130,9 +130,10 @@ __global__ void __launch_bounds__(256) k_zero32(int32_t* __restrict__ p, int64_t
 // not depend on their order.
 __global__ void __launch_bounds__(256)
 k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
-           int n, int k, int score_index) {
+           const int32_t* __restrict__ need_full, int n, int k, int score_index) {
   __shared__ __attribute__((aligned(16))) int32_t tile[RANK_JT];
   const int b = blockIdx.z;
+  if (need_full && need_full[b] == 0) return;  // k_nms_topk_rank has ranked this batch
   if (batch_state(valid_count, b, n) != 0) return;
   const int vc = clamp_vc(valid_count[b], n);
   const int base = blockIdx.y * RANK_JT;
@@ -159,6 +160,154 @@ k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_coun
   if (i < vc && r) atomicAdd(&rank[(int64_t)b * n + i], r);
 }
 
+// With 0 < top_k < valid rows only the top_k best rows are ever looked at again, so only they need a
+// rank.  One workgroup per batch keeps every score in registers (thread t owns rows t, t + 1024, ...),
+// finds the top_k-th largest score T by bisection on the bits in which scores differ (ballot counts, no
+// atomics on data), and ranks: rows above T among themselves (fewer than top_k; listed in LDS as
+// (score, ~index) words so one 64-bit compare orders them as the stable sort would); rows equal to T
+// by their position among the equal rows in index order; every other row gets the marker rank top_k,
+// which only says "not among the first top_k".  When the condition does not hold the batch is handed
+// to k_nms_rank (need_full = 1, ranks zeroed).  All counts are integers, so the result is exact.
+constexpr int TOPK_THREADS = 1024, TOPK_ROWS = 32, TOPK_WAVES = TOPK_THREADS / 64;  // rows per thread
+constexpr int TOPK_MAX_N = TOPK_THREADS * TOPK_ROWS, TOPK_MAX_K = 2048;
+
+__global__ void __launch_bounds__(TOPK_THREADS)
+k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
+                int32_t* __restrict__ need_full, int n, int k, int score_index, int topk) {
+  __shared__ __attribute__((aligned(16))) unsigned long long s_comp[TOPK_MAX_K];
+  __shared__ int s_cnt[TOPK_MAX_K];
+  __shared__ int s_tab[TOPK_ROWS * TOPK_WAVES], s_part[2][TOPK_WAVES], s_wsum[TOPK_WAVES];
+  __shared__ uint32_t s_and[TOPK_WAVES], s_or[TOPK_WAVES];
+  __shared__ int s_gcount;
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) need_full[b] = 0;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  const int R = (vc + TOPK_THREADS - 1) / TOPK_THREADS;
+  int32_t* rk = rank + (int64_t)b * n;
+  if (!(topk > 0 && topk < vc)) {  // every valid row needs its rank: the all-pairs kernel adds them up from zero
+    for (int i = tid; i < vc; i += TOPK_THREADS) rk[i] = 0;
+    if (tid == 0) need_full[b] = 1;
+    return;
+  }
+  const int32_t* xb = x + (int64_t)b * n * k;
+  for (int i = tid; i < TOPK_MAX_K; i += TOPK_THREADS) { s_cnt[i] = 0; s_comp[i] = 0; }
+  if (tid == 0) s_gcount = 0;
+  // scores as unsigned keys that compare like the signed values; rows past the end hold key 0 and are
+  // told apart by their index wherever a real key could be 0 too
+  uint32_t key[TOPK_ROWS];
+#pragma unroll
+  for (int r = 0; r < TOPK_ROWS; ++r) {
+    const int i = r * TOPK_THREADS + tid;
+    key[r] = (r < R && i < vc) ? (uint32_t)xb[(int64_t)i * k + score_index] ^ 0x80000000u : 0u;
+  }
+  // Bits above the highest bit in which two live keys differ are common to all keys: the bisection
+  // only walks the bits below (8 steps for scores that span 8 bits, whatever their offset).
+  uint32_t kand = 0xffffffffu, kor = 0;
+#pragma unroll
+  for (int r = 0; r < TOPK_ROWS; ++r) {
+    if (r >= R) break;
+    if (r * TOPK_THREADS + tid < vc) { kand &= key[r]; kor |= key[r]; }
+  }
+  for (int d = 32; d >= 1; d >>= 1) {
+    kand &= (uint32_t)__shfl_xor((int)kand, d, 64);
+    kor |= (uint32_t)__shfl_xor((int)kor, d, 64);
+  }
+  if (lane == 0) { s_and[wave] = kand; s_or[wave] = kor; }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < TOPK_WAVES; ++w) { kand &= s_and[w]; kor |= s_or[w]; }
+  const uint32_t diff = kand ^ kor;
+  const int top_bit = diff ? 31 - __clz((int)diff) : -1;
+  // T becomes the top_k-th largest key: the largest T with at least top_k keys >= T
+  uint32_t T = top_bit >= 0 ? (kor & ~((2u << top_bit) - 1u)) : kor;
+  for (int bit = top_bit; bit >= 0; --bit) {
+    const uint32_t cand = T | (1u << bit);
+    int c = 0;
+#pragma unroll
+    for (int r = 0; r < TOPK_ROWS; ++r) {
+      if (r >= R) break;
+      c += __popcll(__ballot(key[r] >= cand));
+    }
+    int* part = s_part[bit & 1];
+    if (lane == 0) part[wave] = c;
+    __syncthreads();
+    int tot = 0;
+#pragma unroll
+    for (int w = 0; w < TOPK_WAVES; ++w) tot += part[w];
+    if (tot >= topk) T = cand;
+  }
+  // rows above T: listed in any order (the 64-bit word carries the index); rows equal to T: counted
+  // per (row block r, wavefront), which is index order
+  const unsigned long long lt = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int r = 0; r < TOPK_ROWS; ++r) {
+    if (r >= R) break;
+    const int i = r * TOPK_THREADS + tid;
+    const bool up = key[r] > T;
+    const unsigned long long bu = __ballot(up), be = __ballot(i < vc && key[r] == T);
+    int base = 0;
+    if (lane == 0) {
+      s_tab[r * TOPK_WAVES + wave] = __popcll(be);
+      if (bu) base = atomicAdd(&s_gcount, __popcll(bu));
+    }
+    base = __shfl(base, 0, 64);
+    if (up) s_comp[base + __popcll(bu & lt)] = ((unsigned long long)key[r] << 32) | (uint32_t)~(uint32_t)i;
+  }
+  __syncthreads();
+  const int g = s_gcount;           // rows above T: fewer than top_k
+  const int from_equal = topk - g;  // this many of the equal rows, in index order, complete the top_k
+  // exclusive prefix of the equal-row counts over (r, wavefront)
+  {
+    const int cells = R * TOPK_WAVES;
+    const int v = tid < cells ? s_tab[tid] : 0;
+    int inc = v;
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(inc, d, 64);
+      if (lane >= d) inc += o;
+    }
+    if (lane == 63) s_wsum[wave] = inc;
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += s_wsum[w];
+    if (tid < cells) s_tab[tid] = before + inc - v;
+  }
+  // ranks among the rows above T: element p counts the words larger than its own, its q range split
+  // over `slices` threads whose partial counts add up in LDS
+  const int P = (g + 63) & ~63;
+  const int slices = P > 0 && P < TOPK_THREADS ? TOPK_THREADS / P : 1;
+  const int chunk = ((g + slices - 1) / slices + 1) & ~1;
+  for (int item = tid; item < P * slices; item += TOPK_THREADS) {
+    const int p = item % P, sl = item / P;
+    if (p >= g) continue;
+    const unsigned long long me = s_comp[p];
+    int q0 = sl * chunk, q1 = q0 + chunk;   // the list is zero-padded past g: zeros are below every real word
+    if (q1 > TOPK_MAX_K) q1 = TOPK_MAX_K;
+    int c = 0;
+    for (int q = q0; q < q1 && q < g; q += 2) {
+      const ulonglong2 o = *reinterpret_cast<const ulonglong2*>(&s_comp[q]);
+      c += (o.x > me) + (o.y > me);
+    }
+    if (c) atomicAdd(&s_cnt[p], c);
+  }
+  __syncthreads();
+  for (int p = tid; p < g; p += TOPK_THREADS) rk[(int)~(uint32_t)s_comp[p]] = s_cnt[p];
+#pragma unroll
+  for (int r = 0; r < TOPK_ROWS; ++r) {
+    if (r >= R) break;
+    const int i = r * TOPK_THREADS + tid;
+    const bool eq = i < vc && key[r] == T;
+    const unsigned long long be = __ballot(eq);
+    if (i >= vc || key[r] > T) continue;
+    if (eq) {
+      const int e = s_tab[r * TOPK_WAVES + wave] + __popcll(be & lt);
+      rk[i] = e < from_equal ? g + e : topk;
+    } else {
+      rk[i] = topk;
+    }
+  }
+}
+
 // Row i moves to its sorted slot; rows ranked at or past top_k are then overwritten with -1 in the input
 // tensor (nms.cc:92-96).  Every output row starts as -1: k_nms_select writes the kept rows over the front.
 __global__ void __launch_bounds__(256)
@@ -177,11 +326,13 @@ k_nms_scatter(int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, 
   if (i >= vc) return;
   int32_t* xrow = x + ((int64_t)b * n + i) * k;
   const int r = rank[(int64_t)b * n + i];
+  if (topk > 0 && r >= topk) {  // never looked at again (its rank may be the marker top_k, shared by many rows)
+    for (int c = 0; c < k; ++c) xrow[c] = -1;
+    return;
+  }
   order[b * ws_stride + r] = i;
   int32_t* dst = sorted + b * ws_stride * k + (int64_t)r * k;
   for (int c = 0; c < k; ++c) dst[c] = xrow[c];
-  if (topk > 0 && r >= topk)
-    for (int c = 0; c < k; ++c) xrow[c] = -1;
 }
 
 constexpr int NMS_BM_ROWS = 512, NMS_BM_WORDS = 16;  // rows of the suppression bit matrix and its words per row
@@ -399,9 +550,9 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
   return check_launch("get_valid_counts.scatter");
 }
 
-// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix, one flag
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
-  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 1 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS) * sizeof(int32_t);
+  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 2 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS) * sizeof(int32_t);
 }
 
 int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
@@ -422,16 +573,25 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
   int32_t* removed = nextneg + (size_t)batches * (n + 1);
   int32_t* sorted = removed + (size_t)batches * n;
   int32_t* rank = sorted + (size_t)batches * n * k;
-  k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
+  uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
+  int32_t* need_full = reinterpret_cast<int32_t*>(mask + (size_t)batches * NMS_BM_ROWS * NMS_BM_WORDS);
+  const bool select_first = topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N;
+  int rc;
+  if (select_first) {
+    k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, need_full, n, k, score_index, topk);
+    rc = check_launch("nms.topk_rank");
+    if (rc) return rc;
+  } else {
+    k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
+  }
   dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
-  k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, n, k, score_index);
-  int rc = check_launch("nms.rank");
+  k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, select_first ? need_full : nullptr, n, k, score_index);
+  rc = check_launch("nms.rank");
   if (rc) return rc;
   dim3 grid((n + 255) / 256, batches);
   k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, y, n, k, topk, (int64_t)n);
   rc = check_launch("nms.scatter");
   if (rc) return rc;
-  uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
   int rows = n < NMS_BM_ROWS ? n : NMS_BM_ROWS;  // upper bound of the rows the walk can see, when the matrix is used
   if (topk >= 0 && topk < rows) rows = topk;
   if (rows > 0 && k <= NMS_LDS_K) {

@@ -291,6 +291,24 @@ def test_non_max_suppression(case, dev):
     same(tx, x_after, "nms input after the call")
 
 
+@pytest.mark.parametrize("score,topk,n", [((-2 ** 31, 2 ** 31 - 1), 400, 5000),   # keys differ in every bit
+                                          ((7, 7), 50, 900),                      # all scores equal: order by index alone
+                                          ((-3, 3), 300, 4000),                   # long runs of equal scores around the cut
+                                          ((2 ** 31 - 5, 2 ** 31 - 1), 2048, 3000),  # the largest top_k of the selection path
+                                          ((-2 ** 31, -2 ** 31 + 2), 2049, 3000),    # one more: all-pairs ranking
+                                          ((0, 1000), 1, 700)])
+def test_nms_top_k_selection(score, topk, n, dev):
+    """Rows past top_k only need to be known as such; the first top_k must come out in the stable-sort order."""
+    x = _boxes("nms-topk-%s-%d" % (score, topk), 2, n, -1, 3, score=score, extent=256)
+    vc = np.array([n, n - 7], np.int32)
+    init = np.full_like(x, 5)
+    y_ref, x_after = oracle.non_max_suppression(x, vc, 60, False, topk, y_init=init)
+    tx, ty = T(x, dev), T(init, dev)
+    hipops.non_max_suppression(tx, T(vc, dev), ty, 60, False, topk)
+    same(ty, y_ref, "nms output")
+    same(tx, x_after, "nms input after the call")
+
+
 def test_nms_stops_at_first_batch_without_valid_rows(dev):
     x = _boxes("nms-early", 3, 40, 0, 3, extent=32)
     vc = np.array([12, 0, 30], np.int32)
