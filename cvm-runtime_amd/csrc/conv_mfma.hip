@@ -115,9 +115,43 @@ __device__ __forceinline__ void mask_channels(uint32_t (&d)[N], int first, int O
 // For a pixel-blocked int8 tensor two half-wave swaps turn the 4 packed dwords of a
 // tile into 16 consecutive channels per lane, so the wavefront reads the
 // residual and writes the result as one contiguous KiB per tile.
+// Residual values of the groups u0 .. u0+NG-1 of a wavefront (same numbering as finish_groups), as
+// they lie in memory: for whole tiles the 16 bytes per lane of each tile's KiB block, otherwise the 4
+// bytes of each group.  Separate from finish_groups so that a kernel can issue these loads before its
+// K loop and find them in registers when the accumulators are ready.
+template <int TN, int NG>
+__device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch_wave, int oc0, int px_wave, int lane,
+                                              const ConvGeom& g, const Epilogue& ep) {
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int P = (int)g.P;
+  const int ocp = ep.out_cp;
+  const bool whole = act_blocked(ocp) && (NG % 4 == 0);
+  if (whole) {
+#pragma unroll
+    for (int t = 0; t < NG / 4; ++t) {
+      const int tt = (u0 >> 2) + t;
+      const int gj = tt % TN, chb = ch_wave + (tt / TN) * 32;
+      // the block exists (all 32 pixel rows of it are allocated) unless it lies past the tensor
+      const bool tile_ok = (px_wave + gj * 32) < P && (oc0 + chb) < ocp;
+      const int64_t off = ((int64_t)((px_wave >> 5) + gj) * (ocp >> 5) + ((oc0 + chb) >> 5)) * 1024;
+      const int4 r4 = tile_ok ? *reinterpret_cast<const int4*>(ep.residual + off + lane * 16) : zero4();
+      rp[t * 4] = r4.x; rp[t * 4 + 1] = r4.y; rp[t * 4 + 2] = r4.z; rp[t * 4 + 3] = r4.w;
+    }
+  } else {
+#pragma unroll
+    for (int m = 0; m < NG; ++m) {
+      const int u = u0 + m, t = u >> 2;
+      const int p = px_wave + (t % TN) * 32 + lrow;
+      const int oc = oc0 + ch_wave + (t / TN) * 32 + (u & 3) * 8 + lgrp * 4;
+      rp[m] = *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ocp ? oc : 0, ocp));
+    }
+  }
+}
+
 template <int TN, int NG, int OUT>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
-                                              int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep) {
+                                              int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
+                                              uint32_t (&rp)[NG]) {
   const int lrow = lane & 31, lgrp = lane >> 5;
   const int P = (int)g.P;
   const int ocp = ep.out_cp;
@@ -143,25 +177,14 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   const bool whole = blocked && (NG % 4 == 0);   // whole tiles: 16 bytes per lane
   const bool halves = blocked && NG == 2;         // half a tile (q pair): 8 bytes per lane
 
-  if (ep.residual) {
-    uint32_t rp[NG];
+  if (ep.residual) {   // rp holds what load_residual fetched
     if (whole) {
 #pragma unroll
       for (int t = 0; t < NG / 4; ++t) {
-        // the block exists (all 32 pixel rows of it are allocated) unless it lies past the tensor
-        const bool tile_ok = (px_wave + gj[t * 4] * 32) < P && (oc0 + ch[t * 4] - lgrp * 4) < ocp;
-        const int4 r4 = tile_ok ? *reinterpret_cast<const int4*>(ep.residual + block_off(t * 4) + lane * 16) : zero4();
-        uint32_t a = r4.x, b = r4.y, c = r4.z, d = r4.w;
+        uint32_t a = rp[t * 4], b = rp[t * 4 + 1], c = rp[t * 4 + 2], d = rp[t * 4 + 3];
         half_swap(a, b);
         half_swap(c, d);
         rp[t * 4] = a; rp[t * 4 + 1] = c; rp[t * 4 + 2] = b; rp[t * 4 + 3] = d;
-      }
-    } else {
-#pragma unroll
-      for (int m = 0; m < NG; ++m) {
-        const int p = px_wave + gj[m] * 32 + lrow;
-        const int oc = oc0 + ch[m];
-        rp[m] = *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ocp ? oc : 0, ocp));
       }
     }
     run_chain(ep.chain, val);
@@ -423,7 +446,9 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) val[(i * WN + j) * 16 + e] = acc[i][j][e];
-  finish_groups<WN, WM * WN * 4, OUT>(val, 0, sBias, wm * WM * 32, oc0, (int)px0 + wn * WN * 32, lane, out, g, ep);
+  uint32_t rp[WM * WN * 4];
+  if (ep.residual) load_residual<WN, WM * WN * 4>(rp, 0, wm * WM * 32, oc0, (int)px0 + wn * WN * 32, lane, g, ep);
+  finish_groups<WN, WM * WN * 4, OUT>(val, 0, sBias, wm * WM * 32, oc0, (int)px0 + wn * WN * 32, lane, out, g, ep, rp);
 }
 
 // ---------------------------------------------------------------- wavefront-private kernel
@@ -648,6 +673,10 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
     }
   };
 
+  // the residual of the groups this wavefront will finalise travels with the first operands
+  uint32_t rp[NU];
+  if (ep.residual) load_residual<TN, NU>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+
   regs_t R0 = fetch();
   regs_t R1;
   for (int it = 0; it < niter; it += 2) {
@@ -691,7 +720,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
         for (int e = 0; e < 16; ++e) val[((i * TN + j) * 16 + e) % (NU * 4)] = acc[i][j][e];
   }
-  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, out, g, ep);
+  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, out, g, ep, rp);
 }
 
 constexpr int KSTEP = 64;  // granularity K is padded to
