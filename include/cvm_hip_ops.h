@@ -139,8 +139,9 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
 /* ---- non_max_suppression: cuda_non_max_suppression (cuda_ops.h:228, nms.cu:310-430);
  * semantics of the CPU operator (nms.cc:65-140), including its early exit on a
  * batch with no valid rows, its stop at the first negative id and its in-place
- * overwrite of x rows past top_k.  No host synchronisation: valid_count is read
- * on the device.  `workspace`: cvmhip_nms_workspace_bytes() bytes of scratch. */
+ * overwrite of x rows past top_k (x is therefore written, and must not alias y).
+ * No host synchronisation: valid_count is read on the device.
+ * `workspace`: cvmhip_nms_workspace_bytes() bytes of scratch. */
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k);
 int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
                                int batches, int n, int k, int max_output_size,
