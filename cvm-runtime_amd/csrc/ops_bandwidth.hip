@@ -158,15 +158,19 @@ static int launch_broadcast(const int32_t* a, const int32_t* b, int32_t* c, int6
 }
 
 // ---------------------------------------------------------------- max_pool2d
+// One thread per output element; I is the index type (32-bit whenever the tensors allow it: the three
+// divisions per element are what this kernel would otherwise spend most of its time on).
+template <typename I>
 __global__ void __launch_bounds__(256) k_max_pool(const int32_t* __restrict__ x, int32_t* __restrict__ y,
                                                   int64_t total, int h, int w, int oh, int ow, int kh, int kw,
                                                   int sh, int sw, int ph, int pw) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int q = (int)(i % ow);
-    const int p = (int)((i / ow) % oh);
-    const int64_t nc = i / ((int64_t)ow * oh);
-    const int32_t* xp = x + nc * h * w;
+  const I stride = (I)gridDim.x * blockDim.x;
+  for (I i = (I)blockIdx.x * blockDim.x + threadIdx.x; i < (I)total; i += stride) {
+    const I row = i / (I)ow;
+    const int q = (int)(i - row * (I)ow);
+    const I nc = row / (I)oh;
+    const int p = (int)(row - nc * (I)oh);
+    const int32_t* xp = x + (int64_t)nc * h * w;
     int32_t m = INT32_MIN;
     for (int r = 0; r < kh; ++r) {
       const int ih = p * sh + r - ph;
@@ -174,7 +178,7 @@ __global__ void __launch_bounds__(256) k_max_pool(const int32_t* __restrict__ x,
       for (int t = 0; t < kw; ++t) {
         const int iw = q * sw + t - pw;
         if (iw < 0 || iw >= w) continue;
-        const int32_t v = xp[(int64_t)ih * w + iw];
+        const int32_t v = xp[ih * w + iw];
         m = v > m ? v : m;
       }
     }
@@ -475,8 +479,11 @@ int cvmhip_max_pool2d(const int32_t* x, int32_t* y, int n, int c, int h, int w,
       pad_h < 0 || pad_w < 0)
     return arg_error("max_pool2d");
   const int64_t total = (int64_t)n * c * oh * ow;
-  k_max_pool<<<grid_for(total, 256), 256, 0, as_stream(stream)>>>(x, y, total, h, w, oh, ow, kh, kw, stride_h,
-                                                                stride_w, pad_h, pad_w);
+  const unsigned grid = grid_for(total, 256, 256 * 64);
+  if (total + (int64_t)grid * 256 < INT32_MAX && (int64_t)h * w < INT32_MAX)
+    k_max_pool<uint32_t><<<grid, 256, 0, as_stream(stream)>>>(x, y, total, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
+  else
+    k_max_pool<int64_t><<<grid, 256, 0, as_stream(stream)>>>(x, y, total, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
   return check_launch("max_pool2d");
 }
 
