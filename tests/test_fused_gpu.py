@@ -123,6 +123,59 @@ def test_conv2d_i8(case, conv_kernel, dev):
         eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32")
 
 
+def _random_conv_cases(count):
+    """Seeded geometries across the addressing modes of both kernels: 1x1 / strided / padded / dilated,
+    channel counts on both sides of the 4-8-16-32 padding steps, ragged pixel counts."""
+    rng = np.random.RandomState(20240611)
+    cases = []
+    while len(cases) < count:
+        ic = int(rng.choice([1, 3, 5, 8, 13, 16, 24, 32, 40, 64, 96, 160]))
+        oc = int(rng.choice([1, 7, 16, 31, 32, 33, 64, 100, 130]))
+        k = int(rng.choice([1, 1, 2, 3, 3, 5]))
+        st = int(rng.choice([1, 1, 2, 3]))
+        pd = int(rng.choice([0, 0, 1, 2]))
+        dl = int(rng.choice([1, 1, 1, 2]))
+        n = int(rng.choice([1, 2, 3]))
+        h, w = int(rng.randint(1, 15)), int(rng.randint(1, 15))
+        if h + 2 * pd < dl * (k - 1) + 1 or w + 2 * pd < dl * (k - 1) + 1:
+            continue
+        cases.append((n, ic, h, w, oc, k, st, pd, dl, bool(rng.randint(2)), bool(rng.randint(2)), bool(rng.randint(2))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(48), ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%dd%d" % c[:9])
+def test_conv2d_i8_random_geometries(case, dev):
+    n, ic, h, w, oc, k, st, pd, dl, bias, with_res, i8 = case
+    cid = "rconv-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768) if bias else None
+    shift = max(1, int(np.ceil(np.log2(ic * k * k * 127 * 127 / 100.0))))
+    ch1 = [("cvm_right_shift", 8, shift)]
+    ch2 = [("relu",), ("cvm_right_shift", 8, 1)]
+    ref = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (dl, dl), 1), ch1)
+    oh, ow = ref.shape[2:]
+    res_t = None
+    if with_res:
+        r = synth.tensor(cid, "r", ref.shape, -127, 127)
+        ref = run_chain(oracle.elemwise("elemwise_add", ref, r), ch2)
+        res_t = hipops.pack_act_i8(T(r, dev))
+    xp, wp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev))
+    for kind in ("lds", "wave"):
+        os.environ["CVM_HIP_CONV"] = kind
+        try:
+            out = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1), res_t,
+                                   hipops.chain(*ch2) if with_res else None, out_is_i8=i8, strides=(st, st),
+                                   padding=(pd, pd), dilation=(dl, dl))
+        finally:
+            os.environ.pop("CVM_HIP_CONV", None)
+        if i8:
+            eq(act_to_nchw(out, n, oc, oh, ow), ref, "conv2d_i8 (%s)" % kind)
+        else:
+            torch.cuda.synchronize()
+            eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32 (%s)" % kind)
+
+
 HEAD_CASES = [
     # n, ic, h, w, oc, k, pad, elements before the slice, elements after it
     (1, 64, 8, 8, 84, 3, 1, 0, 0),        # SSD class head: 4 anchors x 21 classes
