@@ -93,6 +93,25 @@ def test_config4_vgg16_full_size_batch1(dev):
     _check(out, tsize, ref)
 
 
+def test_config4_vgg16_batch16_matches_per_image_runs(dev):
+    # full-size batch 16 (the large-layer regime of both convolution kernels): images are independent, so
+    # every image must equal its batch-1 result; batch 1 equals the oracle through the test above
+    g16, h16 = graphgen.vgg16(16)
+    js16, pb = g16.build(h16)
+    x = synth.tensor("cfg4-b16", "data", (16, 3, 224, 224), -127, 127).astype(np.int8)
+    m16 = runtime.HipModel(js16, pb)
+    out16 = np.frombuffer(m16.inference(x.tobytes()), np.int32).reshape(16, 1000)
+    m16.close()
+    g1, h1 = graphgen.vgg16(1)
+    js1, pb1 = g1.build(h1)
+    assert pb1 == pb
+    m1 = runtime.HipModel(js1, pb1)
+    for i in (0, 5, 15):
+        o = np.frombuffer(m1.inference(x[i:i + 1].tobytes()), np.int32)
+        assert np.array_equal(o, out16[i]), "image %d differs between batch 16 and batch 1" % i
+    m1.close()
+
+
 @pytest.mark.parametrize("neg_ids", [False, True])
 def test_config5_ssd_mobilenet_detector(neg_ids, dev):
     g, heads = graphgen.ssd_mobilenet(neg_ids=neg_ids, config_id="cfg5-%d" % neg_ids)
