@@ -87,7 +87,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on exactly one GPU (got --gpus %d); the path shards by batch "
-                 "with no exchange step, see DESIGN.md" % args.gpus)
+                 "with no exchange step, each GPU running this same program on its share" % args.gpus)
 
     import numpy as np
     import torch
