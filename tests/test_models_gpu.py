@@ -175,3 +175,36 @@ def test_int8_input_is_clamped_like_the_reference(dev):
     m.close()
     ref = og.run_graph(js, graphgen.load_params(pb), np.clip(x, -127, 127))
     assert np.array_equal(out, ref[0].ravel())
+
+
+def test_two_nets_on_two_threads_and_many_replays(dev):
+    """Distinct nets may run on different threads (the reference's threading rule): two models of
+    different graphs run 40 inferences each at the same time; every result equals the one the model
+    gives alone.  Also covers many replays of the captured graph of each model."""
+    import threading
+    ga, ha = graphgen.resnet20_cifar(4)
+    gb, hb = graphgen.ssd_mobilenet(size=128, alpha=0.25, config_id="threads-ssd", neg_ids=True)
+    specs = []
+    for g, h, cid in ((ga, ha, "threads-a"), (gb, hb, "threads-b")):
+        js, pb = g.build(h)
+        x = synth.tensor(cid, "data", g.shape((0, 0)), -127, 127).astype(np.int8).tobytes()
+        m = runtime.HipModel(js, pb)
+        specs.append((m, x, m.inference(x)))
+    errors = []
+
+    def work(m, x, want):
+        try:
+            for _ in range(40):
+                if m.inference(x) != want:
+                    errors.append("result changed")
+                    return
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(repr(e))
+    threads = [threading.Thread(target=work, args=s) for s in specs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for m, _, _ in specs:
+        m.close()
+    assert not errors, errors
