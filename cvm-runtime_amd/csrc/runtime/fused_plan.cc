@@ -134,6 +134,31 @@ void HipGraphRuntime::BuildPlan() {
   std::map<uint32_t, std::shared_ptr<DeviceBuffer>> own_storage;
   std::vector<std::vector<bool>> head_safe(ne);  // per concatenated entry: int8 range of each part written in place
 
+  // Moves an int32 tensor to storage of its own and points every node that reads or writes it there.
+  // Needed wherever a fused step writes such a tensor earlier than the node that produces it in the
+  // graph's order: the graph's storage plan may still lend that storage to another tensor then.
+  std::vector<int> sid_users(pool_.size(), 0);
+  for (uint32_t e = 0; e < ne; ++e) ++sid_users[storage_id_[e]];
+  auto privatize = [&](uint32_t eid) {
+    if (own_storage.count(eid)) return;
+    auto buf = std::make_shared<DeviceBuffer>();
+    Check(cvmhip_alloc(&buf->ptr, std::max<size_t>(static_cast<size_t>(shape_size(shape_[eid])) * 4, 4)), "tensor storage");
+    own_storage[eid] = buf;
+    own_storage_.push_back(buf);
+    entry_ptr_[eid] = static_cast<int32_t*>(buf->ptr);
+    for (Exec& e : execs_) {
+      const Node& en = nodes_[e.nid];
+      for (size_t k = 0; k < en.inputs.size(); ++k)
+        if (entry_id(en.inputs[k]) == eid) e.call.in[k].data = entry_ptr_[eid];
+      for (uint32_t k = 0; k < en.num_outputs; ++k)
+        if (entry_id(e.nid, k) == eid) e.call.out[k].data = entry_ptr_[eid];
+    }
+  };
+  // int32 result of a fused step: written at the position of the step's first node
+  auto early_i32 = [&](uint32_t eid) {
+    if (sid_users[storage_id_[eid]] > 1) privatize(eid);
+  };
+
   std::vector<PlanStep> plan;
   auto need_i32 = [&](uint32_t eid) {
     if (has_i32[eid]) return;
@@ -200,6 +225,7 @@ void HipGraphRuntime::BuildPlan() {
     } else {
       has_i32[out] = true;
       safe[out] = FitsI8(b);
+      early_i32(out);
     }
   };
 
@@ -242,21 +268,8 @@ void HipGraphRuntime::BuildPlan() {
     }
     if (at < 0) return false;
     const uint32_t ce = entry_id(cn, 0);
-    // The slice is written long before the concatenate node's place in the order, while the graph's
-    // storage plan may still lend that storage to other tensors: the concatenated tensor moves to
-    // storage of its own, and every node that reads or writes it is pointed there.
-    if (!own_storage.count(ce)) {
-      auto buf = std::make_shared<DeviceBuffer>();
-      Check(cvmhip_alloc(&buf->ptr, static_cast<size_t>(shape_size(shape_[ce])) * 4), "concatenated tensor");
-      own_storage[ce] = buf;
-      entry_ptr_[ce] = static_cast<int32_t*>(buf->ptr);
-      for (Exec& e : execs_) {
-        const Node& en = nodes_[e.nid];
-        for (size_t k = 0; k < en.inputs.size(); ++k)
-          if (entry_id(en.inputs[k]) == ce) e.call.in[k].data = entry_ptr_[ce];
-        if (e.nid == cn) e.call.out[0].data = entry_ptr_[ce];
-      }
-    }
+    // the slice is written long before the concatenate node's place in the order
+    privatize(ce);
     st->aux = own_storage[ce];
     st->nhwc = true;
     st->dst = ce;
@@ -406,6 +419,7 @@ void HipGraphRuntime::BuildPlan() {
           } else {
             has_i32[out] = true;
             safe[out] = FitsI8(b);
+            early_i32(out);
           }
           folded = true;
         }
@@ -476,6 +490,7 @@ void HipGraphRuntime::BuildPlan() {
         } else {
           has_i32[out] = true;
           safe[out] = FitsI8(b);
+          early_i32(out);
         }
         plan.push_back(st);
         done = true;

@@ -448,6 +448,7 @@ void HipGraphRuntime::Release() {
   if (in_stage_dev_) { cvmhip_free(in_stage_dev_); in_stage_dev_ = nullptr; }
   if (in_stage_host_) { cvmhip_host_free(in_stage_host_); in_stage_host_ = nullptr; }
   if (stream_) cvmhip_stream_sync(stream_);
+  own_storage_.clear();
   if (workspace_) cvmhip_free(workspace_);
   if (slab_) cvmhip_free(slab_);
   if (stream_) cvmhip_stream_destroy(stream_);

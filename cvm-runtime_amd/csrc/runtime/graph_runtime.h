@@ -193,6 +193,7 @@ class HipGraphRuntime {
   bool fused_ = false;
   std::vector<PlanStep> plan_;
   std::vector<void*> i8_ptr_;      // per entry: int8 NHWC form (nullptr if never materialised)
+  std::vector<std::shared_ptr<void>> own_storage_;  // int32 tensors the planner moved out of the shared storage pool
   void* i8_slab_ = nullptr;
 };
 

@@ -403,3 +403,40 @@ def test_detection_heads_written_in_place_with_other_concat_inputs(dev):
     ref = og.run_graph(js, graphgen.load_params(pb), xv)
     got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
+def test_storage_shared_by_liveness_is_not_clobbered_by_early_writes(dev):
+    """A memory-planned graph lends the storage of a dead tensor to a later one.  A fused step writes
+    its chain's final int32 output at the position of the chain's first node, i.e. possibly while the
+    previous owner of that storage is still alive: the planner must move such an output to storage
+    of its own.  Here `t` (read by `u = abs(t)` between the convolution and the end of its chain)
+    shares its storage with the chain's output."""
+    import json as _json
+    g = graphgen.GraphBuilder("shared-storage")
+    x = g.var("data", (1, 32, 6, 6), 8)
+    t = g.unary("negative", x)                       # int32 tensor, alive until u is computed
+    c, _ = g.conv(x, 32, 3, 1, 1)                    # first node of the fused chain
+    u = g.unary("abs", t)                            # still needs t
+    q = g.clip8(g.rshift(c, 12))                     # rest of the chain; its output takes over t's storage
+    (out,) = g.op("broadcast_add", [q, u], {}, [g.shape(q)])
+    js, pb = g.build([out])
+    d = _json.loads(js)
+    sid = d["attrs"]["storage_id"][1]
+    sid[g._eid(q)] = sid[g._eid(t)]
+    js = _json.dumps(d)
+    xv = synth.tensor("shared-storage", "data", (1, 32, 6, 6), -127, 127)
+    outs = {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_FUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(xv.astype(np.int8).tobytes())
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FUSE", None)
+    ref = og.run_graph(js, graphgen.load_params(pb), xv)
+    want = np.concatenate([r.ravel() for r in ref])
+    for mode in ("0", "1"):
+        got = np.frombuffer(outs[mode], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+        assert np.array_equal(got, want), "planner %s" % ("on" if mode == "1" else "off")
