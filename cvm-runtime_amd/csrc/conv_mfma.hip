@@ -60,7 +60,11 @@ __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
     const int32_t s1 = t == 0 ? q0.s1 : t == 1 ? q1.s1 : t == 2 ? q2.s1 : q3.s1;
     const int32_t ad = t == 0 ? q0.add : t == 1 ? q1.add : t == 2 ? q2.add : q3.add;
     const int32_t s2 = t == 0 ? q0.s2 : t == 1 ? q1.s2 : t == 2 ? q2.s2 : q3.s2;
-    if ((s1 | ad | s2) == 0) {
+    const int32_t mu = t == 0 ? q0.mul : t == 1 ? q1.mul : t == 2 ? q2.mul : q3.mul;
+    if (mu != 1) {   // a multiplication stage (rare: one more instruction per value)
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = wadd(wmul(clamp3(v[e], lo, hi), mu) >> s1, ad) >> s2;
+    } else if ((s1 | ad | s2) == 0) {
 #pragma unroll
       for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], lo, hi);
     } else if (s1 == 0) {

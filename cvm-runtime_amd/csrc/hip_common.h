@@ -124,6 +124,7 @@ __device__ __forceinline__ int32_t apply_rshift(const RShift& r, int32_t t) {
 struct DevStage {
   int32_t lo, hi;
   int32_t s1, add, s2;
+  int32_t mul;   // applied after the clamp, before the shifts (1 unless the stage is a multiplication)
 };
 struct DevChain {
   int count;
@@ -133,6 +134,7 @@ struct DevChain {
 __device__ __forceinline__ int32_t apply_stage(const DevStage& s, int32_t v) {
   v = v < s.lo ? s.lo : v;
   v = v > s.hi ? s.hi : v;
+  if (s.mul != 1) v = wmul(v, s.mul);   // uniform across the launch
   return wadd(v >> s.s1, s.add) >> s.s2;
 }
 
@@ -145,7 +147,7 @@ __device__ __forceinline__ int32_t apply_chain(const DevChain& c, int32_t v) {
   return v;
 }
 
-inline bool stage_is_clamp(const DevStage& s) { return s.s1 == 0 && s.add == 0 && s.s2 == 0; }
+inline bool stage_is_clamp(const DevStage& s) { return s.s1 == 0 && s.add == 0 && s.s2 == 0 && s.mul == 1; }
 
 // host: validates and converts the C-ABI chain; returns false on a bad stage
 inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
@@ -154,7 +156,7 @@ inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
   if (in->count < 0 || in->count > 4) return false;
   for (int i = 0; i < in->count; ++i) {
     const cvmhip_stage& s = in->stage[i];
-    DevStage d = {INT32_MIN, INT32_MAX, 0, 0, 0};
+    DevStage d = {INT32_MIN, INT32_MAX, 0, 0, 0, 1};
     if (s.kind == CVMHIP_STAGE_RELU) {
       d.lo = 0;
     } else if (s.kind == CVMHIP_STAGE_CLIP) {
@@ -174,6 +176,8 @@ inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
           d.s1 = 0; d.add = (int32_t)1 << r.sh; d.s2 = r.sh + 1;
         }
       }
+    } else if (s.kind == CVMHIP_STAGE_MUL) {
+      d.mul = s.lo;   // wrapping int32 product, as broadcast_mul computes it (broadcast.cc:75-86)
     } else {
       return false;
     }

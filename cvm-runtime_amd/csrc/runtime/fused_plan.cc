@@ -196,10 +196,29 @@ void HipGraphRuntime::BuildPlan() {
     while (chain->count < 4 && uses[cur].size() == 1 && !is_head[cur]) {
       const uint32_t cn = uses[cur][0];
       const Node& c = nodes_[cn];
-      if (absorbed[cn] || c.inputs.size() != 1) break;
+      if (absorbed[cn]) break;
       cvmhip_stage st = {};
       Bound nb = *bound;
-      if (!ChainStage(c, &st, &nb)) break;
+      if (c.func_name == "broadcast_mul" && c.inputs.size() == 2) {
+        // the requantisation scale: a product with a constant scalar, its result shaped like the chain's value
+        const uint32_t a = entry_id(c.inputs[0]), b = entry_id(c.inputs[1]);
+        const uint32_t other = a == cur ? b : a;
+        const Node& on = nodes_[(a == cur ? c.inputs[1] : c.inputs[0]).node_id];
+        if (a == b || !on.is_variable() || on.is_data() || shape_size(shape_[other]) != 1 ||
+            shape_[entry_id(cn, 0)] != shape_[cur])
+          break;
+        int32_t m = 0;
+        Check(cvmhip_copy_d2h(&m, entry_ptr_[other], sizeof(m), stream_), "read scale");
+        Check(cvmhip_stream_sync(stream_), "read scale");
+        st.kind = CVMHIP_STAGE_MUL;
+        st.lo = m;
+        const int64_t p = nb.lo * m, q = nb.hi * m;   // |bounds| <= 2^31 and |m| <= 2^31: no int64 overflow
+        nb.lo = std::min(p, q);
+        nb.hi = std::max(p, q);
+        if (nb.lo < INT32_MIN || nb.hi > INT32_MAX) nb = Bound();   // the product may wrap
+      } else if (c.inputs.size() != 1 || !ChainStage(c, &st, &nb)) {
+        break;
+      }
       chain->stage[chain->count++] = st;
       *bound = nb;
       absorbed[cn] = true;

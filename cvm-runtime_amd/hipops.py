@@ -306,7 +306,8 @@ class Chain(ctypes.Structure):
 
 
 def chain(*stages):
-    """stages: ("relu",) | ("cvm_right_shift", precision, shift_bit) | ("cvm_clip", precision) | ("clip", lo, hi)"""
+    """stages: ("relu",) | ("cvm_right_shift", precision, shift_bit) | ("cvm_clip", precision) | ("clip", lo, hi)
+    | ("mul", m)"""
     c = Chain()
     c.count = len(stages)
     for i, st in enumerate(stages):
@@ -319,6 +320,8 @@ def chain(*stages):
             c.stage[i] = Stage(3, 0, 0, -r, r)
         elif st[0] == "clip":
             c.stage[i] = Stage(3, 0, 0, st[1], st[2])
+        elif st[0] == "mul":
+            c.stage[i] = Stage(4, 0, 0, st[1], 0)
         else:
             raise ValueError(st)
     return c

@@ -222,12 +222,13 @@ int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, 
  * channels, each stored as the 1 KiB operand fragment of v_mfma_i32_32x32x32_i8:
  *   offset(p, c) = ((p/32)*(cp/32) + c/32)*1024 + ((c/16)%2)*512 + (p%32)*16 + c%16
  * A buffer for npix pixels has cvmhip_packed_act_bytes(npix, c) bytes, 16-byte aligned. */
-enum { CVMHIP_STAGE_RELU = 1, CVMHIP_STAGE_RSHIFT = 2, CVMHIP_STAGE_CLIP = 3 };
+enum { CVMHIP_STAGE_RELU = 1, CVMHIP_STAGE_RSHIFT = 2, CVMHIP_STAGE_CLIP = 3, CVMHIP_STAGE_MUL = 4 };
 typedef struct {
   int32_t kind;        /* CVMHIP_STAGE_* */
   int32_t precision;   /* RSHIFT */
   int32_t shift_bit;   /* RSHIFT */
-  int32_t lo, hi;      /* CLIP: max(min(v, hi), lo) */
+  int32_t lo, hi;      /* CLIP: max(min(v, hi), lo).  MUL: v * lo, wrapping (broadcast_mul by a constant scalar,
+                          the requantisation scale in front of a cvm_right_shift; broadcast.cc:75-86) */
 } cvmhip_stage;
 typedef struct {
   int32_t count;       /* 0..4 stages, applied in order to the int32 value */

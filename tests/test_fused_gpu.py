@@ -38,6 +38,8 @@ def run_chain(v, stages):
             v = oracle.cvm_right_shift(v, st[1], st[2])
         elif st[0] == "cvm_clip":
             v = oracle.cvm_clip(v, st[1])
+        elif st[0] == "mul":
+            v = oracle.broadcast("broadcast_mul", v, np.array([st[1]], np.int32))
         else:
             v = oracle.clip(v, st[1], st[2])
     return v
@@ -81,6 +83,9 @@ FUSED_CONV = [
     (1, 16, 6, 6, 20, 3, 1, 1, True, [("cvm_right_shift", 8, 31)], None, True),          # shift regime b >= 31
     (1, 16, 6, 6, 20, 3, 1, 1, True, [("cvm_right_shift", 8, 24), ("cvm_clip", 8)], None, True),  # regime p + b >= 32
     (16, 512, 7, 7, 512, 3, 1, 1, True, [("relu",), ("cvm_right_shift", 8, 12)], None, True),      # deep K (4608), few pixels
+    (2, 64, 9, 9, 48, 3, 1, 1, True, [("relu",), ("mul", 93), ("cvm_right_shift", 8, 17)], None, True),   # scale then shift
+    (1, 32, 8, 8, 32, 1, 1, 0, True, [("mul", -70001), ("cvm_right_shift", 8, 20), ("cvm_clip", 8)],
+     [("mul", 3), ("cvm_right_shift", 8, 2)], True),                                               # products that wrap
     (4, 1024, 14, 14, 256, 1, 1, 0, False, [("relu",), ("cvm_right_shift", 8, 11)], None, True),
 ]
 
@@ -440,3 +445,47 @@ def test_storage_shared_by_liveness_is_not_clobbered_by_early_writes(dev):
     for mode in ("0", "1"):
         got = np.frombuffer(outs[mode], np.int32 if tsize == 4 else np.int8).astype(np.int32)
         assert np.array_equal(got, want), "planner %s" % ("on" if mode == "1" else "off")
+
+
+def test_requantisation_scale_is_folded_into_the_chain(dev):
+    """conv2d -> relu -> broadcast_mul(constant scalar) -> cvm_right_shift (the scale-then-shift form of a
+    requantisation), the same behind a residual add, and behind the global sum: all folded into the
+    producing launch, equal to node-by-node execution and to the oracle."""
+    g = graphgen.GraphBuilder("scale-chain")
+    x = g.var("data", (2, 3, 20, 20), 8)
+
+    def scaled(v, m, shift, name):
+        s = g.param(name, (1,), m, m, int(abs(m)).bit_length() + 1, np.int32)
+        (y,) = g.op("broadcast_mul", [v, s], {}, [g.shape(v)])
+        return g.clip8(g.rshift(y, shift))
+
+    c1, _ = g.conv(x, 32, 3, 1, 1)
+    a = scaled(g.relu(c1), 77, 18, "scale1")
+    c2, _ = g.conv(a, 32, 3, 1, 1)
+    b = scaled(g.relu(c2), 20, 19, "scale2")
+    c3, _ = g.conv(b, 32, 1, 1, 0)
+    r = scaled(c3, -100, 19, "scale3")                       # negative scale, no relu
+    (added,) = g.op("elemwise_add", [r, a], {}, [g.shape(a)])
+    z = scaled(added, 3, 2, "scale4")
+    (gap,) = g.op("sum", [z], {"axis": "(2, 3)"}, [(2, 32)])
+    out = scaled(gap, 5, 9, "scale5")
+    d, _ = g.dense(out, 10)
+    js, pb = g.build([d])
+    xv = synth.tensor("scale-chain", "data", (2, 3, 20, 20), -127, 127)
+    outs = {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_FUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(xv.astype(np.int8).tobytes())
+            if mode == "1":
+                labels = m.profile_ops()
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FUSE", None)
+    assert "broadcast_mul" not in labels and "cvm_right_shift" not in labels, labels
+    assert outs["1"] == outs["0"]
+    ref = og.run_graph(js, graphgen.load_params(pb), xv)
+    got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
