@@ -130,10 +130,9 @@ __global__ void __launch_bounds__(256) k_zero32(int32_t* __restrict__ p, int64_t
 // not depend on their order.
 __global__ void __launch_bounds__(256)
 k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
-           const int32_t* __restrict__ need_full, int n, int k, int score_index) {
+           int n, int k, int score_index) {
   __shared__ __attribute__((aligned(16))) int32_t tile[RANK_JT];
   const int b = blockIdx.z;
-  if (need_full && need_full[b] == 0) return;  // k_nms_topk_rank has ranked this batch
   if (batch_state(valid_count, b, n) != 0) return;
   const int vc = clamp_vc(valid_count[b], n);
   const int base = blockIdx.y * RANK_JT;
@@ -160,36 +159,32 @@ k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_coun
   if (i < vc && r) atomicAdd(&rank[(int64_t)b * n + i], r);
 }
 
-// With 0 < top_k < valid rows only the top_k best rows are ever looked at again, so only they need a
+// With 0 < top_k <= TOPK_MAX_K only the top_k best rows are ever looked at again, so only they need a
 // rank.  One workgroup per batch keeps every score in registers (thread t owns rows t, t + 1024, ...),
 // finds the top_k-th largest score T by bisection on the bits in which scores differ (ballot counts, no
 // atomics on data), and ranks: rows above T among themselves (fewer than top_k; listed in LDS as
 // (score, ~index) words so one 64-bit compare orders them as the stable sort would); rows equal to T
 // by their position among the equal rows in index order; every other row gets the marker rank top_k,
-// which only says "not among the first top_k".  When the condition does not hold the batch is handed
-// to k_nms_rank (need_full = 1, ranks zeroed).  All counts are integers, so the result is exact.
+// which only says "not among the first top_k".  With top_k >= valid rows every row is ranked in the list.
+// All counts are integers, so the result is exact.
 constexpr int TOPK_THREADS = 1024, TOPK_ROWS = 32, TOPK_WAVES = TOPK_THREADS / 64;  // rows per thread
 constexpr int TOPK_MAX_N = TOPK_THREADS * TOPK_ROWS, TOPK_MAX_K = 2048;
 
 __global__ void __launch_bounds__(TOPK_THREADS)
 k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
-                int32_t* __restrict__ need_full, int n, int k, int score_index, int topk) {
+                int n, int k, int score_index, int topk) {
   __shared__ __attribute__((aligned(16))) unsigned long long s_comp[TOPK_MAX_K];
   __shared__ int s_cnt[TOPK_MAX_K];
   __shared__ int s_tab[TOPK_ROWS * TOPK_WAVES], s_part[2][TOPK_WAVES], s_wsum[TOPK_WAVES];
   __shared__ uint32_t s_and[TOPK_WAVES], s_or[TOPK_WAVES];
   __shared__ int s_gcount;
   const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) need_full[b] = 0;
   if (batch_state(valid_count, b, n) != 0) return;
   const int vc = clamp_vc(valid_count[b], n);
   const int R = (vc + TOPK_THREADS - 1) / TOPK_THREADS;
   int32_t* rk = rank + (int64_t)b * n;
-  if (!(topk > 0 && topk < vc)) {  // every valid row needs its rank: the all-pairs kernel adds them up from zero
-    for (int i = tid; i < vc; i += TOPK_THREADS) rk[i] = 0;
-    if (tid == 0) need_full[b] = 1;
-    return;
-  }
+  // top_k >= valid rows (at most TOPK_MAX_K of them then): every row is "above" and is ranked in the list
+  const bool all = topk >= vc;
   const int32_t* xb = x + (int64_t)b * n * k;
   for (int i = tid; i < TOPK_MAX_K; i += TOPK_THREADS) { s_cnt[i] = 0; s_comp[i] = 0; }
   if (tid == 0) s_gcount = 0;
@@ -221,7 +216,7 @@ k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid
   const int top_bit = diff ? 31 - __clz((int)diff) : -1;
   // T becomes the top_k-th largest key: the largest T with at least top_k keys >= T
   uint32_t T = top_bit >= 0 ? (kor & ~((2u << top_bit) - 1u)) : kor;
-  for (int bit = top_bit; bit >= 0; --bit) {
+  for (int bit = all ? -1 : top_bit; bit >= 0; --bit) {
     const uint32_t cand = T | (1u << bit);
     int c = 0;
 #pragma unroll
@@ -244,8 +239,8 @@ k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid
   for (int r = 0; r < TOPK_ROWS; ++r) {
     if (r >= R) break;
     const int i = r * TOPK_THREADS + tid;
-    const bool up = key[r] > T;
-    const unsigned long long bu = __ballot(up), be = __ballot(i < vc && key[r] == T);
+    const bool up = all ? i < vc : key[r] > T;
+    const unsigned long long bu = __ballot(up), be = __ballot(!all && i < vc && key[r] == T);
     int base = 0;
     if (lane == 0) {
       s_tab[r * TOPK_WAVES + wave] = __popcll(be);
@@ -296,9 +291,9 @@ k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid
   for (int r = 0; r < TOPK_ROWS; ++r) {
     if (r >= R) break;
     const int i = r * TOPK_THREADS + tid;
-    const bool eq = i < vc && key[r] == T;
+    const bool eq = !all && i < vc && key[r] == T;
     const unsigned long long be = __ballot(eq);
-    if (i >= vc || key[r] > T) continue;
+    if (all || i >= vc || key[r] > T) continue;
     if (eq) {
       const int e = s_tab[r * TOPK_WAVES + wave] + __popcll(be & lt);
       rk[i] = e < from_equal ? g + e : topk;
@@ -550,7 +545,7 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
   return check_launch("get_valid_counts.scatter");
 }
 
-// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix, one flag
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
   return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 2 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS) * sizeof(int32_t);
 }
@@ -574,19 +569,16 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
   int32_t* sorted = removed + (size_t)batches * n;
   int32_t* rank = sorted + (size_t)batches * n * k;
   uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
-  int32_t* need_full = reinterpret_cast<int32_t*>(mask + (size_t)batches * NMS_BM_ROWS * NMS_BM_WORDS);
-  const bool select_first = topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N;
   int rc;
-  if (select_first) {
-    k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, need_full, n, k, score_index, topk);
+  if (topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N) {
+    k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, n, k, score_index, topk);
     rc = check_launch("nms.topk_rank");
-    if (rc) return rc;
   } else {
     k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
+    dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
+    k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, n, k, score_index);
+    rc = check_launch("nms.rank");
   }
-  dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
-  k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, select_first ? need_full : nullptr, n, k, score_index);
-  rc = check_launch("nms.rank");
   if (rc) return rc;
   dim3 grid((n + 255) / 256, batches);
   k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, y, n, k, topk, (int64_t)n);

@@ -296,7 +296,9 @@ def test_non_max_suppression(case, dev):
                                           ((-3, 3), 300, 4000),                   # long runs of equal scores around the cut
                                           ((2 ** 31 - 5, 2 ** 31 - 1), 2048, 3000),  # the largest top_k of the selection path
                                           ((-2 ** 31, -2 ** 31 + 2), 2049, 3000),    # one more: all-pairs ranking
-                                          ((0, 1000), 1, 700)])
+                                          ((0, 1000), 1, 700),
+                                          ((-50, 50), 400, 300),                  # top_k above the row count: every row ranked in the list
+                                          ((-2 ** 31, 2 ** 31 - 1), 2048, 2048)]) # ... with the list full
 def test_nms_top_k_selection(score, topk, n, dev):
     """Rows past top_k only need to be known as such; the first top_k must come out in the stable-sort order."""
     x = _boxes("nms-topk-%s-%d" % (score, topk), 2, n, -1, 3, score=score, extent=256)
