@@ -289,7 +289,6 @@ void HipGraphRuntime::BuildPlan() {
     const uint32_t ce = entry_id(cn, 0);
     // the slice is written long before the concatenate node's place in the order
     privatize(ce);
-    st->aux = own_storage[ce];
     st->nhwc = true;
     st->dst = ce;
     st->dst_off = before * inner;
