@@ -447,6 +447,8 @@ void HipGraphRuntime::Release() {
   if (i8_slab_) { cvmhip_free(i8_slab_); i8_slab_ = nullptr; }
   if (in_stage_dev_) { cvmhip_free(in_stage_dev_); in_stage_dev_ = nullptr; }
   if (in_stage_host_) { cvmhip_host_free(in_stage_host_); in_stage_host_ = nullptr; }
+  if (out_stage_host_) { cvmhip_host_free(out_stage_host_); out_stage_host_ = nullptr; }
+  out_host_.clear();
   if (stream_) cvmhip_stream_sync(stream_);
   own_storage_.clear();
   if (workspace_) cvmhip_free(workspace_);
@@ -727,6 +729,26 @@ void HipGraphRuntime::CopyOutputTo(int index, int32_t* host) {
   const uint32_t eid = entry_id(outputs_[index]);
   HipCheck(cvmhip_copy_d2h(host, entry_ptr_[eid], static_cast<size_t>(shape_size(shape_[eid])) * 4, stream_), "copy output");
   HipCheck(cvmhip_stream_sync(stream_), "copy output");
+}
+
+const std::vector<const int32_t*>& HipGraphRuntime::FetchOutputs() {
+  if (!out_stage_host_) {
+    size_t total = 0;
+    for (const NodeEntry& e : outputs_) total += AlignUp(static_cast<size_t>(shape_size(shape_[entry_id(e)])) * 4, 64);
+    HipCheck(cvmhip_host_alloc(&out_stage_host_, std::max<size_t>(total, 64)), "output staging buffer");
+    size_t off = 0;
+    for (const NodeEntry& e : outputs_) {
+      out_host_.push_back(reinterpret_cast<const int32_t*>(static_cast<char*>(out_stage_host_) + off));
+      off += AlignUp(static_cast<size_t>(shape_size(shape_[entry_id(e)])) * 4, 64);
+    }
+  }
+  for (size_t k = 0; k < outputs_.size(); ++k) {
+    const uint32_t eid = entry_id(outputs_[k]);
+    HipCheck(cvmhip_copy_d2h(const_cast<int32_t*>(out_host_[k]), entry_ptr_[eid], static_cast<size_t>(shape_size(shape_[eid])) * 4,
+                             stream_), "copy output");
+  }
+  HipCheck(cvmhip_stream_sync(stream_), "copy output");
+  return out_host_;
 }
 
 int32_t* HipGraphRuntime::DataDevicePtr() {

@@ -120,6 +120,8 @@ class HipGraphRuntime {
   void Run();      // replays the captured graph once it exists
   void Launch();   // issues every launch of a run on the stream, one by one
   void CopyOutputTo(int index, int32_t* host);  // synchronises the stream
+  // every output copied into pinned host memory owned by the runtime (valid until the next call); one synchronisation
+  const std::vector<const int32_t*>& FetchOutputs();
 
   // device-resident variants used to time Run() alone
   int32_t* DataDevicePtr();
@@ -180,6 +182,8 @@ class HipGraphRuntime {
   void* stream_ = nullptr;
   void* in_stage_host_ = nullptr;  // pinned staging copy of an int8 input
   void* in_stage_dev_ = nullptr;   // its device copy before widening
+  void* out_stage_host_ = nullptr; // pinned copies of the outputs, back to back
+  std::vector<const int32_t*> out_host_;
   std::vector<int32_t*> entry_ptr_;
   struct Exec { uint32_t nid; const OpKernel* kernel; OpCall call; };
   std::vector<Exec> execs_;

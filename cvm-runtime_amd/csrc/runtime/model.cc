@@ -59,22 +59,17 @@ void HipModel::SetInput(const void* input, int size) {
 }
 
 void HipModel::GetOutput(char* mem) {
-  std::vector<std::vector<int32_t>> outs(out_num_);
-  for (int k = 0; k < out_num_; ++k) {
-    outs[k].resize(static_cast<size_t>(out_size_[k]));
-    rt_->CopyOutputTo(k, outs[k].data());
-  }
-  SaveTensor(outs, mem);
+  SaveTensor(rt_->FetchOutputs(), mem);   // all heads in pinned host memory, one synchronisation
 }
 
 // model.cc:181-263, restated including its loop bounds
-void HipModel::SaveTensor(const std::vector<std::vector<int32_t>>& outputs, char* mem) const {
+void HipModel::SaveTensor(const std::vector<const int32_t*>& outputs, char* mem) const {
   if (postprocess_ == "argmax") {
     int32_t* cp = reinterpret_cast<int32_t*>(mem);
     for (int k = 0; k < out_num_; ++k) {
       const uint32_t last_dim = static_cast<uint32_t>(out_shape_[k].back());
       const uint32_t rows = static_cast<uint32_t>(out_size_[k]) / last_dim;
-      const int32_t* data = outputs[k].data();
+      const int32_t* data = outputs[k];
       // the row cursor advances by last_dim while bounded by the row count
       for (size_t i = 0; i < rows; i += last_dim) {
         uint32_t max_id = 0;
@@ -100,21 +95,21 @@ void HipModel::SaveTensor(const std::vector<std::vector<int32_t>>& outputs, char
       const int32_t nx = static_cast<int32_t>(xs[0]);
       for (int x = 0; x < nx; ++x)
         for (size_t k = 0; k < outputs.size(); ++k) {
-          const int32_t* row = outputs[k].data() + static_cast<size_t>(x) * ys[k];
+          const int32_t* row = outputs[k] + static_cast<size_t>(x) * ys[k];
           for (size_t i = 0; i < ys[k]; ++i) *cp++ = row[i];
         }
     } else {
       char* cp = mem;
       for (size_t x = 0; x < xs[0]; ++x)
         for (size_t k = 0; k < outputs.size(); ++k) {
-          const int32_t* row = outputs[k].data() + x * ys[k];
+          const int32_t* row = outputs[k] + x * ys[k];
           for (size_t i = 0; i < ys[k]; ++i) *cp++ = static_cast<int8_t>(row[i]);
         }
     }
   } else if (output_bytes_ == 4) {
     int32_t* ref = reinterpret_cast<int32_t*>(mem);
     for (size_t k = 0; k < outputs.size(); ++k) {
-      std::memcpy(ref, outputs[k].data(), sizeof(int32_t) * static_cast<size_t>(out_size_[k]));
+      std::memcpy(ref, outputs[k], sizeof(int32_t) * static_cast<size_t>(out_size_[k]));
       ref += out_size_[k];
     }
   } else {

@@ -32,7 +32,7 @@ class HipModel {
   HipGraphRuntime* runtime() { return rt_.get(); }
 
  private:
-  void SaveTensor(const std::vector<std::vector<int32_t>>& outputs, char* mem) const;
+  void SaveTensor(const std::vector<const int32_t*>& outputs, char* mem) const;
   std::unique_ptr<HipGraphRuntime> rt_;
   int64_t in_size_ = 0;
   std::vector<int64_t> out_size_;
