@@ -46,33 +46,32 @@ __device__ __forceinline__ int32_t clamp3(int32_t v, int32_t lo, int32_t hi) {
   return r;
 }
 
-// A requantisation chain over N values held in registers, stage by stage: the
-// stage parameters are wave-uniform, so a stage costs four vector instructions
-// per value.  The stages are copied to scalar registers first; indexing the
-// kernel argument with the loop counter would move it to private memory.
+// A requantisation chain over N values held in registers.  The stage parameters are wave-uniform
+// (scalar registers), so a stage costs one instruction per value for the clamp and two for the
+// rounding shift.  Straight-line code over the (at most four) stages, each part of a stage an update
+// in place under a wave-uniform condition: a loop over the stages, or alternative forms of a stage
+// that meet at a join, make the compiler copy all N registers from one set to another at every edge
+// (measured: 40 % of the vector instructions of an epilogue were such copies).
 template <int N>
 __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
-  const DevStage q0 = c.st[0], q1 = c.st[1], q2 = c.st[2], q3 = c.st[3];
-#pragma unroll 1
-  for (int t = 0; t < c.count; ++t) {
-    const int32_t lo = t == 0 ? q0.lo : t == 1 ? q1.lo : t == 2 ? q2.lo : q3.lo;
-    const int32_t hi = t == 0 ? q0.hi : t == 1 ? q1.hi : t == 2 ? q2.hi : q3.hi;
-    const int32_t s1 = t == 0 ? q0.s1 : t == 1 ? q1.s1 : t == 2 ? q2.s1 : q3.s1;
-    const int32_t ad = t == 0 ? q0.add : t == 1 ? q1.add : t == 2 ? q2.add : q3.add;
-    const int32_t s2 = t == 0 ? q0.s2 : t == 1 ? q1.s2 : t == 2 ? q2.s2 : q3.s2;
-    const int32_t mu = t == 0 ? q0.mul : t == 1 ? q1.mul : t == 2 ? q2.mul : q3.mul;
-    if (mu != 1) {   // a multiplication stage (rare: one more instruction per value)
 #pragma unroll
-      for (int e = 0; e < N; ++e) v[e] = wadd(wmul(clamp3(v[e], lo, hi), mu) >> s1, ad) >> s2;
-    } else if ((s1 | ad | s2) == 0) {
+  for (int t = 0; t < 4; ++t) {
+    if (t < c.count) {
+      const DevStage q = c.st[t];
 #pragma unroll
-      for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], lo, hi);
-    } else if (s1 == 0) {
+      for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], q.lo, q.hi);
+      if (q.mul != 1) {   // a multiplication stage (rare)
 #pragma unroll
-      for (int e = 0; e < N; ++e) v[e] = wadd(clamp3(v[e], lo, hi), ad) >> s2;
-    } else {
+        for (int e = 0; e < N; ++e) v[e] = wmul(v[e], q.mul);
+      }
+      if (q.s1 != 0) {
 #pragma unroll
-      for (int e = 0; e < N; ++e) v[e] = wadd(clamp3(v[e], lo, hi) >> s1, ad) >> s2;
+        for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s1;
+      }
+      if ((q.add | q.s2) != 0) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = wadd(v[e], q.add) >> q.s2;
+      }
     }
   }
 }
