@@ -180,6 +180,9 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   const bool whole = blocked && (NG % 4 == 0);   // whole tiles: 16 bytes per lane
   const bool halves = blocked && NG == 2;         // half a tile (q pair): 8 bytes per lane
 
+  // one copy of each step, the residual part an update in place under a uniform condition (two
+  // alternative paths that meet again cost a register-to-register copy of every value)
+  run_chain(ep.chain, val);
   if (ep.residual) {   // rp holds what load_residual fetched
     if (whole) {
 #pragma unroll
@@ -190,12 +193,9 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
         rp[t * 4] = a; rp[t * 4 + 1] = c; rp[t * 4 + 2] = b; rp[t * 4 + 3] = d;
       }
     }
-    run_chain(ep.chain, val);
 #pragma unroll
     for (int e = 0; e < NG * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
     run_chain(ep.chain2, val);
-  } else {
-    run_chain(ep.chain, val);
   }
 
   if (OUT == OUT_I32_NCHW) {
@@ -225,8 +225,9 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       half_swap(a, c);   // lower half wave: channels 0..15 of the tile, upper: 16..31
       half_swap(b, d);
       uint32_t w[4] = {a, c, b, d};
-      const int first = oc0 + ch_wave + ((u0 >> 2) + t) / TN * 32 + lgrp * 16;
-      mask_channels(w, first, g.OC);
+      const int tile_first = oc0 + ch_wave + ((u0 >> 2) + t) / TN * 32;   // same for every lane
+      const int first = tile_first + lgrp * 16;
+      if (tile_first + 32 > g.OC) mask_channels(w, first, g.OC);          // only the last tile of a ragged channel count
       const int p = px_wave + gj[t * 4] * 32 + lrow;
       if (p < P && first < ocp) *reinterpret_cast<int4*>(y8 + block_off(t * 4) + lane * 16) = make_int4(w[0], w[1], w[2], w[3]);
     }
