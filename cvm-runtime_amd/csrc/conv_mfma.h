@@ -43,6 +43,8 @@ struct ConvGeom {
   int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
   FastDiv div_ohw, div_ow, div_ct, div_kw;  // filled by conv_igemm: division by OH*OW, OW, Cp/32 and KW
   int row_bytes;           // > 0: row-window input (see stem_* below): bytes of K per filter row, 16 or 32
+  int octiles;             // filled by conv_igemm for the wavefront kernel: channel tiles of the grid, and division by it
+  FastDiv div_octiles;
 };
 
 // What happens to an accumulator before it is stored:

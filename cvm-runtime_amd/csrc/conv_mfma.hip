@@ -500,9 +500,8 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   int pid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
-  const int oc_tiles = (g.OC + BM - 1) / BM;
-  const int ptile = pid / oc_tiles;
-  const int oc0 = (pid - ptile * oc_tiles) * BM;
+  const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);   // g.octiles = ceil(OC / BM), set by the host for this tile
+  const int oc0 = (pid - ptile * g.octiles) * BM;
   const int px0 = ptile * BN;              // P < 2^31 is checked on the host
   const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
@@ -570,15 +569,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
   for (int j = 0; j < TN; ++j) { tapptr[j] = zero; okv[j] = 0; }
 
-  stage_bias<BM>(sBias, ep, g.OC, oc0, tid);
-
-  v16i acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+  v16i acc[TM][TN];   // first written by the first MFMA of each tile, whose addend is the constant 0
 
   // one batch = D chunks of both operands, one SSA value (see k_conv_igemm)
   typedef int regs_t __attribute__((ext_vector_type(4 * (TM + TN) * D)));
@@ -656,7 +647,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
     }
     return R;
   };
-  auto consume = [&](const regs_t R) __attribute__((always_inline)) {
+  auto consume = [&](const regs_t R, const bool first) __attribute__((always_inline)) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       v4i a[TM], b[TN];
@@ -670,26 +661,35 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
         const int o = (d * (TM + TN) + TM + j) * 4;
         b[j] = v4i{R[o], R[o + 1], R[o + 2], R[o + 3]};
       }
+      const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], (first && d == 0) ? zero16 : acc[i][j], 0, 0, 0);
     }
   };
 
-  // the residual of the groups this wavefront will finalise travels with the first operands
+  // Order of the requests: operands of the first batch, then what is only needed after the K loop --
+  // the residual of the groups this wavefront will finalise and the bias (kept in a register and
+  // staged in LDS after the loop; staging it here would put a full memory latency in front of the
+  // first operand request).
+  regs_t R0 = fetch();
   uint32_t rp[NU];
   if (ep.residual) load_residual<TN, NU>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+  int bias_mine = 0;
+  if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
 
-  regs_t R0 = fetch();
-  regs_t R1;
-  for (int it = 0; it < niter; it += 2) {
-    R1 = fetch();
-    consume(R0);
-    if (it + 1 >= niter) break;
+  regs_t R1 = fetch();
+  consume(R0, true);
+  for (int it = 1; it < niter; it += 2) {
     R0 = fetch();
-    consume(R1);
+    consume(R1, false);
+    if (it + 1 >= niter) break;
+    R1 = fetch();
+    consume(R0, false);
   }
+  if (tid < BM) sBias[tid] = bias_mine;
 
   // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
   // wavefront kw_ then finalises the groups kw_*NU .. kw_*NU + NU-1 of the tile set
@@ -1122,6 +1122,8 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
                                 ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
+    g.octiles = (g.OC + 32 * kWaveCfgs[cfg].tm - 1) / (32 * kWaveCfgs[cfg].tm);
+    g.div_octiles = make_fastdiv((uint32_t)g.octiles);
     KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
     launch_wave(cfg, mode, (unsigned)wnb, s, xp, wp, out, g, ep);
     return check_launch("conv_wave");
