@@ -578,21 +578,28 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   };
   auto fetch = [&]() __attribute__((always_inline)) -> regs_t {
     regs_t R;
-    if (MODE == WAVE_IDENT && cur + D <= c_end) {
-      // whole batch inside the range: one pointer per operand block, chunks at constant offsets
+    if (MODE == WAVE_IDENT) {
+      // One path, loads always in the same order (filter blocks, then pixel blocks; the chunks of a
+      // block together): with alternative paths that issue them in different orders the compiler
+      // no longer knows how many younger loads may stay outstanding and drains them all before
+      // every MFMA group.  A chunk past the end multiplies the all-zero filter chunk with a valid
+      // activation address.
+      int ca[D], cb[D];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int8_t* pa = wa[i] + (int64_t)cur * 1024;
-#pragma unroll
-        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(pa + d * 1024));
+      for (int d = 0; d < D; ++d) {
+        const bool live = cur + d < c_end;
+        ca[d] = live ? cur + d : nch;
+        cb[d] = live ? cur + d : (c_begin < nlive ? c_begin : 0);
       }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int8_t* pb = xb[j] + (int64_t)cur * 1024;
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(pb + d * 1024));
-      }
-      cur += D;
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)ca[d] * 1024));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb[d] * 1024));
+      cur = cur + D < c_end ? cur + D : c_end;
       return R;
     }
 #pragma unroll
@@ -602,11 +609,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       const int chunk = live ? cur : nch;
 #pragma unroll
       for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024));
-      if (MODE == WAVE_IDENT) {
-        const int cb = live ? cur : c_begin < nlive ? c_begin : 0;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb * 1024));
-      } else if (MODE == WAVE_ROWS) {
+      if (MODE == WAVE_ROWS) {
         // 16-byte unit k16 of K: filter row k16 / (row_bytes/16), part k16 % (row_bytes/16) of its window
         const int k16 = (live ? cur : 0) * 2 + lgrp;
         const int sh16 = g.row_bytes >> 5;   // 0 or 1
@@ -634,7 +637,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       }
       if (live) {
         ++cur;
-        if (MODE != WAVE_IDENT && MODE != WAVE_ROWS) {
+        if (MODE != WAVE_ROWS) {
           ch += 32;
           if (ch >= g.Cp) {
             ch = 0;
@@ -670,13 +673,14 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
     }
   };
 
-  // Order of the requests: operands of the first batch, then what is only needed after the K loop --
-  // the residual of the groups this wavefront will finalise and the bias (kept in a register and
-  // staged in LDS after the loop; staging it here would put a full memory latency in front of the
-  // first operand request).
-  regs_t R0 = fetch();
+  // Order of the requests: the residual of the groups this wavefront will finalise (nothing waits for
+  // it before the epilogue; requested after the operands, its predicated form makes the compiler drain
+  // every outstanding load first), the operands of the first batch, then the bias, which is kept in a
+  // register and staged in LDS after the loop (staging it here would put a full memory latency in
+  // front of the first operand request).
   uint32_t rp[NU];
   if (ep.residual) load_residual<TN, NU>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+  regs_t R0 = fetch();
   int bias_mine = 0;
   if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
 
