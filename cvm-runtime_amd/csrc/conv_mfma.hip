@@ -455,6 +455,25 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   finish_groups<WN, WM * WN * 4, OUT>(val, 0, sBias, wm * WM * 32, oc0, (int)px0 + wn * WN * 32, lane, out, g, ep, rp);
 }
 
+// Bit t set when filter tap t (of k <= 32) of a receptive field that starts at input coordinate x0
+// lies inside [0, extent).  Without dilation the valid taps are the run max(0, -x0) ..
+// min(k - 1, extent - 1 - x0), which needs no loop and no branch.
+__device__ __forceinline__ unsigned tap_mask_dense(int x0, int extent, int k) {
+  int lo = x0 < 0 ? -x0 : 0;
+  int hi = extent - 1 - x0;
+  hi = hi < k - 1 ? hi : k - 1;
+  const bool any = hi >= lo;
+  lo = lo < 31 ? lo : 31;
+  hi = hi > 0 ? hi : 0;
+  const unsigned m = ((2u << hi) - 1u) & ~((1u << lo) - 1u);
+  return any ? m : 0u;
+}
+__device__ __forceinline__ unsigned tap_mask_dilated(int x0, int extent, int k, int d) {
+  unsigned m = 0;
+  for (int t = 0; t < k; ++t) m |= ((unsigned)(x0 + t * d) < (unsigned)extent ? 1u : 0u) << t;
+  return m;
+}
+
 // ---------------------------------------------------------------- wavefront-private kernel
 // Layers whose grid is small (few pixels, deep K) are bound by latency, not by
 // MFMA rate: with one wavefront per SIMD every instruction pays its full
@@ -533,8 +552,13 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       xb[j] = xp;
       unsigned rm = 0, cm = 0;
       if (MODE == WAVE_PAD) {
-        for (int t = 0; t < g.KH; ++t) rm |= ((unsigned)(ih0 + t * g.DH) < (unsigned)g.H ? 1u : 0u) << t;
-        for (int t = 0; t < g.KW; ++t) cm |= ((unsigned)(iw0 + t * g.DW) < (unsigned)g.W ? 1u : 0u) << t;
+        if (g.DH == 1 && g.DW == 1) {
+          rm = tap_mask_dense(ih0, g.H, g.KH);
+          cm = tap_mask_dense(iw0, g.W, g.KW);
+        } else {
+          rm = tap_mask_dilated(ih0, g.H, g.KH, g.DH);
+          cm = tap_mask_dilated(iw0, g.W, g.KW, g.DW);
+        }
         rm = ok ? rm : 0u;
       }
       rowmask[j] = rm;
@@ -625,7 +649,13 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
           for (int j = 0; j < TN; ++j) {
             const int pin = rowbase[j] + soff;
             const bool ok = MODE != WAVE_PAD || ((((rowmask[j] >> r) & (colmask[j] >> s)) & 1u) != 0);
-            tapptr[j] = ok ? xp + ((int64_t)((pin >> 5) * ctiles) * 1024 + ((pin & 31) << 4) + lconst) : zero;
+            // Byte offset of the pixel's granule: block (pin / 32) * Cp * 32 + row (pin % 32) * 16.  The tensor
+            // is smaller than 2^31 bytes (checked by the host), so a 24-bit multiply (full rate) is exact; for a
+            // tap outside the image the offset is meaningless and the select below discards it -- a select, not
+            // a branch, so that the two pointers cost a dozen instructions per tap instead of fifty.
+            const unsigned off = __umul24((unsigned)pin >> 5, (unsigned)g.Cp << 5) + (((unsigned)pin & 31u) << 4) + (unsigned)lconst;
+            const int8_t* inside = xp + off;
+            tapptr[j] = ok ? inside : zero;
             okv[j] = ok ? 1 : 0;
           }
           need_tap = false;
