@@ -87,6 +87,11 @@ FUSED_CONV = [
     (1, 32, 8, 8, 32, 1, 1, 0, True, [("mul", -70001), ("cvm_right_shift", 8, 20), ("cvm_clip", 8)],
      [("mul", 3), ("cvm_right_shift", 8, 2)], True),                                               # products that wrap
     (4, 1024, 14, 14, 256, 1, 1, 0, False, [("relu",), ("cvm_right_shift", 8, 11)], None, True),
+    # tap masks at their limits: a 32-tap filter side (bit 31 of the mask), and padding wider than the
+    # filter so that whole receptive fields lie outside the image
+    (1, 32, 8, 8, 32, 32, 1, 12, True, [("cvm_right_shift", 8, 14)], None, True),
+    (2, 64, 5, 5, 64, 3, 1, 5, True, [("cvm_right_shift", 8, 9)], None, True),
+    (1, 32, 6, 6, 64, 3, 2, 40, True, [("cvm_right_shift", 8, 9)], None, True),
 ]
 
 
