@@ -515,6 +515,15 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kw_ = wave % KSPLIT, pw_ = wave / KSPLIT;
   const int lrow = lane & 31, lgrp = lane >> 5;
+  // After a K split a wavefront finalises the groups kw_*NU .. kw_*NU + NU-1 of the workgroup's tile
+  // set.  It computes them in its register groups 0 .. NU-1: register group u (tile u / 4, quarter
+  // u % 4) holds the workgroup's group u ^ G, G = kw_ * NU.  The own groups then never travel through
+  // LDS and every register index is still a constant; the permutation costs nothing, because it only
+  // changes addresses: tiles are exchanged by swapping operand pointers (X), quarters of a tile by
+  // letting each lane fetch the filter row (lane ^ 8 Q) of its 32-row block.
+  const int G = KSPLIT > 1 ? kw_ * NU : 0;
+  const int X = G >> 2, Q = G & 3;
+  const int Xi = X / TN, Xj = X % TN;
 
   int pid = blockIdx.x;
   const int nb = gridDim.x;
@@ -533,13 +542,13 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     if (MODE == WAVE_IDENT) {
-      int t = (px0 >> 5) + pw_ * TN + j;
+      int t = (px0 >> 5) + pw_ * TN + (j ^ Xj);
       const int last = (P - 1) >> 5;
       t = t < last ? t : last;             // blocks past the tensor re-read its last block; their pixels are never stored
       xb[j] = xp + (int64_t)t * ctiles * 1024 + lane * 16;
       rowbase[j] = 0; rowmask[j] = 0; colmask[j] = 0;
     } else {
-      const int p = px0 + (pw_ * TN + j) * 32 + lrow;
+      const int p = px0 + (pw_ * TN + (j ^ Xj)) * 32 + lrow;
       const bool ok = p < P;
       const unsigned pp = ok ? (unsigned)p : 0u;
       const int n = (int)fastdiv(pp, g.div_ohw);
@@ -584,7 +593,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 
   const int8_t* wa[TM];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + i) * (nch + 1)) * 1024 + lane * 16;
+  for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + (i ^ Xi)) * (nch + 1)) * 1024 + (lane ^ (Q << 3)) * 16;
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   const int lconst = lgrp * 512;
   const int8_t* tapptr[TN];                // per-lane operand address of the current filter tap
@@ -731,20 +740,22 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   if (KSPLIT > 1) {
     int* mine = sPart + wave * U * 256;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<int4*>(mine + (((i * TN + j) * 4 + q) * 64 + lane) * 4) =
-              make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+    for (int u = NU; u < U; ++u) {   // the other wavefronts' groups
+      const int t = u >> 2, q = u & 3;
+      *reinterpret_cast<int4*>(mine + ((u ^ G) * 64 + lane) * 4) =
+          make_int4(acc[t / TN][t % TN][q * 4], acc[t / TN][t % TN][q * 4 + 1], acc[t / TN][t % TN][q * 4 + 2],
+                    acc[t / TN][t % TN][q * 4 + 3]);
+    }
     __syncthreads();
 #pragma unroll
-    for (int m = 0; m < NU; ++m) {
-      int4 sum = zero4();
+    for (int m = 0; m < NU; ++m) {   // own register group m = workgroup group G + m
+      const int t = m >> 2, q = m & 3;
+      int4 sum = make_int4(acc[t / TN][t % TN][q * 4], acc[t / TN][t % TN][q * 4 + 1], acc[t / TN][t % TN][q * 4 + 2],
+                           acc[t / TN][t % TN][q * 4 + 3]);
 #pragma unroll
-      for (int k = 0; k < KSPLIT; ++k) {
-        const int4 v = *reinterpret_cast<const int4*>(sPart + (((pw_ * KSPLIT + k) * U + kw_ * NU + m) * 64 + lane) * 4);
+      for (int d = 1; d < KSPLIT; ++d) {
+        const int k = (kw_ + d) % KSPLIT;
+        const int4 v = *reinterpret_cast<const int4*>(sPart + (((pw_ * KSPLIT + k) * U + G + m) * 64 + lane) * 4);
         sum.x = wadd(sum.x, v.x); sum.y = wadd(sum.y, v.y); sum.z = wadd(sum.z, v.z); sum.w = wadd(sum.w, v.w);
       }
       val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
