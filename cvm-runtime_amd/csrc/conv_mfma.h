@@ -43,6 +43,8 @@ struct ConvGeom {
   int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
   FastDiv div_ohw, div_ow, div_ct, div_kw;  // filled by conv_igemm: division by OH*OW, OW, Cp/32 and KW
   int row_bytes;           // > 0: row-window input (see stem_* below): bytes of K per filter row, 16 or 32
+  int dw;                  // 1: depthwise convolution through MFMA -- output channel tile t reads input channels 32t .. 32t+31 only,
+                           //    filter packed by pack_depthwise_diag (OC == C, Cp % 32 == 0)
   int octiles;             // filled by conv_igemm for the wavefront kernel: channel tiles of the grid, and division by it
   FastDiv div_octiles;
 };
@@ -120,6 +122,8 @@ int pack_stem_weights(const int32_t* w, int8_t* wp, int oc, int c, int kh, int k
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp);
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw);
 
+size_t packed_depthwise_diag_bytes(int c, int kh, int kw);
+int pack_depthwise_diag(const int32_t* w, int8_t* wp, int c, int kh, int kw, hipStream_t s);
 int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStream_t s);
 int unpack_activations(const int8_t* xp, int32_t* x, int n, int c, int hw, hipStream_t s);
 int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, hipStream_t s);

@@ -586,10 +586,13 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   int tap = 0, ch = 0, r = 0, s = 0;
   if (MODE != WAVE_IDENT && MODE != WAVE_ROWS) {
     tap = (int)fastdiv((unsigned)cur, g.div_ct);
-    ch = (cur - tap * ctiles) * 32;
+    ch = (cur - tap * (g.dw ? 1 : ctiles)) * 32;
     r = (int)fastdiv((unsigned)tap, g.div_kw);
     s = tap - r * g.KW;
   }
+  // depthwise form: K has one chunk per tap, the 32 input channels of this workgroup's own output channels
+  const int cp_k = g.dw ? 32 : g.Cp;       // channels of one tap in K
+  const int ch_first = g.dw ? oc0 : 0;     // first input channel this workgroup reads
 
   const int8_t* wa[TM];
 #pragma unroll
@@ -669,7 +672,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
           }
           need_tap = false;
         }
-        const int coff = live ? (ch >> 5) * 1024 : 0;
+        const int coff = live ? ((ch + ch_first) >> 5) * 1024 : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(tapptr[j] + (okv[j] ? coff : 0)));
@@ -678,7 +681,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
         ++cur;
         if (MODE != WAVE_ROWS) {
           ch += 32;
-          if (ch >= g.Cp) {
+          if (ch >= cp_k) {
             ch = 0;
             ++tap;
             if (++s == g.KW) { s = 0; ++r; }
@@ -931,6 +934,41 @@ int pad_channels(int c) {
 
 size_t packed_act_bytes(int64_t npix, int c) { return ((size_t)act_bytes(npix, pad_channels(c)) + 255) / 256 * 256; }
 
+// Depthwise filter int32 [C][1][KH][KW] as the MFMA operand of a convolution whose 32 output channels
+// of a tile read only their own 32 input channels: per tile, one 1 KiB chunk per tap holding the
+// 32x32 diagonal matrix diag(w[c][tap]) in fragment order (lane l: row l & 31, bytes (l >> 5)*16 .. +15
+// of K), then the zero chunks up to Kp/32 + 1.  One thread per dword of the destination.
+__global__ void __launch_bounds__(256) k_pack_depthwise_diag(const int32_t* __restrict__ w, uint32_t* __restrict__ wp,
+                                                             int64_t total, int c, int taps, int nch1) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int dword = (int)(i & 255);            // inside the KiB chunk
+    const int64_t chunk_lin = i >> 8;
+    const int chunk = (int)(chunk_lin % nch1);
+    const int tile = (int)(chunk_lin / nch1);
+    const int lane = dword >> 2, part = dword & 3;
+    const int row = lane & 31, k0 = (lane >> 5) * 16 + part * 4;   // this dword holds K columns k0 .. k0+3 of the row
+    uint32_t v = 0;
+    const int ch = tile * 32 + row;
+    if (chunk < taps && ch < c && row >= k0 && row < k0 + 4)
+      v = (uint32_t)(uint8_t)(int8_t)w[(int64_t)ch * taps + chunk] << (8 * (row - k0));
+    wp[i] = v;
+  }
+}
+
+size_t packed_depthwise_diag_bytes(int c, int kh, int kw) {
+  const int kp = (kh * kw * 32 + KSTEP - 1) / KSTEP * KSTEP;
+  const int tiles = (c + 127) / 128 * 4;
+  return (size_t)tiles * (kp / 32 + 1) * 1024 + 8192;
+}
+
+int pack_depthwise_diag(const int32_t* w, int8_t* wp, int c, int kh, int kw, hipStream_t s) {
+  const int kp = (kh * kw * 32 + KSTEP - 1) / KSTEP * KSTEP;
+  const int64_t total = (int64_t)packed_depthwise_diag_bytes(c, kh, kw) / 4;   // the slack behind the last tile is written as zeros too
+  k_pack_depthwise_diag<<<grid_for(total, 256), 256, 0, s>>>(w, reinterpret_cast<uint32_t*>(wp), total, c, kh * kw, kp / 32 + 1);
+  return check_launch("pack_depthwise_diag");
+}
+
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp) {
   const int cp = pad_channels(ic);
   *kp = (kh * kw * cp + KSTEP - 1) / KSTEP * KSTEP;
@@ -1117,8 +1155,10 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
     return arg_error("conv int8 output layout");
   if (((uintptr_t)out | (uintptr_t)ep0.residual) & 3) return arg_error("conv output alignment");
   if (ep0.out_mode == OUT_I8_ACT && ep0.out_cp >= 16 && ((uintptr_t)out & 15)) return arg_error("conv output alignment");
+  if (g.dw && ((g.Cp % 32) != 0 || g.row_bytes != 0 || g.OC > g.Cp || g.KH > 32 || g.KW > 32))
+    return arg_error("depthwise geometry (channels padded to 32, filter side at most 32)");
   g.taps = g.KH * g.KW;
-  g.K = g.row_bytes ? g.KH * g.row_bytes : g.taps * g.Cp;
+  g.K = g.row_bytes ? g.KH * g.row_bytes : g.dw ? g.taps * 32 : g.taps * g.Cp;
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
   if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
@@ -1147,7 +1187,7 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   }
   g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
   g.div_ow = make_fastdiv((uint32_t)g.OW);
-  g.div_ct = make_fastdiv((uint32_t)(g.Cp >= 32 ? g.Cp / 32 : 1));
+  g.div_ct = make_fastdiv((uint32_t)(g.dw ? 1 : g.Cp >= 32 ? g.Cp / 32 : 1));
   g.div_kw = make_fastdiv((uint32_t)g.KW);
   // kernel choice: the wavefront-private kernel when the layout allows it and its grid fits the chip,
   // else the LDS-tiled kernel.  Test and tuning hooks (read per call): CVM_HIP_CONV=lds|wave forces
@@ -1158,18 +1198,25 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   const bool rows = g.row_bytes != 0;
   const bool wave_ok = rows || ((g.Cp % 32) == 0 && (nopad || (g.KH <= 32 && g.KW <= 32)));
   int cfg = wave_ok ? choose_wave_cfg(g) : -1;
+  if (g.dw) {
+    // one 32-channel tile per workgroup (its K is its own channels): the 32-row configurations, unsplit
+    // unless the grid leaves most of the chip idle
+    if (!wave_ok) return arg_error("depthwise geometry");
+    cfg = wave_cfg_blocks(kWaveCfgs[6], g) >= 192 || g.taps < 8 ? 6 : 5;
+    if (wave_forced && wave_forced[0] >= '4' && wave_forced[0] <= '6') cfg = wave_forced[0] - '0';
+  } else
   if (conv_kind && conv_kind[0] == 'l' && !rows) cfg = -1;
   if (wave_ok && conv_kind && conv_kind[0] == 'w' && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
   if (cfg >= 0) {
     const int mode = rows ? WAVE_ROWS
-                          : (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                          : (!g.dw && g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
                                 ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
     g.octiles = (g.OC + 32 * kWaveCfgs[cfg].tm - 1) / (32 * kWaveCfgs[cfg].tm);
     g.div_octiles = make_fastdiv((uint32_t)g.octiles);
-    KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+    KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (g.dw ? 1.0 : (double)(g.C ? g.C : g.Cp)), s);
     launch_wave(cfg, mode, (unsigned)wnb, s, xp, wp, out, g, ep);
     return check_launch("conv_wave");
   }

@@ -338,6 +338,44 @@ int cvmhip_pack_depthwise_weights(const int32_t* w, void* wp, int c, int kh, int
   return check_launch("pack_depthwise");
 }
 
+// ---- depthwise convolution on the matrix cores: each tile of 32 output channels is a convolution over its own
+// 32 input channels with a diagonal filter matrix per tap
+int cvmhip_depthwise_mfma_eligible(int c, int kh, int kw) {
+  return c >= 1 && kh >= 1 && kw >= 1 && kh <= 32 && kw <= 32 && (pad_channels(c) % 32) == 0 ? 1 : 0;
+}
+
+size_t cvmhip_packed_depthwise_mfma_bytes(int c, int kh, int kw) {
+  if (!cvmhip_depthwise_mfma_eligible(c, kh, kw)) return 0;
+  return packed_depthwise_diag_bytes(c, kh, kw);
+}
+
+int cvmhip_pack_depthwise_weights_mfma(const int32_t* w, void* wp, int c, int kh, int kw, void* stream) {
+  if (!w || !wp || ((uintptr_t)wp & 15) || !cvmhip_depthwise_mfma_eligible(c, kh, kw)) return arg_error("pack_depthwise_weights_mfma");
+  return pack_depthwise_diag(w, reinterpret_cast<int8_t*>(wp), c, kh, kw, as_stream(stream));
+}
+
+int cvmhip_depthwise_conv2d_mfma_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                                    void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
+                                    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  if (!xp || !wp || !out) return arg_error("depthwise_conv2d_mfma_i8 null tensor");
+  if (n < 1 || h < 1 || wd < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1 ||
+      !cvmhip_depthwise_mfma_eligible(c, kh, kw) || h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("depthwise_conv2d_mfma_i8 attributes");
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(c); g.C = c;
+  g.OC = c;
+  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  g.dw = 1;
+  Epilogue ep = {};
+  ep.bias = bias;
+  if (!make_chain(chain, &ep.chain) || !make_chain(nullptr, &ep.chain2)) return arg_error("depthwise_conv2d_mfma_i8 chain");
+  ep.out_mode = out_is_i8 ? OUT_I8_ACT : OUT_I32_NCHW;
+  ep.out_cp = pad_channels(c);
+  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep, as_stream(stream));
+}
+
 int cvmhip_depthwise_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                                void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
                                int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {

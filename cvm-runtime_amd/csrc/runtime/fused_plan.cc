@@ -22,6 +22,7 @@
 // integer arithmetic as in node-by-node execution.
 #include <algorithm>
 #include <climits>
+#include <cstdlib>
 #include <map>
 
 #include "graph_runtime.h"
@@ -301,6 +302,9 @@ void HipGraphRuntime::BuildPlan() {
     return true;
   };
 
+  // test and tuning hook: CVM_HIP_DW=valu keeps depthwise layers on the vector kernel
+  const char* dw_env = std::getenv("CVM_HIP_DW");
+  const bool dw_on_mfma = !(dw_env && dw_env[0] == 'v');
   for (uint32_t nid = 0; nid < nodes_.size(); ++nid) {
     const Node& n = nodes_[nid];
     if (n.is_variable()) {
@@ -391,6 +395,11 @@ void HipGraphRuntime::BuildPlan() {
         if (st.kind == PlanStep::CONV) {
           Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_weight_bytes(st.oc, st.c, st.kh, st.kw)), "filter buffer");
           Check(cvmhip_pack_weights(entry_ptr_[we], buf->ptr, st.oc, st.c, st.kh, st.kw, stream_), "filter pack");
+        } else if (dw_on_mfma && cvmhip_depthwise_mfma_eligible(st.c, st.kh, st.kw)) {
+          // channels in whole tiles of 32: the depthwise layer runs on the matrix cores (diagonal filter blocks)
+          Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_depthwise_mfma_bytes(st.c, st.kh, st.kw)), "filter buffer");
+          Check(cvmhip_pack_depthwise_weights_mfma(entry_ptr_[we], buf->ptr, st.c, st.kh, st.kw, stream_), "filter pack");
+          st.dw_mfma = true;
         } else {
           Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_depthwise_bytes(st.c, st.kh, st.kw)), "filter buffer");
           Check(cvmhip_pack_depthwise_weights(entry_ptr_[we], buf->ptr, st.c, st.kh, st.kw, stream_), "filter pack");
@@ -614,6 +623,12 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
     }
     case PlanStep::DWCONV: {
       void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      if (st.dw_mfma) {
+        Check(cvmhip_depthwise_conv2d_mfma_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias,
+                                              &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.kh, st.kw,
+                                              st.sh, st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "depthwise_conv2d_mfma_i8");
+        break;
+      }
       Check(cvmhip_depthwise_conv2d_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias,
                                        &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.kh, st.kw, st.sh,
                                        st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "depthwise_conv2d_i8");

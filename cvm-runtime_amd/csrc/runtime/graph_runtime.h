@@ -100,6 +100,7 @@ struct PlanStep {
   std::shared_ptr<void> weights;  // packed filter (device)
   std::shared_ptr<void> aux;      // row-window copy of the input (device), see cvmhip_pack_stem_input
   bool stem = false;              // CONV through the row-window form
+  bool dw_mfma = false;           // DWCONV through the implicit-GEMM kernel (filter packed as diagonal blocks)
   bool nhwc = false;              // CONV writes int32 pixel-major rows into a slice of entry dst (a fused detection head)
   int64_t dst_off = 0, img_stride = 0;  // that slice: first element, and elements from one image to the next
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;

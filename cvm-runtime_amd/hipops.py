@@ -398,6 +398,34 @@ def pack_depthwise_weights(w):
     return wp
 
 
+def depthwise_mfma_eligible(c, kh, kw):
+    return bool(lib().cvmhip_depthwise_mfma_eligible(c, kh, kw))
+
+
+def pack_depthwise_weights_mfma(w):
+    c, one, kh, kw = w.shape
+    L = lib()
+    L.cvmhip_packed_depthwise_mfma_bytes.restype = ctypes.c_size_t
+    wp = _workspace(L.cvmhip_packed_depthwise_mfma_bytes(c, kh, kw), w.device)
+    check(L.cvmhip_pack_depthwise_weights_mfma(_ptr(w), _vp(wp), c, kh, kw, _stream()))
+    return wp
+
+
+def depthwise_conv2d_mfma_i8(xp, n, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_i8=True,
+                             strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """depthwise_conv2d_i8 through the implicit-GEMM kernel (diagonal filter blocks); wp from
+    pack_depthwise_weights_mfma."""
+    oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    if out_is_i8:
+        out = _act_buffer(n * oh * ow, c, xp.device)
+    else:
+        out = torch.empty((n, c, oh, ow), dtype=torch.int32, device=xp.device)
+    check(lib().cvmhip_depthwise_conv2d_mfma_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
+                                                _vp(out), int(out_is_i8), n, c, h, w, kh, kw, strides[0], strides[1],
+                                                padding[0], padding[1], dilation[0], dilation[1], _stream()))
+    return out
+
+
 def depthwise_conv2d_i8(xp, n, c, h, w, wp, kh, kw, bias=None, chain1=None, out_is_i8=True,
                         strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
     oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])

@@ -274,6 +274,18 @@ int cvmhip_pack_depthwise_weights(const int32_t* w, void* wp, int c, int kh, int
 int cvmhip_depthwise_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                                void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
                                int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* The same depthwise convolution on the matrix cores, for channel counts padded to a multiple of 32 and
+ * filter sides up to 32: a tile of 32 output channels is a convolution over its own 32 input channels
+ * whose filter matrix is diagonal for every tap (groupwise_conv2d with groups == channels:
+ * ops.cc:333-366), so it runs in the implicit-GEMM kernel of cvmhip_conv2d_i8 with K = taps * 32.  The
+ * filter is packed by cvmhip_pack_depthwise_weights_mfma into cvmhip_packed_depthwise_mfma_bytes bytes.
+ * Operands must be known to fit int8 (this path, like cvmhip_depthwise_conv2d_i8, does not narrow). */
+int cvmhip_depthwise_mfma_eligible(int c, int kh, int kw);
+size_t cvmhip_packed_depthwise_mfma_bytes(int c, int kh, int kw);
+int cvmhip_pack_depthwise_weights_mfma(const int32_t* w, void* wp, int c, int kh, int kw, void* stream);
+int cvmhip_depthwise_conv2d_mfma_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                                    void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
+                                    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
 /* out = chain(a + b) on int8 act tensors of identical geometry */
 int cvmhip_add_i8(const void* a, const void* b, const cvmhip_chain* chain, void* out, int out_is_i8,
                   int n, int c, int hw, void* stream);

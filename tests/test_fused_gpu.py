@@ -276,6 +276,53 @@ def test_conv_wave_kernel_every_configuration(case, cfg, dev):
     eq(out32.cpu().numpy(), conv, "wave cfg %d int32" % cfg)
 
 
+DW_MFMA_CASES = [
+    # n, c, h, w, k, stride, pad, dilation
+    (2, 32, 19, 17, 3, 1, 1, 1),
+    (1, 96, 16, 16, 3, 2, 1, 1),       # three channel tiles, stride 2
+    (1, 256, 8, 8, 5, 1, 2, 1),        # 25 taps
+    (1, 40, 9, 9, 3, 1, 0, 1),         # channels padded 40 -> 64, no padding
+    (3, 64, 7, 7, 3, 1, 2, 2),         # dilated
+    (1, 128, 33, 31, 3, 2, 1, 1),      # ragged pixel count
+    (1, 32, 6, 6, 1, 1, 0, 1),         # a single tap
+    (16, 1024, 4, 4, 3, 1, 1, 1),      # many tiles, few pixels
+]
+
+
+@pytest.mark.parametrize("cfg", [None, "4", "5", "6"])
+@pytest.mark.parametrize("case", DW_MFMA_CASES, ids=lambda c: "n%dc%dh%dw%dk%ds%dp%dd%d" % c)
+def test_depthwise_conv2d_mfma_i8(case, cfg, dev):
+    """Depthwise convolution as diagonal 32x32 filter blocks on the matrix cores, against the oracle's
+    groups == channels convolution, for every configuration of the kernel."""
+    n, c, h, w, k, st, pd, dl = case
+    assert hipops.depthwise_mfma_eligible(c, k, k)
+    cid = "fdwm-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (c, 1, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (c,), -3000, 3000)
+    stages = [("relu",), ("cvm_right_shift", 8, 10)]
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (dl, dl), c)
+    ref = run_chain(conv, stages)
+    xp = hipops.pack_act_i8(T(x, dev))
+    wp = hipops.pack_depthwise_weights_mfma(T(wt, dev))
+    if cfg is not None:
+        os.environ["CVM_HIP_WAVECFG"] = cfg
+    try:
+        out = hipops.depthwise_conv2d_mfma_i8(xp, n, c, h, w, wp, k, k, T(b, dev), hipops.chain(*stages), True, (st, st),
+                                              (pd, pd), (dl, dl))
+        out32 = hipops.depthwise_conv2d_mfma_i8(xp, n, c, h, w, wp, k, k, T(b, dev), None, False, (st, st), (pd, pd), (dl, dl))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+    eq(act_to_nchw(out, n, c, ref.shape[2], ref.shape[3]), ref, "depthwise (matrix cores) int8")
+    eq(out32.cpu().numpy(), conv, "depthwise (matrix cores) int32")
+
+
+def test_depthwise_mfma_rejects_unpadded_channels(dev):
+    assert not hipops.depthwise_mfma_eligible(5, 3, 3)     # padded to 8, not to a multiple of 32
+    assert not hipops.depthwise_mfma_eligible(32, 33, 3)   # filter side beyond the 32-bit tap masks
+
+
 @pytest.mark.parametrize("case", [(2, 32, 19, 17, 3, 1, 1), (1, 96, 16, 16, 3, 2, 1), (1, 5, 9, 9, 3, 1, 0), (1, 256, 8, 8, 5, 1, 2)],
                          ids=lambda c: "n%dc%dh%dw%dk%ds%dp%d" % c)
 def test_depthwise_conv2d_i8(case, dev):

@@ -2,6 +2,8 @@
 CVMAPIInference, include/cvm_c_api.h) against the CPU oracle executing the same
 graph node by node -- the method of the reference's tests/test_model.cc:94-235,
 with the oracle in place of the absent /data fixtures.  Bit-exact."""
+import os
+
 import numpy as np
 import pytest
 
@@ -120,6 +122,21 @@ def test_config5_ssd_mobilenet_detector(neg_ids, dev):
     _check(out, tsize, ref)
     kept = (ref[0][0, :, 0] >= 0).sum()
     assert 0 < kept <= 400
+
+
+def test_depthwise_layers_on_the_vector_kernel_give_the_same_detections(dev):
+    """The planner's two depthwise forms (matrix cores by default, vector kernel behind CVM_HIP_DW=valu)
+    must both reproduce the oracle on a detector whose backbone is depthwise-separable."""
+    g, heads = graphgen.ssd_mobilenet(size=128, alpha=0.5, config_id="cfg5-dw-forms", neg_ids=True)
+    os.environ["CVM_HIP_DW"] = "valu"
+    try:
+        out, tsize, ref = _run_both(g, heads, "cfg5-dw-forms")
+    finally:
+        os.environ.pop("CVM_HIP_DW", None)
+    _check(out, tsize, ref)
+    out2, tsize2, ref2 = _run_both(g, heads, "cfg5-dw-forms")
+    _check(out2, tsize2, ref2)
+    assert out == out2
 
 
 def test_argmax_and_detection_postprocess(dev):
