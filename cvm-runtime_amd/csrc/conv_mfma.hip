@@ -1084,6 +1084,7 @@ static const WaveCfg kWaveCfgs[] = {
     // tile rows x cols of 32, K split, wavefronts, resident workgroups per CU (registers and LDS)
     {2, 2, 8, 8, 1}, {2, 2, 4, 4, 2}, {2, 2, 2, 4, 2}, {2, 2, 1, 4, 2},
     {1, 2, 8, 8, 2}, {1, 2, 4, 4, 2}, {1, 2, 1, 4, 2},
+    {2, 4, 1, 4, 2},
 };
 constexpr int kNumWaveCfgs = sizeof(kWaveCfgs) / sizeof(kWaveCfgs[0]);
 
@@ -1119,12 +1120,18 @@ static int choose_wave_cfg(const ConvGeom& g) {
   // the 64-channel tile leaves SIMDs without a wavefront, so halve the tile instead
   if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < 128) return 4;
   const int first = g.OC > 32 ? 0 : 4;
-  const int last = g.OC > 32 ? 4 : kNumWaveCfgs;
+  const int last = g.OC > 32 ? 4 : 7;   // 64-channel tiles: 0..3 (and 7, see below); 32-channel tiles: 4..6
   for (int i = first; i < last; ++i) {
     const WaveCfg& c = kWaveCfgs[i];
     if (c.ksplit > 1 && nlive < 2 * c.ksplit) continue;
     const int64_t capacity = 256 * (int64_t)c.blocks_per_cu;
-    if (c.ksplit == 1 || wave_cfg_blocks(c, g) <= capacity) return i;
+    if (c.ksplit == 1 || wave_cfg_blocks(c, g) <= capacity) {
+      // Unsplit with a grid of many rounds and a long K loop (the large layers of a VGG): the K loop is bound by
+      // operand delivery, and a 64 x 128 wavefront tile takes 0.75 KiB per MFMA instead of 1 KiB (measured
+      // 1.0 -> 1.2-1.3 POP/s on 28x28x512 and 56x56x256 layers with 3x3 filters).
+      if (c.ksplit == 1 && g.OC > 32 && g.K >= 512 && wave_cfg_blocks(kWaveCfgs[7], g) >= 192) return 7;
+      return i;
+    }
   }
   return last - 1;
 }
@@ -1138,7 +1145,8 @@ static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const i
     case 3: launch_wave_cfg<2, 2, 1, 4, 2, 2>(mode, grid, s, xp, wp, out, g, ep); break;
     case 4: launch_wave_cfg<1, 2, 8, 8, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
     case 5: launch_wave_cfg<1, 2, 4, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
-    default: launch_wave_cfg<1, 2, 1, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    case 6: launch_wave_cfg<1, 2, 1, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    default: launch_wave_cfg<2, 4, 1, 4, 1, 2>(mode, grid, s, xp, wp, out, g, ep); break;
   }
 }
 

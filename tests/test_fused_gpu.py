@@ -245,7 +245,7 @@ def test_conv2d_stem_i8(case, dev):
     eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), run_chain(conv, stages), "stem int8")
 
 
-@pytest.mark.parametrize("cfg", range(7))
+@pytest.mark.parametrize("cfg", range(8))
 @pytest.mark.parametrize("case", [(3, 96, 11, 13, 100, 3, 1, 1, True), (2, 256, 9, 9, 72, 1, 2, 0, False),
                                   (1, 64, 8, 8, 40, 3, 2, 1, True)],
                          ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%d" % c[:8])
