@@ -139,6 +139,81 @@ def test_depthwise_layers_on_the_vector_kernel_give_the_same_detections(dev):
     assert out == out2
 
 
+def _random_graph(seed):
+    """A seeded random network from the building blocks the planner fuses: requantised convolutions
+    (1x1 / 3x3, strided, depthwise), residual adds, pooling, channel concatenation, and one of three
+    tails (global sum -> dense, flatten -> dense, detection heads).  Every tensor kept for reuse is 8-bit."""
+    rng = np.random.RandomState(seed)
+    g = graphgen.GraphBuilder("rand-%d" % seed)
+    n = int(rng.choice([1, 2, 3]))
+    c = int(rng.choice([3, 8, 16, 32]))
+    hw = int(rng.choice([9, 12, 16]))
+    x = g.var("data", (n, c, hw, hw), 8)
+    pool = [x]
+    for _ in range(int(rng.randint(5, 11))):
+        cur = pool[-1]
+        _, cc, h, w = g.shape(cur)
+        kind = rng.choice(["conv", "conv", "conv", "dw", "add", "pool", "concat"])
+        if kind == "conv":
+            k = int(rng.choice([1, 3]))
+            st = int(rng.choice([1, 1, 2])) if h >= 4 else 1
+            oc = int(rng.choice([16, 32, 48, 64, 96]))
+            pool.append(g.conv_relu_q(cur, oc, k, st, k // 2, relu=bool(rng.randint(2))))
+        elif kind == "dw" and cc >= 8:
+            st = int(rng.choice([1, 2])) if h >= 4 else 1
+            pool.append(g.conv_relu_q(cur, cc, 3, st, 1, groups=cc))
+        elif kind == "add":
+            same = [t for t in pool[:-1] if g.shape(t) == g.shape(cur) and t is not x]
+            if same:
+                y = g.add(cur, same[int(rng.randint(len(same)))])
+                if rng.randint(2):
+                    y = g.relu(y)
+                pool.append(g.rshift(y, 1))
+        elif kind == "pool" and h >= 4:
+            pool.append(g.max_pool(cur, 3, 2, 1) if rng.randint(2) else g.max_pool(cur, 2, 2))
+        elif kind == "concat":
+            same = [t for t in pool[:-1] if g.shape(t)[2:] == g.shape(cur)[2:] and g.shape(t)[0] == n and t is not x]
+            if same:
+                pool.append(g.concat([cur, same[int(rng.randint(len(same)))]], 1))
+    cur = pool[-1]
+    _, cc, h, w = g.shape(cur)
+    tail = rng.choice(["sum", "flatten", "heads"])
+    if tail == "sum":
+        s_, cnt = g.global_sum(cur)
+        s_ = g.rshift(s_, max(1, int(np.ceil(np.log2(cnt)))))
+        y, _ = g.dense(g.flatten(s_), int(rng.choice([10, 33])))
+        return g, [y]
+    if tail == "flatten":
+        y, _ = g.dense(g.flatten(cur), int(rng.choice([10, 33])))
+        return g, [y]
+    outs = []
+    for src in (cur, pool[-2] if len(pool) > 2 and pool[-2] is not x else cur):
+        oc = int(rng.choice([12, 24, 84]))
+        y = g.conv_relu_q(src, oc, 3, 1, 1, relu=False)
+        y = g.transpose(y, (0, 2, 3, 1))
+        outs.append(g.reshape(y, (n, int(np.prod(g.shape(y)[1:])))))
+    return g, [g.concat(outs, 1)]
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_graphs_match_the_oracle(seed, dev):
+    g, heads = _random_graph(seed)
+    out, tsize, ref = _run_both(g, heads, "rand-%d" % seed)
+    _check(out, tsize, ref)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_graphs_node_by_node(seed, dev):
+    """The same networks with the load-time fusion switched off: one registry kernel per node."""
+    g, heads = _random_graph(seed)
+    os.environ["CVM_HIP_FUSE"] = "0"
+    try:
+        out, tsize, ref = _run_both(g, heads, "rand-%d" % seed)
+    finally:
+        os.environ.pop("CVM_HIP_FUSE", None)
+    _check(out, tsize, ref)
+
+
 def test_argmax_and_detection_postprocess(dev):
     g, heads = graphgen.resnet20_cifar(1)
     js, pb = g.build(heads, postprocess="argmax")
