@@ -139,15 +139,16 @@ def test_depthwise_layers_on_the_vector_kernel_give_the_same_detections(dev):
     assert out == out2
 
 
-def _random_graph(seed):
+def _random_graph(seed, big=False):
     """A seeded random network from the building blocks the planner fuses: requantised convolutions
     (1x1 / 3x3, strided, depthwise), residual adds, pooling, channel concatenation, and one of three
     tails (global sum -> dense, flatten -> dense, detection heads).  Every tensor kept for reuse is 8-bit."""
-    rng = np.random.RandomState(seed)
-    g = graphgen.GraphBuilder("rand-%d" % seed)
-    n = int(rng.choice([1, 2, 3]))
-    c = int(rng.choice([3, 8, 16, 32]))
-    hw = int(rng.choice([9, 12, 16]))
+    rng = np.random.RandomState(seed + (1000 if big else 0))
+    g = graphgen.GraphBuilder("rand-%d-%d" % (seed, big))
+    n = int(rng.choice([4, 16] if big else [1, 2, 3]))
+    c = int(rng.choice([32, 64] if big else [3, 8, 16, 32]))
+    hw = int(rng.choice([14, 28] if big else [9, 12, 16]))
+    widths = [64, 128, 256, 512] if big else [16, 32, 48, 64, 96]
     x = g.var("data", (n, c, hw, hw), 8)
     pool = [x]
     for _ in range(int(rng.randint(5, 11))):
@@ -157,7 +158,7 @@ def _random_graph(seed):
         if kind == "conv":
             k = int(rng.choice([1, 3]))
             st = int(rng.choice([1, 1, 2])) if h >= 4 else 1
-            oc = int(rng.choice([16, 32, 48, 64, 96]))
+            oc = int(rng.choice(widths))
             pool.append(g.conv_relu_q(cur, oc, k, st, k // 2, relu=bool(rng.randint(2))))
         elif kind == "dw" and cc >= 8:
             st = int(rng.choice([1, 2])) if h >= 4 else 1
@@ -178,6 +179,8 @@ def _random_graph(seed):
     cur = pool[-1]
     _, cc, h, w = g.shape(cur)
     tail = rng.choice(["sum", "flatten", "heads"])
+    if tail == "flatten" and cc * h * w > 32767:   # dense precision 8 + 8 + bitlen(K) + 1 must stay within 32 bits
+        tail = "sum"
     if tail == "sum":
         s_, cnt = g.global_sum(cur)
         s_ = g.rshift(s_, max(1, int(np.ceil(np.log2(cnt)))))
@@ -199,6 +202,15 @@ def _random_graph(seed):
 def test_random_graphs_match_the_oracle(seed, dev):
     g, heads = _random_graph(seed)
     out, tsize, ref = _run_both(g, heads, "rand-%d" % seed)
+    _check(out, tsize, ref)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_wide_graphs_match_the_oracle(seed, dev):
+    """Batches of 4 and 16, up to 512 channels, 14x14 and 28x28 maps: the K-split, unsplit and large-tile
+    configurations of the convolution kernel inside whole networks."""
+    g, heads = _random_graph(seed, big=True)
+    out, tsize, ref = _run_both(g, heads, "rand-%d-1" % seed)
     _check(out, tsize, ref)
 
 
