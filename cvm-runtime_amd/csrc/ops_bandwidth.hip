@@ -186,6 +186,43 @@ __global__ void __launch_bounds__(256) k_max_pool(const int32_t* __restrict__ x,
   }
 }
 
+// 3x3 windows with stride 2 (the pooling layer behind a network's input convolution) on rows whose
+// length is a multiple of 4: one thread per pair of adjacent outputs.  The two windows span five input
+// columns, four of which are one aligned 16-byte load per row, so a pair costs six loads instead of
+// eighteen and a wavefront reads whole contiguous KiBs.  pad_w is 0 or 1.
+__global__ void __launch_bounds__(256) k_max_pool_3x3s2(const int32_t* __restrict__ x, int32_t* __restrict__ y,
+                                                        uint32_t total_pairs, int h, int w, int oh, int ow, int ph, int pw) {
+  const uint32_t pairs = (uint32_t)(ow + 1) >> 1;
+  const uint32_t stride = gridDim.x * blockDim.x;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total_pairs; i += stride) {
+    const uint32_t row = i / pairs;
+    const int j = (int)(i - row * pairs);
+    const uint32_t nc = row / (uint32_t)oh;
+    const int p = (int)(row - nc * (uint32_t)oh);
+    const int32_t* xp = x + (int64_t)nc * h * w + 4 * j;
+    int32_t m0 = INT32_MIN, m1 = INT32_MIN;
+    const int extra = pw ? -1 : 4;                 // the fifth column, relative to 4j
+    const bool extra_ok = pw ? j > 0 : 4 * j + 4 < w;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int ih = 2 * p + r - ph;
+      if (ih < 0 || ih >= h) continue;
+      const int4 v = *reinterpret_cast<const int4*>(xp + (int64_t)ih * w);
+      const int32_t e = extra_ok ? xp[(int64_t)ih * w + extra] : INT32_MIN;
+      if (pw) {   // windows 4j-1..4j+1 and 4j+1..4j+3
+        m0 = max(m0, max(e, max(v.x, v.y)));
+        m1 = max(m1, max(v.y, max(v.z, v.w)));
+      } else {    // windows 4j..4j+2 and 4j+2..4j+4
+        m0 = max(m0, max(v.x, max(v.y, v.z)));
+        m1 = max(m1, max(v.z, max(v.w, e)));
+      }
+    }
+    int32_t* yp = y + (int64_t)row * ow + 2 * j;
+    yp[0] = m0;
+    if (2 * j + 1 < ow) yp[1] = m1;
+  }
+}
+
 // ---------------------------------------------------------------- reductions
 struct RShape {
   int nk, nr;
@@ -479,6 +516,13 @@ int cvmhip_max_pool2d(const int32_t* x, int32_t* y, int n, int c, int h, int w,
       pad_h < 0 || pad_w < 0)
     return arg_error("max_pool2d");
   const int64_t total = (int64_t)n * c * oh * ow;
+  // (the output extent is the caller's: with ceil_mode a last window may start past the row, which only the general kernel handles)
+  if (kh == 3 && kw == 3 && stride_h == 2 && stride_w == 2 && pad_w <= 1 && (w & 3) == 0 && w >= 4 && ((ow + 1) / 2) * 4 <= w &&
+      (((uintptr_t)x) & 15) == 0 && total < INT32_MAX && (int64_t)n * c * h * w < ((int64_t)1 << 40)) {
+    const int64_t pairs = (int64_t)n * c * oh * ((ow + 1) / 2);
+    k_max_pool_3x3s2<<<grid_for(pairs, 256, 256 * 64), 256, 0, as_stream(stream)>>>(x, y, (uint32_t)pairs, h, w, oh, ow, pad_h, pad_w);
+    return check_launch("max_pool2d");
+  }
   const unsigned grid = grid_for(total, 256, 256 * 64);
   if (total + (int64_t)grid * 256 < INT32_MAX && (int64_t)h * w < INT32_MAX)
     k_max_pool<uint32_t><<<grid, 256, 0, as_stream(stream)>>>(x, y, total, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);

@@ -180,7 +180,16 @@ def test_broadcast(op, dev):
 @pytest.mark.parametrize("case", [((16, 64, 112, 112), (3, 3), (2, 2), (1, 1), False),
                                   ((2, 8, 14, 14), (2, 2), (2, 2), (0, 0), False),
                                   ((1, 3, 9, 11), (2, 2), (2, 2), (0, 0), True),
-                                  ((1, 2, 7, 7), (3, 2), (1, 2), (1,), False)])
+                                  ((1, 2, 7, 7), (3, 2), (1, 2), (1,), False),
+                                  # 3x3 stride 2 on rows of a multiple of 4 (the paired kernel): both paddings,
+                                  # odd output widths, one-pair rows, ceil_mode (falls back to the general kernel)
+                                  ((2, 5, 12, 12), (3, 3), (2, 2), (0, 0), False),
+                                  ((3, 4, 9, 8), (3, 3), (2, 2), (1, 1), False),
+                                  ((1, 7, 5, 4), (3, 3), (2, 2), (1, 1), False),
+                                  ((1, 3, 16, 20), (3, 3), (2, 2), (0, 1), False),
+                                  ((1, 3, 16, 20), (3, 3), (2, 2), (1, 0), False),
+                                  ((2, 3, 12, 12), (3, 3), (2, 2), (1, 1), True),
+                                  ((1, 2, 11, 16), (3, 3), (2, 2), (0, 0), True)])
 def test_max_pool2d(case, dev):
     shape, k, s, p, ceil = case
     x = synth.tensor("pool", str(case), shape, -2 ** 31, 2 ** 31 - 1)
