@@ -113,6 +113,20 @@ __global__ void __launch_bounds__(256) k_binary_vec(const int4* a, const int4* b
   }
 }
 
+// one operand is a single element (the reference's fast paths, broadcast.cc:33-36): SCALAR_A selects which
+template <int OP, bool SCALAR_A>
+__global__ void __launch_bounds__(256) k_binary_scalar_vec(const int4* v, const int32_t* scalar, int4* c, int64_t nvec) {
+  const int32_t k = scalar[0];
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    const int4 u = v[i];
+    int4 r;
+    if (SCALAR_A) { r.x = bfun<OP>(k, u.x); r.y = bfun<OP>(k, u.y); r.z = bfun<OP>(k, u.z); r.w = bfun<OP>(k, u.w); }
+    else { r.x = bfun<OP>(u.x, k); r.y = bfun<OP>(u.y, k); r.z = bfun<OP>(u.z, k); r.w = bfun<OP>(u.w, k); }
+    c[i] = r;
+  }
+}
+
 struct BShape {
   int ndim;
   int64_t cdim[CVM_MAXD];     // output extents
@@ -151,6 +165,10 @@ static int launch_broadcast(const int32_t* a, const int32_t* b, int32_t* c, int6
       k_binary_vec<OP><<<grid_for(n / 4, 256), 256, 0, s>>>((const int4*)a, (const int4*)b, (int4*)c, n / 4);
     else
       k_binary<OP><<<grid_for(n, 256), 256, 0, s>>>(a, b, c, n);
+  } else if (amode == 2 && bmode == 1 && (((uintptr_t)a | (uintptr_t)c) & 15) == 0 && (n % 4) == 0) {
+    k_binary_scalar_vec<OP, false><<<grid_for(n / 4, 256), 256, 0, s>>>((const int4*)a, b, (int4*)c, n / 4);
+  } else if (amode == 1 && bmode == 2 && (((uintptr_t)b | (uintptr_t)c) & 15) == 0 && (n % 4) == 0) {
+    k_binary_scalar_vec<OP, true><<<grid_for(n / 4, 256), 256, 0, s>>>((const int4*)b, a, (int4*)c, n / 4);
   } else {
     k_broadcast<OP><<<grid_for(n, 256), 256, 0, s>>>(a, b, c, n, sh, amode, bmode);
   }
