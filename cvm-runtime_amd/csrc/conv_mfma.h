@@ -40,7 +40,13 @@ struct ConvGeom {
   int KH, KW, SH, SW, PH, PW, DH, DW;
   int taps, K, Kp;         // filled by conv_igemm: KH*KW, taps*Cp, K rounded up to 64
   int64_t P;               // filled by conv_igemm: N*OH*OW
-  int adv_c, adv_tap, adv_r, adv_s;  // filled by conv_igemm: cursor advance of one K step (channel, tap, filter row/column)
+  union {   // the two kernels need different extras; sharing the space keeps the kernel argument block at its size
+    struct { int adv_c, adv_tap, adv_r, adv_s; };   // tiled kernel: cursor advance of one K step (channel, tap, filter row/column)
+    struct {                                         // wavefront kernel, filled by conv_igemm_ws: K cut into kslices ranges over
+      int kslices, slice_shift, slice_stride, slice_chunks;   // the grid (0 or 1 = no; else 2 or 4 = 1 << slice_shift, the slice is
+    };                                               // the low bits of the block index), int32 elements from one slice's plane of
+                                                     // partial sums to the next, 32-byte chunks of K per slice
+  };
   FastDiv div_ohw, div_ow, div_ct, div_kw;  // filled by conv_igemm: division by OH*OW, OW, Cp/32 and KW
   int row_bytes;           // > 0: row-window input (see stem_* below): bytes of K per filter row, 16 or 32
   int dw;                  // 1: depthwise convolution through MFMA -- output channel tile t reads input channels 32t .. 32t+31 only,
@@ -128,6 +134,12 @@ int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStre
 int unpack_activations(const int8_t* xp, int32_t* x, int n, int c, int hw, hipStream_t s);
 int pack_weights(const int32_t* w, int8_t* wp, int oc, int ic, int kh, int kw, hipStream_t s);
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, hipStream_t s);
+// The same with a workspace: a layer with at most 64 output pixels and K >= 8192 is then computed in K slices by
+// several workgroups per tile (partial sums in the workspace, a second kernel finishes).  Without a workspace, or for
+// any other layer, identical to conv_igemm.  conv_slices_workspace_bytes() gives the size (0 = not applicable).
+size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep);
+int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, void* ws, size_t ws_bytes,
+                  hipStream_t s);
 
 }  // namespace cvmhip
 #endif

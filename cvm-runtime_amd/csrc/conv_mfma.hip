@@ -496,7 +496,7 @@ __device__ __forceinline__ unsigned tap_mask_dilated(int x0, int extent, int k, 
 //                    out-of-image granules are read from a zero granule
 enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 
-template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE>
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
 __global__ void __launch_bounds__(NW * 64, MINW)
 k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
             const ConvGeom g, const Epilogue ep) {
@@ -528,6 +528,15 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   int pid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
+  // K sliced over the grid (g.kslices > 1: a layer with very few tiles and a very long K, whose filter stream
+  // needs more workgroups than it has tiles): slice index = low bits of the block index (the slices of a tile then share its activation operand in one L2); a slice writes
+  // raw int32 partial sums to its own plane of the workspace and a second kernel adds the planes up.
+  // (SLICES: only the instantiation the host launches for such layers carries the code)
+  int kslice = 0;
+  if (SLICES && g.kslices > 1) {
+    kslice = pid & (g.kslices - 1);
+    pid >>= g.slice_shift;
+  }
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);   // g.octiles = ceil(OC / BM), set by the host for this tile
   const int oc0 = (pid - ptile * g.octiles) * BM;
   const int px0 = ptile * BN;              // P < 2^31 is checked on the host
@@ -577,11 +586,15 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 
   // K range of this wavefront, in chunks of 32 bytes; chunks past the true K are never visited
   const int nch = g.Kp >> 5;
-  const int nlive = (g.K + 31) >> 5;
-  const int per = (nlive + KSPLIT - 1) / KSPLIT;
-  const int c_begin = kw_ * per;
+  int s_begin = 0, nlive = (g.K + 31) >> 5;   // this workgroup's chunks: [s_begin, nlive)
+  if (SLICES && g.kslices > 1) {
+    s_begin = kslice * g.slice_chunks < nlive ? kslice * g.slice_chunks : nlive;
+    nlive = s_begin + g.slice_chunks < nlive ? s_begin + g.slice_chunks : nlive;
+  }
+  const int per = (nlive - s_begin + KSPLIT - 1) / KSPLIT;
+  const int c_begin = s_begin + kw_ * per;
   const int c_end = c_begin + per < nlive ? c_begin + per : nlive;
-  const int niter = (per + D - 1) / D;
+  const int niter = SLICES ? (per > 0 ? (per + D - 1) / D : 1) : (per + D - 1) / D;
   int cur = c_begin;
   int tap = 0, ch = 0, r = 0, s = 0;
   if (MODE != WAVE_IDENT && MODE != WAVE_ROWS) {
@@ -772,7 +785,45 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
         for (int e = 0; e < 16; ++e) val[((i * TN + j) * 16 + e) % (NU * 4)] = acc[i][j][e];
   }
-  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, out, g, ep, rp);
+  void* dst = out;
+  if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
+  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp);
+}
+
+// Second step of a K-sliced convolution: out = chain(sum over slices + bias), stored like the epilogue would
+// (int8 activations or int32 NCHW).  One thread per 4 consecutive channels of a pixel.
+template <int OUT>
+__global__ void __launch_bounds__(256) k_slices_finish(const int32_t* __restrict__ part, void* __restrict__ out, int kslices,
+                                                       int slice_stride, const ConvGeom g, const Epilogue ep) {
+  const int OHW = g.OH * g.OW;
+  const int oc4 = OUT == OUT_I8_ACT ? ep.out_cp >> 2 : (g.OC + 3) >> 2;   // int8: padding channels are written too (as zeros)
+  const int64_t total = g.P * oc4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t p = i / oc4;
+    const int oc = (int)(i - p * oc4) * 4;
+    const int64_t n = p / OHW;
+    const int rem = (int)(p - n * OHW);
+    int32_t v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      int32_t acc = (ep.bias && oc + e < g.OC) ? ep.bias[oc + e] : 0;
+      if (oc + e < g.OC)
+        for (int k = 0; k < kslices; ++k) acc = wadd(acc, part[(int64_t)k * slice_stride + (n * g.OC + oc + e) * OHW + rem]);
+      v[e] = acc;
+    }
+    run_chain(ep.chain, v);
+    if (OUT == OUT_I32_NCHW) {
+      int32_t* y32 = reinterpret_cast<int32_t*>(out) + n * ep.o32_img + (int64_t)oc * ep.o32_ch + (int64_t)rem * ep.o32_px;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (oc + e < g.OC) y32[(int64_t)e * ep.o32_ch] = v[e];
+    } else {
+      uint32_t w[1] = {pack_bytes(v[0], v[1], v[2], v[3])};
+      mask_channels(w, oc, g.OC);
+      if (oc < ep.out_cp) *reinterpret_cast<uint32_t*>(reinterpret_cast<int8_t*>(out) + act_offset(p, oc, ep.out_cp)) = w[0];
+    }
+  }
 }
 
 constexpr int KSTEP = 64;  // granularity K is padded to
@@ -1097,6 +1148,14 @@ static void launch_wave_mode(int mode, unsigned grid, hipStream_t s, const int8_
   else k_conv_wave<TM, TN, KSPLIT, NW, D, MINW, OUT, WAVE_PAD><<<grid, NW * 64, 0, s>>>(xp, wp, out, g, ep);
 }
 
+// K-sliced launch: 32-channel tiles, 8-way K split inside the workgroup, raw int32 partial sums (no row-window mode)
+static void launch_wave_sliced(int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
+                               const ConvGeom& g, const Epilogue& ep) {
+  if (mode == WAVE_IDENT) k_conv_wave<1, 2, 8, 8, 4, 2, OUT_I32_NCHW, WAVE_IDENT, true><<<grid, 512, 0, s>>>(xp, wp, out, g, ep);
+  else if (mode == WAVE_NOPAD) k_conv_wave<1, 2, 8, 8, 4, 2, OUT_I32_NCHW, WAVE_NOPAD, true><<<grid, 512, 0, s>>>(xp, wp, out, g, ep);
+  else k_conv_wave<1, 2, 8, 8, 4, 2, OUT_I32_NCHW, WAVE_PAD, true><<<grid, 512, 0, s>>>(xp, wp, out, g, ep);
+}
+
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW>
 static void launch_wave_cfg(int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                             const ConvGeom& g, const Epilogue& ep) {
@@ -1150,7 +1209,30 @@ static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const i
   }
 }
 
+// K slices over the grid: for a layer with at most 64 output pixels and K >= 8192 (a fully connected layer at a
+// small batch) the filter stream is the whole cost, and one workgroup per 32 output channels is too few
+// workgroups to keep it flowing.  Returns the number of slices (1 = not applicable).
+static int conv_slices(const ConvGeom& g, const Epilogue& ep) {
+  const int64_t p = (int64_t)g.N * g.OH * g.OW;
+  const int64_t k = (int64_t)g.KH * g.KW * g.Cp;
+  if (g.dw || g.row_bytes || (g.Cp % 32) != 0 || p > 64 || k < 8192 || g.OC < 32 || ep.residual) return 1;
+  if (!(g.PH == 0 && g.PW == 0) && (g.KH > 32 || g.KW > 32)) return 1;
+  const int tiles = (g.OC + 31) / 32;
+  if (tiles > 256) return 1;
+  return tiles <= 128 ? 4 : 2;   // a power of two: the slice is the low bits of the block index
+}
+
+size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep) {
+  const int ks = conv_slices(g, ep);
+  return ks > 1 ? (size_t)ks * g.N * g.OC * g.OH * g.OW * 4 : 0;
+}
+
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
+  return conv_igemm_ws(xp, wp, out, g, ep_in, nullptr, 0, s);
+}
+
+int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, void* ws, size_t ws_bytes,
+                  hipStream_t s) {
   const Epilogue& ep0 = ep_in;
   if (g.N < 1 || g.H < 1 || g.W < 1 || g.OC < 1 || g.OH < 1 || g.OW < 1 || g.KH < 1 || g.KW < 1 || g.SH < 1 ||
       g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
@@ -1216,6 +1298,39 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   if (conv_kind && conv_kind[0] == 'l' && !rows) cfg = -1;
   if (wave_ok && conv_kind && conv_kind[0] == 'w' && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
+  const int kslices = ws ? conv_slices(g, ep) : 1;
+  if (kslices > 1 && wave_ok) {
+    const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
+    if (ws_bytes < need || ((uintptr_t)ws & 15)) return arg_error("conv K-slice workspace");
+    cfg = 4;
+    const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                         ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
+    const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
+    g.octiles = (g.OC + 31) / 32;
+    g.div_octiles = make_fastdiv((uint32_t)g.octiles);
+    g.kslices = kslices;
+    g.slice_shift = kslices == 4 ? 2 : 1;
+    g.slice_chunks = ((g.K + 31) / 32 + kslices - 1) / kslices;
+    g.slice_stride = (int)((int64_t)g.N * g.OC * g.OH * g.OW);   // at most 64 pixels x OC
+    Epilogue raw = {};                 // slices store raw int32 sums, NCHW, into their plane of the workspace
+    raw.out_mode = OUT_I32_NCHW;
+    raw.out_cp = ep.out_cp;
+    raw.o32_img = (int64_t)g.OC * g.OH * g.OW;
+    raw.o32_ch = g.OH * g.OW;
+    raw.o32_px = 1;
+    {
+      KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+      launch_wave_sliced(mode, (unsigned)(wnb * kslices), s, xp, wp, ws, g, raw);
+    }
+    int rc = check_launch("conv_wave (K slices)");
+    if (rc) return rc;
+    const int64_t total = g.P * (ep.out_mode == OUT_I8_ACT ? ep.out_cp / 4 : (g.OC + 3) / 4);
+    if (ep.out_mode == OUT_I8_ACT)
+      k_slices_finish<OUT_I8_ACT><<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const int32_t*>(ws), out, kslices, g.slice_stride, g, ep);
+    else
+      k_slices_finish<OUT_I32_NCHW><<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const int32_t*>(ws), out, kslices, g.slice_stride, g, ep);
+    return check_launch("conv K-slice finish");
+  }
   if (cfg >= 0) {
     const int mode = rows ? WAVE_ROWS
                           : (!g.dw && g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)

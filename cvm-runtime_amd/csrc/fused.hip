@@ -229,7 +229,8 @@ int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void
 static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                          const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8, int64_t nhwc_image_stride,
                          int n, int ic, int h, int wd, int oc, int kh, int kw,
-                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream,
+                         void* ws = nullptr, size_t ws_bytes = 0, size_t* ws_query = nullptr) {
   if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
   if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
       pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
@@ -254,8 +255,31 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
     ep.o32_ch = 1;
     ep.o32_px = oc;
   }
-  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep,
-                    as_stream(stream));
+  if (ws_query) {   // size question only
+    *ws_query = nhwc_image_stride >= 0 ? 0 : conv_slices_workspace_bytes(g, ep);
+    return CVMHIP_OK;
+  }
+  if (nhwc_image_stride >= 0) ws = nullptr;
+  return conv_igemm_ws(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep, ws, ws_bytes,
+                       as_stream(stream));
+}
+
+size_t cvmhip_conv2d_i8_workspace_bytes(int has_residual, int n, int ic, int h, int wd, int oc, int kh, int kw,
+                                        int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w) {
+  size_t bytes = 0;
+  const int dummy = 0;
+  const int rc = conv2d_i8_any(&dummy, &dummy, nullptr, nullptr, has_residual ? &dummy : nullptr, nullptr, const_cast<int*>(&dummy), 1, -1,
+                               n, ic, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, nullptr, nullptr, 0, &bytes);
+  return rc == CVMHIP_OK ? bytes : 0;
+}
+
+int cvmhip_conv2d_i8_ws(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                        const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
+                        int n, int ic, int h, int wd, int oc, int kh, int kw,
+                        int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, out_is_i8, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
+                       pad_h, pad_w, dil_h, dil_w, stream, workspace, workspace_bytes);
 }
 
 int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,

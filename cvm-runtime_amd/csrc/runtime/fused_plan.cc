@@ -575,6 +575,18 @@ void HipGraphRuntime::BuildPlan() {
   }
   for (const NodeEntry& e : outputs_) need_i32(entry_id(e));
 
+  // ---- workspaces of K-sliced launches (layers with a handful of output pixels and a very long K)
+  for (PlanStep& st : plan) {
+    if (st.kind != PlanStep::CONV || st.stem || st.nhwc) continue;
+    const size_t bytes = cvmhip_conv2d_i8_workspace_bytes(st.src2 != kNone, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh, st.sw,
+                                                          st.ph, st.pw, st.dh, st.dw);
+    if (bytes == 0) continue;
+    auto buf = std::make_shared<DeviceBuffer>();
+    Check(cvmhip_alloc(&buf->ptr, bytes), "K-slice workspace");
+    st.ws = buf;
+    st.ws_bytes = bytes;
+  }
+
   if (i8_bytes > 0) {
     Check(cvmhip_alloc(&i8_slab_, i8_bytes), "allocate int8 activation storage");
     for (uint32_t e = 0; e < ne; ++e)
@@ -616,9 +628,10 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
         break;
       }
       const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
-      Check(cvmhip_conv2d_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res,
-                             &st.chain2, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh,
-                             st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "conv2d_i8");
+      Check(cvmhip_conv2d_i8_ws(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res,
+                                &st.chain2, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh,
+                                st.sw, st.ph, st.pw, st.dh, st.dw, st.ws ? static_cast<DeviceBuffer*>(st.ws.get())->ptr : nullptr,
+                                st.ws_bytes, stream_), "conv2d_i8");
       break;
     }
     case PlanStep::DWCONV: {

@@ -100,6 +100,8 @@ struct PlanStep {
   std::shared_ptr<void> weights;  // packed filter (device)
   std::shared_ptr<void> aux;      // row-window copy of the input (device), see cvmhip_pack_stem_input
   bool stem = false;              // CONV through the row-window form
+  std::shared_ptr<void> ws;       // CONV: workspace of a K-sliced launch (cvmhip_conv2d_i8_ws), or empty
+  size_t ws_bytes = 0;
   bool dw_mfma = false;           // DWCONV through the implicit-GEMM kernel (filter packed as diagonal blocks)
   bool nhwc = false;              // CONV writes int32 pixel-major rows into a slice of entry dst (a fused detection head)
   int64_t dst_off = 0, img_stride = 0;  // that slice: first element, and elements from one image to the next

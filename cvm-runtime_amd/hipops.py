@@ -380,6 +380,26 @@ def conv2d_i8(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=
     return out
 
 
+def conv2d_i8_ws(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, out_is_i8=True,
+                 strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """conv2d_i8 with the workspace the library asks for (K slices over the grid for small-batch dense
+    layers); returns (output, workspace bytes used)."""
+    L = lib()
+    L.cvmhip_conv2d_i8_workspace_bytes.restype = ctypes.c_size_t
+    oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    need = L.cvmhip_conv2d_i8_workspace_bytes(0, n, ic, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                              dilation[0], dilation[1])
+    ws = _workspace(need, xp.device) if need else None
+    if out_is_i8:
+        out = _act_buffer(n * oh * ow, oc, xp.device)
+    else:
+        out = torch.empty((n, oc, oh, ow), dtype=torch.int32, device=xp.device)
+    check(L.cvmhip_conv2d_i8_ws(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None, None, None,
+                                _vp(out), int(out_is_i8), n, ic, h, w, oc, kh, kw, strides[0], strides[1],
+                                padding[0], padding[1], dilation[0], dilation[1], _vp(ws), ctypes.c_size_t(need), _stream()))
+    return out, need
+
+
 def conv2d_i8_nhwc(xp, n, ic, h, w, wp, oc, kh, kw, out, offset, image_stride, bias=None, chain1=None,
                    strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
     """The convolution's int32 result written pixel-major into the flat int32 tensor `out`:

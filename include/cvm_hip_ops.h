@@ -247,6 +247,19 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                      const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
                      int n, int ic, int h, int wd, int oc, int kh, int kw,
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* The same with a workspace.  A layer with at most 64 output pixels and K = kh*kw*ic >= 8192 (dense at a small
+ * batch: ops.cc:34-75 computed as a convolution; VGG-16's 25088 -> 4096 layer) is all filter streaming, and
+ * one workgroup per 32 output channels cannot keep HBM busy: with a workspace K is cut into up to 4 slices
+ * computed by different workgroups (int32 partial sums, added in a fixed order by a second kernel, so the
+ * result is the same wrap-around sum).  cvmhip_conv2d_i8_workspace_bytes returns the size needed (0: the
+ * layer does not qualify, pass NULL); with workspace NULL the call equals cvmhip_conv2d_i8. */
+size_t cvmhip_conv2d_i8_workspace_bytes(int has_residual, int n, int ic, int h, int wd, int oc, int kh, int kw,
+                                        int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+int cvmhip_conv2d_i8_ws(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                        const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8,
+                        int n, int ic, int h, int wd, int oc, int kh, int kw,
+                        int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                        void* workspace, size_t workspace_bytes, void* stream);
 /* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values
  * are contiguous at out + n*image_stride (elements).  This is what conv2d -> transpose(0,2,3,1) ->
  * reshape -> concatenate produces for a detection head (transpose: ops.cc:743-789, concatenate:

@@ -186,6 +186,38 @@ def test_conv2d_i8_random_geometries(case, dev):
             eq(out.cpu().numpy(), ref, "conv2d_i8 -> int32 (%s)" % kind)
 
 
+KSLICE_CASES = [
+    # n, ic, h, w, oc, k   (output 1x1: a dense layer over the flattened map, or a plain dense layer)
+    (16, 512, 7, 7, 256, 7),      # the shape of VGG-16's first dense layer, fewer units
+    (5, 8192, 1, 1, 100, 1),      # plain dense, ragged unit count, K exactly at the threshold
+    (33, 1024, 3, 3, 64, 3),      # 33 rows: second half of the pixel tile partly empty
+    (1, 9216, 1, 1, 8192, 1),     # more than 256 tiles: not sliced, same answer
+    (2, 4096, 1, 1, 64, 1),       # K below the threshold: no workspace
+]
+
+
+@pytest.mark.parametrize("i8", [True, False])
+@pytest.mark.parametrize("case", KSLICE_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%d" % c)
+def test_conv2d_i8_in_k_slices_equals_the_plain_launch(case, i8, dev):
+    n, ic, h, w, oc, k = case
+    cid = "kslice-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    shift = max(1, int(np.ceil(np.log2(ic * k * k * 127 * 127 / 100.0))))
+    ch = [("relu",), ("cvm_right_shift", 8, shift)] if i8 else []
+    ref = run_chain(oracle.conv2d(x, wt, b, (1, 1), (0, 0), (1, 1), 1), ch)
+    xp, wp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev))
+    out, used = hipops.conv2d_i8_ws(xp, n, ic, h, w, wp, oc, k, k, T(b, dev), hipops.chain(*ch) if ch else None, i8)
+    tiles = (oc + 31) // 32
+    assert (used > 0) == (ic * k * k >= 8192 and tiles <= 256)
+    if i8:
+        eq(act_to_nchw(out, n, oc, 1, 1), ref, "K-sliced conv2d_i8")
+    else:
+        torch.cuda.synchronize()
+        eq(out.cpu().numpy(), ref, "K-sliced conv2d_i8 -> int32")
+
+
 HEAD_CASES = [
     # n, ic, h, w, oc, k, pad, elements before the slice, elements after it
     (1, 64, 8, 8, 84, 3, 1, 0, 0),        # SSD class head: 4 anchors x 21 classes
