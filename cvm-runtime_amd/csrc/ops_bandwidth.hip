@@ -292,6 +292,24 @@ __global__ void __launch_bounds__(256) k_reduce_wave(const int32_t* __restrict__
   }
 }
 
+// Short contiguous runs (the trailing dims are the reduced ones and hold at most a few hundred elements: a
+// sum over a 7x7 map, a max over 21 class scores): L lanes per output instead of a whole wavefront, so a
+// wavefront finishes 64 / L outputs at a time and neighbouring lanes read neighbouring elements.
+template <int OP, int L>
+__global__ void __launch_bounds__(256) k_reduce_rows(const int32_t* __restrict__ x, int32_t* __restrict__ y,
+                                                     int64_t ksize, int rsize) {
+  const int sub = threadIdx.x % L;
+  const int64_t step = ((int64_t)gridDim.x * blockDim.x) / L;
+  for (int64_t o = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / L; o < ksize; o += step) {
+    const int32_t* row = x + o * rsize;
+    int32_t acc = OP == CVMHIP_SUM ? 0 : row[0];
+    for (int r = sub; r < rsize; r += L) acc = rfun<OP>(acc, row[r]);
+#pragma unroll
+    for (int d = L / 2; d >= 1; d >>= 1) acc = rfun<OP>(acc, __shfl_xor(acc, d, 64));
+    if (sub == 0) y[o] = acc;
+  }
+}
+
 // Full reduction starting from 0 (the reference's "no axis" case, reduce.cc:42-47).
 template <int OP>
 __global__ void __launch_bounds__(1024) k_reduce_all(const int32_t* __restrict__ x, int32_t* __restrict__ y, int64_t n) {
@@ -588,6 +606,18 @@ int cvmhip_reduce(int op, const int32_t* x, const int64_t* xshape, int ndim,
   // contiguous run: the reduced dims are the trailing dims
   sh.contiguous = 1;
   for (int d = ndim - nreal; d < ndim; ++d) if (!red[d]) sh.contiguous = 0;
+  if (sh.contiguous && sh.rsize <= 512) {
+    if (sh.rsize <= 64) {
+      const unsigned grid = grid_for(ksize * 8, 256);
+      if (op == CVMHIP_SUM) k_reduce_rows<CVMHIP_SUM, 8><<<grid, 256, 0, s>>>(x, y, ksize, (int)sh.rsize);
+      else k_reduce_rows<CVMHIP_RMAX, 8><<<grid, 256, 0, s>>>(x, y, ksize, (int)sh.rsize);
+    } else {
+      const unsigned grid = grid_for(ksize * 32, 256);
+      if (op == CVMHIP_SUM) k_reduce_rows<CVMHIP_SUM, 32><<<grid, 256, 0, s>>>(x, y, ksize, (int)sh.rsize);
+      else k_reduce_rows<CVMHIP_RMAX, 32><<<grid, 256, 0, s>>>(x, y, ksize, (int)sh.rsize);
+    }
+    return check_launch("reduce");
+  }
   const int64_t threads = ksize * 64;
   if (op == CVMHIP_SUM) k_reduce_wave<CVMHIP_SUM><<<grid_for(threads, 256), 256, 0, s>>>(x, y, ksize, sh);
   else k_reduce_wave<CVMHIP_RMAX><<<grid_for(threads, 256), 256, 0, s>>>(x, y, ksize, sh);

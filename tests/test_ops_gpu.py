@@ -209,6 +209,12 @@ def test_reduce(op, dev):
                  "%s axes=%s keep=%s excl=%s" % (op, axes, keep, excl))
     gap = synth.tensor("reduce", "gap", (16, 2048, 7, 7), -127, 127)
     same(hipops.reduce(op, T(gap, dev), (2, 3)), oracle.reduce(op, gap, (2, 3)), "global pool")
+    # short contiguous runs on both sides of the lane-group sizes (1, 8, 9, 21, 64, 65, 300, 512, 513 elements)
+    for run in (1, 8, 9, 21, 64, 65, 300, 512, 513):
+        v = synth.tensor("reduce", "run%d" % run, (37, run), -2 ** 31, 2 ** 31 - 1)
+        same(hipops.reduce(op, T(v, dev), (1,)), oracle.reduce(op, v, (1,)), "run of %d" % run)
+        w = -np.abs(synth.tensor("reduce", "neg%d" % run, (5, 3, run), -1000, 1000)) - 1   # all negative: max stays negative
+        same(hipops.reduce(op, T(w, dev), (2,)), oracle.reduce(op, w, (2,)), "negative run of %d" % run)
     big = synth.tensor("reduce", "big", (1 << 20,), -2 ** 31, 2 ** 31 - 1)   # full reduction wraps
     same(hipops.reduce(op, T(big, dev)), oracle.reduce(op, big), "full")
 
