@@ -656,6 +656,33 @@ int cvmhip_concatenate(const int32_t* const* inputs, const int64_t* const* ishap
   return CVMHIP_OK;
 }
 
+// Batched 2-D transpose through LDS: x [B][R][C] -> y [B][C][R], both sides read and written in whole
+// 128-byte rows of a 32 x 32 tile (the padding column keeps the transposed LDS reads free of bank conflicts).
+// Covers every permutation that moves a trailing group of dims in front of the group before it, e.g. the
+// NCHW -> NHWC transpose (0, 2, 3, 1) of a detection head and the reference's fast path (1, 2, 0) (ops.cc:759-766).
+__global__ void __launch_bounds__(256) k_transpose2d(const int32_t* __restrict__ x, int32_t* __restrict__ y,
+                                                     int64_t rows, int64_t cols, int64_t tiles_r, int64_t tiles_c) {
+  __shared__ int32_t tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8 threads
+  const int64_t per_batch = tiles_r * tiles_c;
+  const int64_t b = blockIdx.x / per_batch;
+  const int64_t t = blockIdx.x - b * per_batch;
+  const int64_t tr = t / tiles_c, tc = t - tr * tiles_c;
+  const int32_t* xb = x + b * rows * cols;
+  int32_t* yb = y + b * rows * cols;
+#pragma unroll
+  for (int i = 0; i < 32; i += 8) {
+    const int64_t r = tr * 32 + ty + i, c = tc * 32 + tx;
+    if (r < rows && c < cols) tile[ty + i][tx] = xb[r * cols + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 32; i += 8) {
+    const int64_t c = tc * 32 + ty + i, r = tr * 32 + tx;
+    if (r < rows && c < cols) yb[c * rows + r] = tile[tx][ty + i];
+  }
+}
+
 int cvmhip_transpose(const int32_t* x, const int64_t* xshape, int ndim,
                      const int64_t* axes, int naxes, int32_t* y, void* stream) {
   if (ndim < 1 || ndim > CVM_MAXD || (naxes != 0 && naxes != ndim)) return arg_error("transpose");
@@ -670,6 +697,30 @@ int cvmhip_transpose(const int32_t* x, const int64_t* xshape, int ndim,
     m.ydim[j] = xshape[p];
     m.div[j] = 1; m.mod[j] = INT64_MAX; m.begin[j] = 0; m.step[j] = 1;
     m.xstride[j] = xstride[p];
+  }
+  // a prefix kept in place, then the trailing group of dims moved in front of the group before it?
+  {
+    int64_t perm[CVM_MAXD];
+    for (int j = 0; j < ndim; ++j) perm[j] = naxes ? (axes[j] < 0 ? axes[j] + ndim : axes[j]) : ndim - 1 - j;
+    int b = 0;
+    while (b < ndim && perm[b] == b) ++b;
+    if (b < ndim) {
+      const int mid = (int)perm[b];            // first dim of the trailing group
+      bool ok = mid > b;
+      for (int j = b; ok && j < ndim; ++j) ok = perm[j] == (j - b < ndim - mid ? mid + (j - b) : b + (j - b - (ndim - mid)));
+      if (ok) {
+        int64_t batch = 1, rows = 1, cols = 1;
+        for (int d = 0; d < b; ++d) batch *= xshape[d];
+        for (int d = b; d < mid; ++d) rows *= xshape[d];
+        for (int d = mid; d < ndim; ++d) cols *= xshape[d];
+        const int64_t tiles_r = (rows + 31) / 32, tiles_c = (cols + 31) / 32;
+        const int64_t blocks = batch * tiles_r * tiles_c;
+        if (rows > 1 && cols > 1 && blocks > 0 && blocks < 0x7fffffff) {
+          k_transpose2d<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(x, y, rows, cols, tiles_r, tiles_c);
+          return check_launch("transpose");
+        }
+      }
+    }
   }
   return launch_remap(x, y, m, stream, "transpose");
 }

@@ -230,6 +230,12 @@ def test_remap_ops(dev):
         same(hipops.transpose(t, axes), oracle.transpose(x, axes), "transpose %s" % (axes,))
     x3 = x[:, 0]
     same(hipops.transpose(T(x3, dev), (1, 2, 0)), oracle.transpose(x3, (1, 2, 0)), "transpose (1,2,0)")
+    # the tiled path (a trailing group of dims moved in front of the group before it), ragged against the 32x32 tile
+    for shape, axes in [((2, 33, 7, 9), (0, 2, 3, 1)), ((1, 126, 64, 64), (0, 2, 3, 1)), ((3, 5, 6, 40), (0, 3, 1, 2)),
+                        ((65, 31), (1, 0)), ((4, 3, 70), (2, 0, 1)), ((2, 3, 4, 5, 6), (0, 1, 4, 2, 3)),
+                        ((2, 1, 50), (0, 2, 1)), ((5, 1, 1, 8), (0, 3, 1, 2))]:
+        v = synth.tensor("remap", "t%s" % (shape,), shape, -2 ** 31, 2 ** 31 - 1)
+        same(hipops.transpose(T(v, dev), axes), oracle.transpose(v, axes), "transpose %s %s" % (shape, axes))
     for b, e, s in [((0, 0, 1), (3, 1, 4), (2, 1, 2)), ((2, 0, 3), (0, 1, 0), (-1, 1, -2)), ((1,), (3,), ())]:
         ref = oracle.strided_slice(x, b, e, s)
         same(hipops.strided_slice(t, b, e, s, ref.shape), ref, "strided_slice")
