@@ -956,22 +956,38 @@ k_conv_grouped(const int32_t* __restrict__ x, const int32_t* __restrict__ w, con
   }
 }
 
-// dense on int32 operands without narrowing: one wavefront per output element.
+// dense on int32 operands without narrowing (ops.cc:53-62 multiplies the full int32 values): one
+// wavefront per output column j and block of DENSE_MB rows, so a filter row is read once per block.
+constexpr int DENSE_MB = 8;
 __global__ void __launch_bounds__(256)
 k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const int32_t* __restrict__ bias,
-            int32_t* __restrict__ y, int64_t total, int k, int n) {
+            int32_t* __restrict__ y, int m, int k, int n) {
   const int lane = threadIdx.x & 63;
   const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  const int mblocks = (m + DENSE_MB - 1) / DENSE_MB;
+  const int64_t total = (int64_t)mblocks * n;
   for (int64_t o = wave; o < total; o += nwaves) {
-    const int64_t m = o / n;
-    const int j = (int)(o - m * n);
-    const int32_t* xr = x + m * k;
+    const int mb = (int)(o / n);
+    const int j = (int)(o - (int64_t)mb * n);
+    const int m0 = mb * DENSE_MB;
+    const int rows = m - m0 < DENSE_MB ? m - m0 : DENSE_MB;
     const int32_t* wr = w + (int64_t)j * k;
-    int32_t acc = 0;
-    for (int t = lane; t < k; t += 64) acc = wadd(acc, wmul(xr[t], wr[t]));
-    for (int d = 32; d >= 1; d >>= 1) acc = wadd(acc, __shfl_xor(acc, d, 64));
-    if (lane == 0) y[o] = wadd(acc, bias ? bias[j] : 0);
+    int32_t acc[DENSE_MB];
+#pragma unroll
+    for (int r = 0; r < DENSE_MB; ++r) acc[r] = 0;
+    for (int t = lane; t < k; t += 64) {
+      const int32_t wv = wr[t];
+#pragma unroll
+      for (int r = 0; r < DENSE_MB; ++r)
+        if (r < rows) acc[r] = wadd(acc[r], wmul(x[(int64_t)(m0 + r) * k + t], wv));
+    }
+#pragma unroll
+    for (int r = 0; r < DENSE_MB; ++r) {
+      int32_t a = acc[r];
+      for (int d = 32; d >= 1; d >>= 1) a = wadd(a, __shfl_xor(a, d, 64));
+      if (lane == 0 && r < rows) y[(int64_t)(m0 + r) * n + j] = wadd(a, bias ? bias[j] : 0);
+    }
   }
 }
 
@@ -1416,8 +1432,8 @@ int cvmhip_dense(const int32_t* x, const int32_t* w, const int32_t* bias, int32_
   if (!x || !w || !y || m < 1 || k < 1 || n < 1) return arg_error("dense");
   hipStream_t s = as_stream(stream);
   if (operand_bits > 8) {
-    const int64_t total = (int64_t)m * n;
-    k_dense_i32<<<grid_for(total * 64, 256, 1 << 20), 256, 0, s>>>(x, w, bias, y, total, k, n);
+    const int64_t total = (int64_t)((m + DENSE_MB - 1) / DENSE_MB) * n;
+    k_dense_i32<<<grid_for(total * 64, 256, 1 << 20), 256, 0, s>>>(x, w, bias, y, m, k, n);
     return check_launch("dense_i32");
   }
   const size_t need = cvmhip_dense_workspace_bytes(m, k, n);

@@ -360,6 +360,9 @@ void HipGraphRuntime::BuildPlan() {
         }
         st.oc = (int)shape_[we][0];
         ok = shape_[we].size() == 2 && shape_[we][1] == (int64_t)st.c * st.kh * st.kw;
+        // dense multiplies the int32 values as they are (ops.cc:53-62; only conv2d narrows), so the int8 form
+        // is exact only for operands proven to lie in [-128, 127]; otherwise the node keeps its int32 kernel
+        ok = ok && safe[src] && safe[we];
       }
       // A few-channel input that only exists as int32 (the image itself) goes through the
       // row-window form: packed once into a zero-padded int8 tensor, convolved without masks.

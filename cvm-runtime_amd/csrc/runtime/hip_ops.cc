@@ -72,34 +72,17 @@ OpKernel ConvKernel() {
   return k;
 }
 
-// dense: [x, w, (b), y] is a 1x1 convolution over m "pixels"
+// dense: [x, w, (b), y].  The reference multiplies the int32 values as they are (ops.cc:53-62; only conv2d
+// narrows), and a declared precision of 8 bits does not bound a tensor: cvm_right_shift with p + b >= 32
+// does not clip (elemwise.cc:133-137) and can emit 128.  A node that runs on its own therefore always
+// takes the exact int32 kernel; the int8 matrix-core form is chosen by the fused planner, and only for
+// operands whose value range it has proven.
 OpKernel DenseKernel() {
   OpKernel k;
-  k.workspace_bytes = [](const OpCall& c) {
-    return cvmhip_dense_workspace_bytes((int)c.in[0].shape[0], (int)c.in[0].shape[1], (int)c.in[1].shape[0]);
-  };
-  k.prepare = [](OpCall& c) {
-    if (!c.in[1].is_param) return;
-    const int kk = (int)c.in[0].shape[1], n = (int)c.in[1].shape[0];
-    auto buf = std::make_shared<DeviceBuffer>();
-    Check(cvmhip_alloc(&buf->ptr, cvmhip_packed_weight_bytes(n, kk, 1, 1)), "dense filter buffer");
-    Check(cvmhip_pack_weights(c.in[1].data, buf->ptr, n, kk, 1, 1, c.stream), "dense filter pack");
-    c.state = buf;
-  };
   k.run = [](OpCall& c) {
     const int m = (int)c.in[0].shape[0], kk = (int)c.in[0].shape[1], n = (int)c.in[1].shape[0];
     const int32_t* bias = c.in.size() == 3 ? c.in[2].data : nullptr;
-    if (c.state) {
-      Check(cvmhip_conv2d_packed(c.in[0].data, static_cast<DeviceBuffer*>(c.state.get())->ptr, bias, c.out[0].data,
-                                 m, kk, 1, 1, n, 1, 1, 1, 1, 0, 0, 1, 1, c.workspace, c.workspace_bytes, c.stream), "dense");
-    } else {
-      // DensePrec guarantees operand precision <= 8 for every accepted graph; a single-operator call
-      // declares what its tensors hold, and wider operands take the exact int32 path
-      const int p0 = c.in[0].precision, p1 = c.in[1].precision;
-      const int bits = (p0 < 1 || p1 < 1) ? 32 : (p0 > p1 ? p0 : p1);
-      Check(cvmhip_dense(c.in[0].data, c.in[1].data, bias, c.out[0].data, m, kk, n, bits, c.workspace, c.workspace_bytes,
-                         c.stream), "dense");
-    }
+    Check(cvmhip_dense(c.in[0].data, c.in[1].data, bias, c.out[0].data, m, kk, n, 32, nullptr, 0, c.stream), "dense");
   };
   return k;
 }

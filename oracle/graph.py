@@ -48,9 +48,9 @@ def ref_lib():
     return _REFLIB
 
 
-def ref_inference(graph_json, param_bytes, input_bytes, device_type=0):
+def ref_inference(graph_json, param_bytes, input_bytes, device_type=0, fill=0):
     """CVMAPILoadModel + CVMAPIInference of the compiled reference (device 0 = CPU, 2 = FORMAL).
-    Returns (status, output bytes or None)."""
+    The output buffer is filled with byte `fill` before the call.  Returns (status, output bytes or None)."""
     L = ref_lib()
     if isinstance(graph_json, str):
         graph_json = graph_json.encode()
@@ -62,7 +62,7 @@ def ref_inference(graph_json, param_bytes, input_bytes, device_type=0):
     try:
         n = ctypes.c_ulonglong()
         L.CVMAPIGetOutputLength(net, ctypes.byref(n))
-        out = ctypes.create_string_buffer(n.value)
+        out = ctypes.create_string_buffer(bytes([fill]) * n.value, n.value)
         rc = L.CVMAPIInference(net, ctypes.c_char_p(input_bytes), len(input_bytes), out)
         return rc, (out.raw if rc == 0 else None)
     finally:

@@ -6,8 +6,10 @@ here once and committed as data:
 
   ops_golden.npz     outputs of cvm.runtime.cpu.<op> for tests/golden/cases.py
   host_golden.json   FInferShape/FInferPrecision results, C-API sizes and gas,
-                     output digests of the shrunk model graphs, status codes
-                     of malformed models
+                     output digests of the shrunk model graphs, output bytes and
+                     status of the post-processing models (argmax, detection,
+                     several heads, graph version cvm_1.1.0), status codes of
+                     malformed models
 
     python tests/golden/make_golden.py      (only where oracle/_ref exists)
 """
@@ -41,6 +43,61 @@ def small_models():
     }
 
 
+def _two_heads(cid, narrow, second_stride=1):
+    """data -> conv -> two convolution heads, each transposed and reshaped to (1, rows, channels)."""
+    g = graphgen.GraphBuilder(cid)
+    x = g.var("data", (1, 3, 8, 8), 8)
+    f = g.conv_relu_q(x, 8, 3, 1, 1)
+    heads = []
+    for oc, stride in ((4, 1), (2, second_stride)):
+        c, fan_in = g.conv(f, oc, 3, stride, 1)
+        if narrow:
+            c = g.rshift(c, graphgen.shift_for(fan_in))
+        n, ch, h, w = g.shape(c)
+        heads.append(g.reshape(g.transpose(c, (0, 2, 3, 1)), (1, h * w, ch)))
+    return g, heads
+
+
+def postprocess_models():
+    """Models that exercise CVMModel::SaveTensor / GetOutputLength (src/core/model.cc:181-331) beyond the plain
+    copy: name -> (builder, heads, postprocess, version).  Graph version cvm_1.1.0 recomputes arg_nodes and
+    node_row_ptr instead of verifying them (graph_runtime.cc:218-250); the keys stay in the JSON, because the
+    compiled reference reads node_row_ptr before that point and crashes on a graph without it."""
+    out = {}
+    g, h = _two_heads("post-det32", narrow=False)
+    out["detection_int32"] = (g, h, "detection", "cvm_1.0.0")          # rows of both heads side by side, int32
+    g, h = _two_heads("post-two8", narrow=True)
+    out["two_heads_int8"] = (g, h, None, "cvm_1.0.0")                  # outputs.size() > 1 without the tag, int8
+    g, h = _two_heads("post-det8", narrow=True)
+    out["detection_narrow_heads"] = (g, h, "detection", "cvm_1.0.0")   # the tag forces 4-byte outputs
+    g, h = _two_heads("post-rows", narrow=False, second_stride=2)
+    out["detection_rows_differ"] = (g, h, "detection", "cvm_1.0.0")    # 64 rows against 16: cannot concat
+    g, h = graphgen.resnet20_cifar(4)
+    out["argmax_batch4"] = (g, h, "argmax", "cvm_1.0.0")
+    g, h = graphgen.conv_op_graph(1, 16, 12, 12, 8)
+    out["version_1_1_0"] = (g, h, None, "cvm_1.1.0")
+    return out
+
+
+def stale_bookkeeping(js):
+    """The same graph with an arg_nodes list that names only the first variable and a dltype that is not
+    int32: version cvm_1.0.0 verifies both and rejects the graph, cvm_1.1.0 recomputes the one and never
+    reads the other (graph_runtime.cc:218-250)."""
+    d = json.loads(js)
+    d["arg_nodes"] = d["arg_nodes"][:1]
+    d["attrs"]["dltype"][1][0] = "float32"
+    return json.dumps(d)
+
+
+def build_postprocess_model(name):
+    g, heads, post, version = postprocess_models()[name]
+    js, pb = g.build(heads, postprocess=post, version=version)
+    if version == "cvm_1.1.0":
+        js = stale_bookkeeping(js)
+    x = synth.tensor("golden-" + name, "data", g.shape((0, 0)), -127, 127)
+    return js, pb, x
+
+
 def malformed_graphs():
     g, heads = graphgen.conv_op_graph(1, 16, 12, 12, 8)
     js, pb = g.build(heads)
@@ -65,6 +122,9 @@ def malformed_graphs():
     variant("node_op_kind", lambda d: d["nodes"][3].__setitem__("op", "tvm_op"))
     variant("row_ptr", lambda d: d["node_row_ptr"].__setitem__(2, 7))
     variant("device_index", lambda d: d["attrs"].__setitem__("device_index", ["list_int", [0] * len(d["attrs"]["shape"][1])]))
+    # what cvm_1.1.0 tolerates (see stale_bookkeeping) is an error at cvm_1.0.0
+    out["stale_bookkeeping_1_0_0"] = stale_bookkeeping(js)
+    out["stale_bookkeeping_1_1_0"] = stale_bookkeeping(js).replace("cvm_1.0.0", "cvm_1.1.0")
     out["not_json"] = "{ this is not json"
     del base
     return out
@@ -108,6 +168,14 @@ def main():
         rc, out = og.ref_inference(js, pb, x.astype(np.int8).tobytes())
         assert rc == 0
         host["models"][name] = {"query": q, "output_sha256": hashlib.sha256(out).hexdigest(), "output_head": list(out[:32])}
+    host["postprocess"] = {}
+    for name in postprocess_models():
+        js, pb, x = build_postprocess_model(name)
+        rc, q = og.ref_query(js, pb)
+        assert rc == 0, name
+        # the output buffer starts as 0x5A bytes, so bytes the reference leaves unwritten show as 90
+        rc, out = og.ref_inference(js, pb, x.astype(np.int8).tobytes(), fill=0x5A)
+        host["postprocess"][name] = {"query": q, "status": rc, "output_hex": out.hex() if rc == 0 else ""}
     L = og.ref_lib()
     import ctypes
     for name, js in malformed_graphs().items():

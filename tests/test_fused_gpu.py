@@ -573,3 +573,44 @@ def test_requantisation_scale_is_folded_into_the_chain(dev):
     ref = og.run_graph(js, graphgen.load_params(pb), xv)
     got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
+@pytest.mark.parametrize("four_d", [False, True])
+def test_dense_keeps_values_that_a_non_clipping_shift_leaves_outside_int8(four_d, dev):
+    """cvm_right_shift with p + b >= 32 does not clip (elemwise.cc:133-137): precision 8, shift 24 turns
+    2^31 - 1 into 128.  dense multiplies the int32 values as they are (ops.cc:53-62), so 128 * w must not
+    become -128 * w on the int8 matrix-core path."""
+    g = graphgen.GraphBuilder("dense-unsafe-%d" % four_d)
+    shape = (3, 16, 2, 2) if four_d else (3, 64)
+    x = g.var("data", shape, 32)
+    s = g.rshift(x, 24, 8)
+    d, _ = g.dense(g.flatten(s) if four_d else s, 24)
+    js, pb = g.build([d])
+    xv = synth.tensor("dense-unsafe", "data", shape, -2 ** 31, 2 ** 31 - 1)
+    xv.flat[:5] = [2 ** 31 - 1, 2 ** 31 - 1, -2 ** 31, 2 ** 31 - 2 ** 23, 2 ** 31 - 2 ** 22]
+    ref = og.run_graph(js, graphgen.load_params(pb), xv)
+    assert oracle.cvm_right_shift(xv, 8, 24).max() == 128      # the case exists in this input
+    want = np.concatenate([r.ravel() for r in ref])
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_FUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            out = m.inference(xv.astype(np.int32).tobytes())
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FUSE", None)
+        got = np.frombuffer(out, np.int32 if tsize == 4 else np.int8).astype(np.int32)
+        assert np.array_equal(got, want), "planner %s" % ("on" if mode == "1" else "off")
+
+
+def test_dense_int32_kernel_blocks_of_rows(dev):
+    """The exact int32 dense kernel (operands wider than 8 bits) with row counts around its row block."""
+    for m, k, n in ((1, 70, 5), (8, 64, 9), (9, 130, 33), (17, 257, 12)):
+        x = synth.tensor("dense32-%d" % m, "x", (m, k), -40000, 40000)
+        w = synth.tensor("dense32-%d" % m, "w", (n, k), -70000, 70000)
+        b = synth.tensor("dense32-%d" % m, "b", (n,), -2 ** 30, 2 ** 30)
+        ref = oracle.dense(x, w, b)
+        y = hipops.dense(T(x, dev), T(w, dev), T(b, dev), operand_bits=32)
+        torch.cuda.synchronize()
+        eq(y.cpu().numpy(), ref, "dense int32 m=%d" % m)

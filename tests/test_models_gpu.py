@@ -226,7 +226,7 @@ def test_random_graphs_node_by_node(seed, dev):
     _check(out, tsize, ref)
 
 
-def test_argmax_and_detection_postprocess(dev):
+def test_argmax_postprocess_batch1_against_the_oracle_logits(dev):
     g, heads = graphgen.resnet20_cifar(1)
     js, pb = g.build(heads, postprocess="argmax")
     x = synth.tensor("post", "data", (1, 3, 32, 32), -127, 127)
@@ -238,6 +238,51 @@ def test_argmax_and_detection_postprocess(dev):
     logits = og.run_graph(js, graphgen.load_params(pb), x)[0].ravel()
     # the reference compares the logits as int8 (src/core/model.cc:193)
     assert out[0] == int(np.argmax(logits.astype(np.int8)))
+
+
+def _golden_host():
+    import json
+    return json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "host_golden.json")))
+
+
+@pytest.mark.parametrize("name", ["detection_int32", "two_heads_int8", "detection_narrow_heads",
+                                  "detection_rows_differ", "argmax_batch4", "version_1_1_0"])
+@pytest.mark.parametrize("fuse", ["1", "0"])
+def test_postprocessing_models_match_the_bytes_the_reference_wrote(name, fuse, dev, capfd):
+    """CVMModel::SaveTensor / GetOutputLength (src/core/model.cc:181-331): rows of several heads side by side
+    in the int32 and the int8 form, heads whose row counts differ (ERROR_LOGIC), argmax over a batch with the
+    reference's loop bound, and a graph of version cvm_1.1.0.  Expected sizes, status and output bytes were
+    written by the compiled reference into an output buffer pre-filled with 0x5A (tests/golden/make_golden.py),
+    so bytes the reference leaves untouched must stay untouched here too."""
+    import ctypes
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import make_golden
+    want = _golden_host()["postprocess"][name]
+    js, pb, x = make_golden.build_postprocess_model(name)
+    os.environ["CVM_HIP_FUSE"] = fuse
+    try:
+        m = runtime.HipModel(js, pb)
+    finally:
+        os.environ.pop("CVM_HIP_FUSE", None)
+    try:
+        q = want["query"]
+        assert m.input_length == q["CVMAPIGetInputLength"]
+        assert m.output_length == q["CVMAPIGetOutputLength"]
+        assert runtime.CVMAPIGetInputTypeSize(m.net) == q["CVMAPIGetInputTypeSize"]
+        assert runtime.CVMAPIGetOutputTypeSize(m.net) == q["CVMAPIGetOutputTypeSize"]
+        assert runtime.CVMAPIGetStorageSize(m.net) == q["CVMAPIGetStorageSize"]
+        assert runtime.CVMAPIGetGasFromModel(m.net) == q["CVMAPIGetGasFromModel"]
+        data = x.astype(np.int8).tobytes()
+        for _ in range(2):                      # eager run, then the replayed graph
+            out = ctypes.create_string_buffer(b"\x5a" * m.output_length, m.output_length)
+            rc = runtime.lib().CVMAPIInference(m.net, ctypes.c_char_p(data), ctypes.c_int(len(data)), out)
+            assert rc == want["status"], name
+            if rc == 0:
+                assert out.raw.hex() == want["output_hex"], name
+    finally:
+        m.close()
+    capfd.readouterr()
 
 
 def test_graph_replay_equals_eager_on_every_replay(dev):
