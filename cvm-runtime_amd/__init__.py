@@ -33,6 +33,7 @@ def lib():
         _lib.cvmhip_last_error.restype = ctypes.c_char_p
         for name in ("cvmhip_conv2d_workspace_bytes", "cvmhip_dense_workspace_bytes",
                      "cvmhip_get_valid_counts_workspace_bytes", "cvmhip_nms_workspace_bytes",
+                     "cvmhip_nms_static_capacity_bytes",
                      "cvmhip_packed_weight_bytes", "cvmhip_packed_act_bytes", "cvmhip_packed_depthwise_bytes"):
             getattr(_lib, name).restype = ctypes.c_size_t
     return _lib

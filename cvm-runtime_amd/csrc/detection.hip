@@ -5,6 +5,8 @@
 // (score descending, original index ascending) is unique, so the result does
 // not depend on scheduling.  Nothing is copied back to the host: valid_count is
 // read on the device and every launch shape depends only on (batches, n, k).
+#include <mutex>
+
 #include "hip_common.h"
 
 namespace cvmhip {
@@ -517,6 +519,95 @@ k_nms_select(const int32_t* __restrict__ valid_count, int32_t* __restrict__ y,
   for (int64_t i = (int64_t)yi * k + tid; i < (int64_t)n * k; i += NMS_THREADS) yb[i] = -1;
 }
 
+// ---- scratch of the entry point that allocates nothing (cvmhip_non_max_suppression_static).
+// One array per GPU, part of the code object, held until the process ends.  In host code its name is only a
+// handle for hipGetSymbolAddress: the device address is looked up once per device, with that device
+// current, and only that address is ever passed to a kernel.
+constexpr size_t NMS_STATIC_WORDS = (size_t)1 << 19;   // 2 MiB: e.g. one batch of 37 000 rows of 6 values
+static __device__ __align__(256) int32_t g_nms_scratch[NMS_STATIC_WORDS];
+
+constexpr int NMS_MAX_DEVICES = 64;
+static std::mutex g_nms_scratch_mu;
+static void* g_nms_scratch_ptr[NMS_MAX_DEVICES] = {};
+
+// device address of the current device's copy of the array
+static int nms_static_scratch(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= NMS_MAX_DEVICES) {
+    set_error("non_max_suppression_static: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return CVMHIP_ERR_RUNTIME;
+  }
+  std::lock_guard<std::mutex> lock(g_nms_scratch_mu);
+  if (!g_nms_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_nms_scratch));
+    if (e != hipSuccess || !p) {
+      set_error("non_max_suppression_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return CVMHIP_ERR_RUNTIME;
+    }
+    g_nms_scratch_ptr[dev] = p;
+  }
+  *ptr = g_nms_scratch_ptr[dev];
+  return CVMHIP_OK;
+}
+
+static int nms_check_args(const int32_t* x, const int32_t* valid_count, const int32_t* y, int batches, int n, int k,
+                          int iou_threshold, int coord_start, int score_index, int id_index) {
+  if (!x || !valid_count || !y || x == y || batches < 1 || n < 1 || k < 2 || batches > 65535)
+    return arg_error("non_max_suppression");
+  if (iou_threshold <= 0) return arg_error("non_max_suppression.iou_threshold must be positive");
+  if (coord_start < 0 || coord_start + 4 > k || score_index < 0 || score_index >= k || id_index >= k)
+    return arg_error("non_max_suppression indices");
+  // 2^24 is the largest dimension the reference's shape check accepts (src/runtime/infer_attr.cc); without top_k
+  // the ranking compares all pairs of valid rows, as the reference's greedy walk does in its worst case
+  if (n > (1 << 24)) return arg_error("non_max_suppression: more than 2^24 anchors per batch");
+  return CVMHIP_OK;
+}
+
+// Validation and launches shared by the two entry points; `workspace` holds cvmhip_nms_workspace_bytes() bytes.
+static int nms_launch(int32_t* x, const int32_t* valid_count, int32_t* y,
+                      int batches, int n, int k, int max_output_size,
+                      int iou_threshold, int topk, int coord_start,
+                      int score_index, int id_index, int force_suppress,
+                      void* workspace, hipStream_t s) {
+  int32_t* order = reinterpret_cast<int32_t*>(workspace);
+  int32_t* nextneg = order + (size_t)batches * n;
+  int32_t* removed = nextneg + (size_t)batches * (n + 1);
+  int32_t* sorted = removed + (size_t)batches * n;
+  int32_t* rank = sorted + (size_t)batches * n * k;
+  uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
+  int rc;
+  if (topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N) {
+    k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, n, k, score_index, topk);
+    rc = check_launch("nms.topk_rank");
+  } else {
+    k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
+    dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
+    k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, n, k, score_index);
+    rc = check_launch("nms.rank");
+  }
+  if (rc) return rc;
+  dim3 grid((n + 255) / 256, batches);
+  k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, y, n, k, topk, (int64_t)n);
+  rc = check_launch("nms.scatter");
+  if (rc) return rc;
+  int rows = n < NMS_BM_ROWS ? n : NMS_BM_ROWS;  // upper bound of the rows the walk can see, when the matrix is used
+  if (topk >= 0 && topk < rows) rows = topk;
+  if (rows > 0 && k <= NMS_LDS_K) {
+    dim3 mgrid((rows + 3) / 4, (rows + 63) / 64, batches);
+    k_nms_mask<<<mgrid, 256, 0, s>>>(valid_count, sorted, mask, n, k, iou_threshold, topk, coord_start, id_index,
+                                     force_suppress, (int64_t)n);
+    rc = check_launch("nms.mask");
+    if (rc) return rc;
+  }
+  k_nms_select<<<batches, NMS_THREADS, 0, s>>>(valid_count, y, sorted, nextneg, removed, mask, n, k,
+                                               max_output_size, iou_threshold, topk, coord_start, id_index,
+                                               force_suppress, (int64_t)n);
+  return check_launch("nms.select");
+}
+
+
 }  // namespace cvmhip
 
 using namespace cvmhip;
@@ -555,48 +646,33 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
                                int iou_threshold, int topk, int coord_start,
                                int score_index, int id_index, int force_suppress,
                                void* workspace, size_t workspace_bytes, void* stream) {
-  if (!x || !valid_count || !y || x == y || batches < 1 || n < 1 || k < 2 || batches > 65535)
-    return arg_error("non_max_suppression");
-  if (iou_threshold <= 0) return arg_error("non_max_suppression.iou_threshold must be positive");
-  if (coord_start < 0 || coord_start + 4 > k || score_index < 0 || score_index >= k || id_index >= k)
-    return arg_error("non_max_suppression indices");
-  if (n > (1 << 18)) return arg_error("non_max_suppression: more than 2^18 anchors per batch is not supported");
+  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index);
+  if (rc) return rc;
   if (!workspace || workspace_bytes < cvmhip_nms_workspace_bytes(batches, n, k)) return arg_error("non_max_suppression workspace");
-  hipStream_t s = as_stream(stream);
-  int32_t* order = reinterpret_cast<int32_t*>(workspace);
-  int32_t* nextneg = order + (size_t)batches * n;
-  int32_t* removed = nextneg + (size_t)batches * (n + 1);
-  int32_t* sorted = removed + (size_t)batches * n;
-  int32_t* rank = sorted + (size_t)batches * n * k;
-  uint32_t* mask = reinterpret_cast<uint32_t*>(rank + (size_t)batches * n);
-  int rc;
-  if (topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N) {
-    k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, n, k, score_index, topk);
-    rc = check_launch("nms.topk_rank");
-  } else {
-    k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
-    dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
-    k_nms_rank<<<rgrid, 256, 0, s>>>(x, valid_count, rank, n, k, score_index);
-    rc = check_launch("nms.rank");
-  }
+  return nms_launch(x, valid_count, y, batches, n, k, max_output_size, iou_threshold, topk, coord_start, score_index,
+                    id_index, force_suppress, workspace, as_stream(stream));
+}
+
+size_t cvmhip_nms_static_capacity_bytes(void) { return sizeof(int32_t) * NMS_STATIC_WORDS; }
+
+int cvmhip_non_max_suppression_static(int32_t* x, const int32_t* valid_count, int32_t* y,
+                                      int batches, int n, int k, int max_output_size,
+                                      int iou_threshold, int topk, int coord_start,
+                                      int score_index, int id_index, int force_suppress, void* stream) {
+  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index);
   if (rc) return rc;
-  dim3 grid((n + 255) / 256, batches);
-  k_nms_scatter<<<grid, 256, 0, s>>>(x, valid_count, rank, order, sorted, y, n, k, topk, (int64_t)n);
-  rc = check_launch("nms.scatter");
-  if (rc) return rc;
-  int rows = n < NMS_BM_ROWS ? n : NMS_BM_ROWS;  // upper bound of the rows the walk can see, when the matrix is used
-  if (topk >= 0 && topk < rows) rows = topk;
-  if (rows > 0 && k <= NMS_LDS_K) {
-    dim3 mgrid((rows + 3) / 4, (rows + 63) / 64, batches);
-    k_nms_mask<<<mgrid, 256, 0, s>>>(valid_count, sorted, mask, n, k, iou_threshold, topk, coord_start, id_index,
-                                     force_suppress, (int64_t)n);
-    rc = check_launch("nms.mask");
-    if (rc) return rc;
+  const size_t need = cvmhip_nms_workspace_bytes(batches, n, k);
+  if (need > cvmhip_nms_static_capacity_bytes()) {
+    set_error("invalid argument: non_max_suppression_static: batches=%d n=%d k=%d needs %zu bytes of scratch, the static "
+              "buffer holds %zu; use cvmhip_non_max_suppression with a caller workspace",
+              batches, n, k, need, cvmhip_nms_static_capacity_bytes());
+    return CVMHIP_ERR_ARG;
   }
-  k_nms_select<<<batches, NMS_THREADS, 0, s>>>(valid_count, y, sorted, nextneg, removed, mask, n, k,
-                                               max_output_size, iou_threshold, topk, coord_start, id_index,
-                                               force_suppress, (int64_t)n);
-  return check_launch("nms.select");
+  void* scratch = nullptr;
+  const int rs = nms_static_scratch(&scratch);
+  if (rs) return rs;
+  return nms_launch(x, valid_count, y, batches, n, k, max_output_size, iou_threshold, topk, coord_start, score_index,
+                    id_index, force_suppress, scratch, as_stream(stream));
 }
 
 }  // extern "C"

@@ -290,6 +290,16 @@ def non_max_suppression(x, valid_count, y, iou_threshold=50, force_suppress=Fals
     return y
 
 
+def non_max_suppression_static(x, valid_count, y, iou_threshold=50, force_suppress=False, top_k=-1,
+                               id_index=0, coord_start=2, score_index=1, max_output_size=-1):
+    """The same operator through the entry point that allocates nothing (scratch inside the library)."""
+    b, n, k = x.shape
+    check(lib().cvmhip_non_max_suppression_static(_ptr(x), _ptr(valid_count), _ptr(y), b, n, k, max_output_size,
+                                                  iou_threshold, top_k, coord_start, score_index, id_index,
+                                                  int(bool(force_suppress)), _stream()))
+    return y
+
+
 # ---------------------------------------------------------------- fused int8 path
 # int8 activation tensors are flat torch int8 buffers in the library's own
 # layout (NHWC for up to 16 padded channels, else blocks of 32 pixels x 32

@@ -148,6 +148,18 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
                                int iou_threshold, int topk, int coord_start,
                                int score_index, int id_index, int force_suppress,
                                void* workspace, size_t workspace_bytes, void* stream);
+/* The same operator for callers that cannot allocate device memory or bring a workspace (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The scratch is
+ * a fixed array inside the library's code object, cvmhip_nms_static_capacity_bytes() bytes (2 MiB) per GPU,
+ * held until the process ends; a call whose cvmhip_nms_workspace_bytes(batches, n, k) exceeds it returns
+ * CVMHIP_ERR_ARG.  The call allocates and frees nothing.  All calls on one GPU share the array: calls that
+ * overlap in time on one GPU (two streams, two threads) race and must be serialised by the caller.  The
+ * first call on a device looks the array's address up (hipGetSymbolAddress); make it outside stream capture. */
+size_t cvmhip_nms_static_capacity_bytes(void);
+int cvmhip_non_max_suppression_static(int32_t* x, const int32_t* valid_count, int32_t* y,
+                                      int batches, int n, int k, int max_output_size,
+                                      int iou_threshold, int topk, int coord_start,
+                                      int score_index, int id_index, int force_suppress, void* stream);
 
 /* ---- device memory and streams: what a DeviceAPI subclass registered as
  * "device_api.hip" needs (include/cvm/runtime/device_api.h:43-108: SetDevice,
