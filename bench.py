@@ -26,17 +26,17 @@ PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 TRAFFIC_BYTES_PER_LAUNCH = {("k_conv_wave", 16): 12.84e6}
 
 
-def cpu_baseline(js1, pb1, budget_s=20.0):
-    """Reference CPU runtime (oracle/_ref, built from the reference sources) on
-    batch-1 inputs of the same model; falls back to the C restatement when the
-    reference build is absent.  Checker code is only timed here, never used to
-    produce the GPU result."""
+def cpu_baseline(js1, pb1, x1, budget_s=20.0):
+    """Reference CPU runtime (oracle/_ref, built from the reference sources) on the first image of the timed
+    batch, as a batch-1 model of the same graph; falls back to the C restatement when the reference build is
+    absent.  Checker code is only timed here, never used to produce the GPU result.  Returns the baseline
+    object and the int32 values the CPU runtime computed for that image (the parity check of the timed
+    configuration compares the GPU's first image with them)."""
     import numpy as np
     import oracle
     import oracle.graph as og
-    from cvm_runtime_amd import graphgen, synth
+    from cvm_runtime_amd import graphgen
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    x = synth.tensor("bench-cpu", "data", (1, 3, 224, 224), -127, 127)
     n = 0
     if oracle.have_ref():
         L = og.ref_lib()
@@ -44,9 +44,13 @@ def cpu_baseline(js1, pb1, budget_s=20.0):
         gj = js1.encode()
         rc = L.CVMAPILoadModel(ctypes.c_char_p(gj), len(gj), ctypes.c_char_p(pb1), len(pb1), ctypes.byref(net), 0, 0)
         assert rc == 0
-        out = ctypes.create_string_buffer(4000)
-        xb = x.astype(np.int8).tobytes()
-        L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out)   # warm-up
+        size, tsize = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        L.CVMAPIGetOutputLength(net, ctypes.byref(size))
+        L.CVMAPIGetOutputTypeSize(net, ctypes.byref(tsize))
+        out = ctypes.create_string_buffer(size.value)
+        xb = x1.astype(np.int8).tobytes()
+        assert L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out) == 0   # warm-up, and the values to compare
+        want = np.frombuffer(out.raw, np.int32 if tsize.value == 4 else np.int8).astype(np.int32)
         t0 = time.perf_counter()
         while True:
             L.CVMAPIInference(net, ctypes.c_char_p(xb), len(xb), out)
@@ -58,17 +62,91 @@ def cpu_baseline(js1, pb1, budget_s=20.0):
         kind = "reference"
     else:
         params = graphgen.load_params(pb1)
-        og.run_graph(js1, params, x)
+        want = np.concatenate([r.ravel() for r in og.run_graph(js1, params, x1)]).astype(np.int32)
         t0 = time.perf_counter()
         while True:
-            og.run_graph(js1, params, x)
+            og.run_graph(js1, params, x1)
             n += 1
             dt = time.perf_counter() - t0
             if dt > budget_s or n >= 1000:
                 break
         kind = "port"
     return {"value": n / dt, "unit": "images/s", "cores": cores, "kind": kind,
-            "sample": "%d batch-1 CVMAPIInference calls of the same ResNet-50 graph, %.1f s" % (n, dt)}
+            "sample": "%d batch-1 CVMAPIInference calls of the same graph on the first image of the timed batch, %.1f s" % (n, dt)}, want
+
+
+def layer_table(args, pkg, L, model, title):
+    """One row per launch of a step, in launch order.  Durations: HIP event pairs around every launch (minus
+    the cost of a pair, calibrated as in the headline run), or -- given the kernel trace of a rocprofv3 run of
+    this same command -- the median over the steps of the traced duration of the launch at that position.
+    Floors: algorithmic operations at 5 POP/s, algorithmic bytes at 8 TB/s, and the duration of a launch that
+    does nothing (a 256-byte copy kernel, launched 50 times back to back after the steps)."""
+    import csv
+    import statistics
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.time_run(args.steps)
+    torch.cuda.synchronize()
+    plain_us = (time.perf_counter() - t0) / args.steps * 1e6
+    L.cvmhip_kernel_timing_begin()
+    model.time_run(args.steps)
+    torch.cuda.synchronize()
+    buf = ctypes.create_string_buffer(1 << 24)
+    pkg.check(L.cvmhip_kernel_timing_end_launches(buf, len(buf)))
+    launches = json.loads(buf.value.decode())
+    per_step = len(launches) // args.steps
+    assert per_step * args.steps == len(launches), "launch count is not a multiple of the step count"
+    step = launches[:per_step]
+    pair_us = [statistics.median(launches[k * per_step + i]["ms"] * 1e3 for k in range(args.steps)) for i in range(per_step)]
+    pair_cost = max(0.0, (sum(pair_us) - plain_us) / per_step)
+    dur = [max(u - pair_cost, 0.0) for u in pair_us]
+    source = "event pairs minus %.2f us per pair" % pair_cost
+    # the launch that does nothing
+    a = torch.zeros(64, dtype=torch.int32, device="cuda")
+    b = torch.zeros(64, dtype=torch.int32, device="cuda")
+    for _ in range(50):
+        pkg.check(L.cvmhip_copy_kernel(ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(a.data_ptr()), ctypes.c_size_t(256), None))
+    torch.cuda.synchronize()
+    empty_us = None
+    if args.trace:
+        rows = list(csv.DictReader(open(args.trace)))
+        base = lambda n: n.split("(")[0].split("<")[0].replace("void ", "").split("::")[-1]
+        seq = [(base(r["Kernel_Name"]), (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3) for r in rows]
+        want = [e["kernel"] for e in step]
+        alias = {"k_max_pool_i8": ("k_max_pool_i8", "k_max_pool_i8x16")}
+        same = lambda got, w: got == w or got in alias.get(w, ())
+        hits, i = [], 0
+        while i + per_step <= len(seq):
+            if all(same(seq[i + j][0], want[j]) for j in range(per_step)):
+                hits.append(i)
+                i += per_step
+            else:
+                i += 1
+        assert hits, "the trace holds no run of launches that matches a step"
+        dur = [statistics.median(seq[h + j][1] for h in hits) for j in range(per_step)]
+        source = "rocprofv3 kernel trace, median of %d steps" % len(hits)
+        empties = [d for n, d in seq if n == "k_copy16"]
+        if empties:
+            empty_us = statistics.median(empties[-50:])
+    print("# %s, batch %d: %d launches per step, %.1f us per step without instrumentation" % (title, args.batch, per_step, plain_us))
+    print("# durations: %s; sum %.1f us" % (source, sum(dur)))
+    if empty_us is not None:
+        print("# a launch that does nothing (256-byte copy kernel): %.2f us in the same trace" % empty_us)
+    print("# floors: ops / 5 POP/s, bytes / 8 TB/s; excess = duration - max(floors)")
+    print("%3s %-14s %-78s %8s %8s %7s %7s %7s %7s %7s" % ("#", "kernel", "launch", "GOP", "MB", "us", "mfma_us", "hbm_us", "TOP/s", "TB/s"))
+    tot_ops = tot_bytes = 0.0
+    for i, (e, u) in enumerate(zip(step, dur)):
+        is_conv = e["kernel"].startswith("k_conv")
+        ops = e["work"] if is_conv else 0.0
+        byts = e["bytes"] if is_conv else e["work"]
+        tot_ops += ops
+        tot_bytes += byts
+        print("%3d %-14s %-78s %8.3f %8.2f %7.2f %7.2f %7.2f %7.0f %7.2f" % (
+            i, e["kernel"], e["desc"][:78], ops / 1e9, byts / 1e6, u, ops / 5e15 * 1e6, byts / 8e12 * 1e6,
+            ops / max(u, 1e-3) / 1e6, byts / max(u, 1e-3) / 1e6))
+    print("# step: %.1f GOP = %.1f us at 5 POP/s; %.1f MB = %.1f us at 8 TB/s" % (
+        tot_ops / 1e9, tot_ops / 5e15 * 1e6, tot_bytes / 1e6, tot_bytes / 8e12 * 1e6))
 
 
 def main():
@@ -86,6 +164,12 @@ def main():
     ap.add_argument("--suite", choices=("model", "ops"), default="model",
                     help="model: the headline line (default); ops: one JSON line per bandwidth-bound operator at the "
                          "shapes of the configurations, achieved GB/s against the 8 TB/s HBM peak")
+    ap.add_argument("--layers", action="store_true",
+                    help="print one row per launch of a step instead of the headline line: what the launch is, its "
+                         "duration, and its floors (matrix-core peak, HBM peak, an empty launch)")
+    ap.add_argument("--trace", default=None,
+                    help="with --layers: kernel_trace.csv of a `rocprofv3 --kernel-trace` run of this same command; "
+                         "the durations of the table are then the medians of the trace instead of event pairs")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain copy kernel of known size (256 MiB read + 256 MiB written, 5 times): "
                          "under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counter reading gives the scale of the counters")
@@ -127,6 +211,11 @@ def main():
     model.time_run(max(args.warmup, 1))
     torch.cuda.synchronize()
 
+    if args.layers:
+        layer_table(args, pkg, L, model, names[args.workload])
+        model.close()
+        return
+
     # timed region: exactly `steps` graph runs, nothing else on the stream
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -146,6 +235,7 @@ def main():
     pkg.check(L.cvmhip_kernel_timing_end(buf, len(buf)))
     kt = json.loads(buf.value.decode())
     raw = model.get_output()
+    out_tsize = runtime.CVMAPIGetOutputTypeSize(model.net)
     out = np.frombuffer(raw + b"\0" * (-len(raw) % 4), np.int32)
 
     # two models of the same graph in flight (two nets on two host threads, each with its own stream, as the
@@ -229,6 +319,8 @@ def main():
                      "frac": achieved / PEAK_I8_TOPS,
                      "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((dom, args.batch)) if args.workload == "resnet50" else None,
                      "traffic_unit": "bytes per launch",
+                     "traffic_source": "recorded from the FETCH_SIZE / WRITE_SIZE counter passes summarised in "
+                                       "profiles/k_conv_wave_resnet50_b16_traffic.txt, not measured by this run",
                      "kernel": dom, "launches_per_step": conv["launches"] / args.steps,
                      "avg_launch_us": avg_s * 1e6, "avg_launch_us_with_event_pair": raw_avg_s * 1e6,
                      "event_pair_cost_us": pair_cost_us, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
@@ -238,10 +330,35 @@ def main():
                                                  "ms_per_step": all_s * 1e3 / args.steps},
                      "other_kernels_ms_per_step": {k: v["ms"] / args.steps for k, v in kt.items() if k != dom}},
     }
-    if not args.no_cpu_baseline and args.workload == "resnet50":
-        g1, h1 = graphgen.resnet50(1)
-        js1, pb1 = g1.build(h1)
-        line["cpu_baseline"] = cpu_baseline(js1, pb1)
+    # batch 1 of the same graph (the other half of the metric), measured the same way: input resident, `steps` runs
+    b1 = {"resnet50": lambda: graphgen.resnet50(1), "vgg16": lambda: graphgen.vgg16(1),
+          "resnet20": lambda: graphgen.resnet20_cifar(1), "ssd512": graphgen.ssd_mobilenet}[args.workload]
+    g1, h1 = b1()
+    js1, pb1 = g1.build(h1)
+    if args.batch != 1:
+        m1 = runtime.HipModel(js1, pb1)
+        m1.set_input(x[:1].tobytes())
+        m1.time_run(max(args.warmup, 1))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        m1.time_run(args.steps)
+        torch.cuda.synchronize()
+        b1_s = (time.perf_counter() - t0) / args.steps
+        m1.close()
+        line["config"]["images_per_s_batch1"] = 1.0 / b1_s
+        line["config"]["ms_per_step_batch1"] = b1_s * 1e3
+    # The CPU baseline leg runs the reference CPU runtime on the first image of the timed batch; its values also
+    # check the timed configuration: the GPU's output for that image must equal them bit for bit.
+    if not args.no_cpu_baseline:
+        base, want = cpu_baseline(js1, pb1, x[:1].astype(np.int32), 20.0 if args.workload == "resnet50" else 5.0)
+        line["cpu_baseline"] = base
+        per_image = len(raw) // args.batch
+        got = np.frombuffer(raw[:per_image], np.int32 if out_tsize == 4 else np.int8).astype(np.int32)
+        ok = got.shape == want.shape and bool(np.array_equal(got, want))
+        line["parity_checked"] = ok
+        if not ok:
+            print(json.dumps(line))
+            sys.exit("bench.py: the output of the timed configuration differs from the CPU runtime's on the first image")
     print(json.dumps(line))
 
 

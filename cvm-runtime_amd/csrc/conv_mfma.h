@@ -104,6 +104,12 @@ __host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c
   }
 }
 
+// Forced kernel choice of the calling thread (thread-local; automatic by default): which implicit-GEMM kernel,
+// which configuration of the wavefront kernel (-1 = automatic), which tile of the tiled kernel (0 = automatic).
+enum { CONV_KERNEL_AUTO = 0, CONV_KERNEL_LDS = 1, CONV_KERNEL_WAVE = 2 };
+struct ConvTuning { int kernel, wave_cfg, tile_wm, tile_wn; };
+void set_conv_tuning(const ConvTuning& t);
+
 int pad_channels(int c);
 size_t packed_act_bytes(int64_t npix, int c);
 

@@ -992,6 +992,10 @@ k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const 
 }
 
 // ---------------------------------------------------------------- host side
+// Kernel choice forced by the calling thread (tests and tuning runs); automatic unless set.
+static thread_local ConvTuning t_conv_tuning = {CONV_KERNEL_AUTO, -1, 0, 0};
+void set_conv_tuning(const ConvTuning& t) { t_conv_tuning = t; }
+
 int pad_channels(int c) {
   if (c <= 4) return 4;
   if (c <= 8) return 8;
@@ -1243,6 +1247,26 @@ size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep) {
   return ks > 1 ? (size_t)ks * g.N * g.OC * g.OH * g.OW * 4 : 0;
 }
 
+// Algorithmic HBM bytes of a convolution launch (true channels, each tensor once) and a one-line description
+// of it, for the measurement harness (only evaluated while kernel timing is on).
+static double conv_bytes(const ConvGeom& g, const Epilogue& ep) {
+  const double c = g.C ? g.C : g.Cp;
+  const double in = (double)g.N * g.H * g.W * (g.row_bytes ? 4.0 : c);
+  const double flt = (double)g.OC * (g.dw ? 1.0 : c) * g.taps;
+  const double outb = (double)g.P * g.OC * (ep.out_mode == OUT_I8_ACT ? 1.0 : 4.0);
+  return in + flt + outb + (ep.residual ? (double)g.P * g.OC : 0.0);
+}
+struct ConvDesc {
+  char text[160];
+  ConvDesc(const ConvGeom& g, const Epilogue& ep, const char* kernel, int cfg, int mode, long grid) {
+    text[0] = 0;
+    if (!kernel_timing_enabled()) return;
+    snprintf(text, sizeof(text), "%s%dx%d/%d %d->%d in %dx%dx%d out %dx%d%s%s %s cfg %d mode %d grid %ld", g.dw ? "dw " : "",
+             g.KH, g.KW, g.SH, g.C ? g.C : g.Cp, g.OC, g.N, g.H, g.W, g.OH, g.OW, ep.residual ? " +res" : "",
+             ep.out_mode == OUT_I8_ACT ? " i8" : " i32", kernel, cfg, mode, grid);
+  }
+};
+
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
   return conv_igemm_ws(xp, wp, out, g, ep_in, nullptr, 0, s);
 }
@@ -1285,21 +1309,21 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   int wm = g.OC > 64 ? 2 : 1, wn = 2;
   if (blocks(64 * wm, 64 * wn) < 512 && wn == 2) wn = 1;
   if (blocks(64 * wm, 64 * wn) < 512 && wm == 2) wm = 1;
-  // tuning hook: CVM_HIP_TILE="wm,wn" forces a tile shape (read once)
-  static const char* forced = getenv("CVM_HIP_TILE");
-  if (forced && forced[0] >= '1' && forced[0] <= '2' && forced[1] == ',' && forced[2] >= '1' && forced[2] <= '2') {
-    wm = forced[0] - '0';
-    wn = forced[2] - '0';
+  // test and tuning hook (cvmhip_set_conv_tuning): a forced tile shape of the tiled kernel
+  const ConvTuning tune = t_conv_tuning;
+  if (tune.tile_wm >= 1 && tune.tile_wm <= 2 && tune.tile_wn >= 1 && tune.tile_wn <= 2) {
+    wm = tune.tile_wm;
+    wn = tune.tile_wn;
   }
   g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
   g.div_ow = make_fastdiv((uint32_t)g.OW);
   g.div_ct = make_fastdiv((uint32_t)(g.dw ? 1 : g.Cp >= 32 ? g.Cp / 32 : 1));
   g.div_kw = make_fastdiv((uint32_t)g.KW);
   // kernel choice: the wavefront-private kernel when the layout allows it and its grid fits the chip,
-  // else the LDS-tiled kernel.  Test and tuning hooks (read per call): CVM_HIP_CONV=lds|wave forces
-  // one of them, CVM_HIP_WAVECFG=<index> a configuration.
-  const char* conv_kind = getenv("CVM_HIP_CONV");
-  const char* wave_forced = getenv("CVM_HIP_WAVECFG");
+  // else the LDS-tiled kernel.  The calling thread's tuning (cvmhip_set_conv_tuning) can force one of
+  // them or a configuration of the wavefront kernel; nothing is read from the environment here.
+  const bool force_lds = tune.kernel == CONV_KERNEL_LDS, force_wave = tune.kernel == CONV_KERNEL_WAVE;
+  const int wave_forced = tune.wave_cfg;
   const bool nopad = g.PH == 0 && g.PW == 0;
   const bool rows = g.row_bytes != 0;
   const bool wave_ok = rows || ((g.Cp % 32) == 0 && (nopad || (g.KH <= 32 && g.KW <= 32)));
@@ -1309,11 +1333,11 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     // unless the grid leaves most of the chip idle
     if (!wave_ok) return arg_error("depthwise geometry");
     cfg = wave_cfg_blocks(kWaveCfgs[6], g) >= 192 || g.taps < 8 ? 6 : 5;
-    if (wave_forced && wave_forced[0] >= '4' && wave_forced[0] <= '6') cfg = wave_forced[0] - '0';
+    if (wave_forced >= 4 && wave_forced <= 6) cfg = wave_forced;
   } else
-  if (conv_kind && conv_kind[0] == 'l' && !rows) cfg = -1;
-  if (wave_ok && conv_kind && conv_kind[0] == 'w' && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
-  if (wave_ok && cfg >= 0 && wave_forced && wave_forced[0] >= '0' && wave_forced[0] < '0' + kNumWaveCfgs) cfg = wave_forced[0] - '0';
+  if (force_lds && !rows) cfg = -1;
+  if (wave_ok && force_wave && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
+  if (wave_ok && cfg >= 0 && wave_forced >= 0 && wave_forced < kNumWaveCfgs) cfg = wave_forced;
   const int kslices = ws ? conv_slices(g, ep) : 1;
   if (kslices > 1 && wave_ok) {
     const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
@@ -1335,7 +1359,8 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     raw.o32_ch = g.OH * g.OW;
     raw.o32_px = 1;
     {
-      KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+      const ConvDesc desc(g, ep, "wave-sliced", cfg, mode, (long)(wnb * kslices));
+      KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s, conv_bytes(g, ep), desc.text);
       launch_wave_sliced(mode, (unsigned)(wnb * kslices), s, xp, wp, ws, g, raw);
     }
     int rc = check_launch("conv_wave (K slices)");
@@ -1355,7 +1380,9 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
     g.octiles = (g.OC + 32 * kWaveCfgs[cfg].tm - 1) / (32 * kWaveCfgs[cfg].tm);
     g.div_octiles = make_fastdiv((uint32_t)g.octiles);
-    KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (g.dw ? 1.0 : (double)(g.C ? g.C : g.Cp)), s);
+    const ConvDesc desc(g, ep, "wave", cfg, mode, (long)wnb);
+    KernelTimer timer("k_conv_wave", 2.0 * (double)g.P * g.OC * (double)g.taps * (g.dw ? 1.0 : (double)(g.C ? g.C : g.Cp)), s,
+                      conv_bytes(g, ep), desc.text);
     launch_wave(cfg, mode, (unsigned)wnb, s, xp, wp, out, g, ep);
     return check_launch("conv_wave");
   }
@@ -1363,7 +1390,9 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (nb > 0x7fffffff) return arg_error("conv grid too large");
   const unsigned grid = (unsigned)nb;
   // algorithmic work of this launch: 2 * pixels * OC * (true channels * taps); padding not counted
-  KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s);
+  const ConvDesc desc(g, ep, "lds", wm * 10 + wn, gran, (long)nb);
+  KernelTimer timer("k_conv_igemm", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s, conv_bytes(g, ep),
+                    desc.text);
   const int ks = (wide && wm + wn < 4) ? 128 : 64;
   g.adv_c = ks % g.Cp;
   g.adv_tap = ks / g.Cp;
@@ -1379,6 +1408,12 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
 using namespace cvmhip;
 
 extern "C" {
+
+int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn) {
+  if (kernel < CONV_KERNEL_AUTO || kernel > CONV_KERNEL_WAVE) return arg_error("set_conv_tuning kernel");
+  set_conv_tuning(ConvTuning{kernel, wave_cfg, tile_wm, tile_wn});
+  return CVMHIP_OK;
+}
 
 size_t cvmhip_conv2d_workspace_bytes(int n, int ic, int h, int w, int oc, int kh, int kw, int groups) {
   if (groups != 1) return 0;

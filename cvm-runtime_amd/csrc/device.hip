@@ -21,18 +21,20 @@ using namespace cvmhip;
 namespace cvmhip {
 
 namespace {
-struct TimedLaunch { std::string name; double work; hipEvent_t e0, e1; };
+struct TimedLaunch { std::string name, desc; double work, bytes; hipEvent_t e0, e1; };
 bool g_timing = false;
 std::vector<TimedLaunch> g_launches;
 }  // namespace
 
 bool kernel_timing_enabled() { return g_timing; }
 
-void kernel_timing_mark(const char* name, double work, hipStream_t s, bool start) {
+void kernel_timing_mark(const char* name, double work, double bytes, const char* desc, hipStream_t s, bool start) {
   if (start) {
     TimedLaunch t;
     t.name = name;
+    t.desc = desc ? desc : "";
     t.work = work;
+    t.bytes = bytes;
     if (hipEventCreate(&t.e0) != hipSuccess || hipEventCreate(&t.e1) != hipSuccess) return;
     hipEventRecord(t.e0, s);
     g_launches.push_back(t);
@@ -166,12 +168,14 @@ int cvmhip_kernel_timing_begin(void) {
   return CVMHIP_OK;
 }
 
-// Writes {"kernel": {"launches": n, "ms": total, "work": total}, ...}
-int cvmhip_kernel_timing_end(char* json_out, int capacity) {
+// Writes {"kernel": {"launches": n, "ms": total, "work": total}, ...}; with per_launch a list, in launch
+// order, of {"kernel", "desc", "work", "bytes", "ms"}
+static int timing_end(char* json_out, int capacity, bool per_launch) {
   g_timing = false;
   HIP_TRY(hipDeviceSynchronize(), "kernel_timing_end");
   struct Acc { long n = 0; double ms = 0, work = 0; };
   std::map<std::string, Acc> acc;
+  std::string list = "[";
   for (TimedLaunch& t : g_launches) {
     float ms = 0;
     if (hipEventElapsedTime(&ms, t.e0, t.e1) == hipSuccess) {
@@ -179,10 +183,17 @@ int cvmhip_kernel_timing_end(char* json_out, int capacity) {
       a.n += 1;
       a.ms += ms;
       a.work += t.work;
+      if (per_launch) {
+        char buf[512];
+        snprintf(buf, sizeof(buf), "%s{\"kernel\": \"%s\", \"desc\": \"%s\", \"work\": %.6e, \"bytes\": %.6e, \"ms\": %.6f}",
+                 list.size() > 1 ? ", " : "", t.name.c_str(), t.desc.c_str(), t.work, t.bytes, ms);
+        list += buf;
+      }
     }
     hipEventDestroy(t.e0);
     hipEventDestroy(t.e1);
   }
+  list += "]";
   g_launches.clear();
   std::string out = "{";
   bool first = true;
@@ -194,10 +205,15 @@ int cvmhip_kernel_timing_end(char* json_out, int capacity) {
     first = false;
   }
   out += "}";
-  if (!json_out || (int)out.size() >= capacity) return arg_error("kernel_timing_end buffer");
-  memcpy(json_out, out.c_str(), out.size() + 1);
+  const std::string& res = per_launch ? list : out;
+  if (!json_out || (int)res.size() >= capacity) return arg_error("kernel_timing_end buffer");
+  memcpy(json_out, res.c_str(), res.size() + 1);
   return CVMHIP_OK;
 }
+
+int cvmhip_kernel_timing_end(char* json_out, int capacity) { return timing_end(json_out, capacity, false); }
+
+int cvmhip_kernel_timing_end_launches(char* json_out, int capacity) { return timing_end(json_out, capacity, true); }
 
 int cvmhip_event_create(void** event) {
   if (!event) return arg_error("event_create");

@@ -35,18 +35,20 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 // launches bracketed by KernelTimer record a HIP event pair on the launch
 // stream; totals per kernel name are read back when timing ends.
 bool kernel_timing_enabled();
-void kernel_timing_mark(const char* name, double work, hipStream_t s, bool start);
+void kernel_timing_mark(const char* name, double work, double bytes, const char* desc, hipStream_t s, bool start);
 
 struct KernelTimer {
   const char* name;
   hipStream_t s;
   bool on;
-  // `work` = algorithmic operations (or bytes) of this launch
-  KernelTimer(const char* n, double work, hipStream_t st) : name(n), s(st), on(kernel_timing_enabled()) {
-    if (on) kernel_timing_mark(name, work, s, true);
+  // `work` = algorithmic operations (or bytes) of this launch; `bytes` = algorithmic HBM bytes where the
+  // work is counted in operations; `desc` = what the launch is (layer shape, kernel configuration)
+  KernelTimer(const char* n, double work, hipStream_t st, double bytes = 0, const char* desc = nullptr)
+      : name(n), s(st), on(kernel_timing_enabled()) {
+    if (on) kernel_timing_mark(name, work, bytes, desc, s, true);
   }
   ~KernelTimer() {
-    if (on) kernel_timing_mark(name, 0, s, false);
+    if (on) kernel_timing_mark(name, 0, 0, nullptr, s, false);
   }
 };
 

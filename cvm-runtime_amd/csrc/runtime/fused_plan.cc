@@ -303,8 +303,7 @@ void HipGraphRuntime::BuildPlan() {
   };
 
   // test and tuning hook: CVM_HIP_DW=valu keeps depthwise layers on the vector kernel
-  const char* dw_env = std::getenv("CVM_HIP_DW");
-  const bool dw_on_mfma = !(dw_env && dw_env[0] == 'v');
+  const bool dw_on_mfma = hooks_.dw_on_mfma;
   for (uint32_t nid = 0; nid < nodes_.size(); ++nid) {
     const Node& n = nodes_[nid];
     if (n.is_variable()) {

@@ -420,6 +420,7 @@ void HipGraphRuntime::SetupOpExecs() {
 
 HipGraphRuntime::HipGraphRuntime(const std::string& graph_json, int device_id, bool with_device)
     : device_id_(device_id), with_device_(with_device) {
+  ReadHooks();
   Load(Json::Parse(graph_json));
   PrepareGraph();
   SetupShape();
@@ -437,6 +438,20 @@ HipGraphRuntime::HipGraphRuntime(const std::string& graph_json, int device_id, b
   } catch (...) {
     Release();
     throw;
+  }
+}
+
+void HipGraphRuntime::ReadHooks() {
+  auto env = [](const char* name) { const char* v = std::getenv(name); return std::string(v ? v : ""); };
+  hooks_.fuse = env("CVM_HIP_FUSE") != "0";
+  hooks_.graph = env("CVM_HIP_GRAPH") != "0";
+  hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
+  const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
+  hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : 0;
+  if (!cfg.empty() && cfg[0] >= '0' && cfg[0] <= '9') hooks_.wave_cfg = std::atoi(cfg.c_str());
+  if (tile.size() >= 3 && tile[1] == ',') {
+    hooks_.tile_wm = tile[0] - '0';
+    hooks_.tile_wn = tile[2] - '0';
   }
 }
 
@@ -628,14 +643,15 @@ void HipGraphRuntime::LoadParams(const std::string& blob) {
   }
   for (Exec& ex : execs_)
     if (ex.kernel->prepare) ex.kernel->prepare(ex.call);
-  const char* fuse = std::getenv("CVM_HIP_FUSE");
-  if (fuse == nullptr || std::string(fuse) != "0") BuildPlan();
+  if (hooks_.fuse) BuildPlan();
   HipCheck(cvmhip_stream_sync(stream_), "prepare operators");
   params_loaded_ = true;
 }
 
 // ---------------------------------------------------------------- execution
 void HipGraphRuntime::Launch() {
+  // the kernel choice this model was loaded with, for the launches of this thread
+  HipCheck(cvmhip_set_conv_tuning(hooks_.conv_kernel, hooks_.wave_cfg, hooks_.tile_wm, hooks_.tile_wn), "conv tuning");
   if (fused_) {
     for (PlanStep& st : plan_) RunStep(st);
   } else {
@@ -649,10 +665,7 @@ void HipGraphRuntime::Launch() {
 // needs the eager path (its event pairs must not end up inside a graph);
 // CVM_HIP_GRAPH=0 keeps it for good.
 void HipGraphRuntime::Run() {
-  if (graph_state_ == 0) {
-    const char* env = std::getenv("CVM_HIP_GRAPH");
-    graph_state_ = (env && std::string(env) == "0") ? -1 : 1;
-  }
+  if (graph_state_ == 0) graph_state_ = hooks_.graph ? 1 : -1;
   if (graph_state_ < 0 || cvmhip_kernel_timing_active()) {
     Launch();
     return;

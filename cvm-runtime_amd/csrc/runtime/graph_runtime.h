@@ -194,6 +194,17 @@ class HipGraphRuntime {
   void* graph_exec_ = nullptr;
   int graph_state_ = 0;  // 0 undecided, -1 eager for good, 1 before the first run, 2 ready to capture, 3 captured
 
+  // Test and tuning hooks, read from the environment once, when the model is constructed (never on the
+  // launch path): CVM_HIP_FUSE=0 no load-time fusion, CVM_HIP_GRAPH=0 no graph replay, CVM_HIP_DW=valu
+  // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
+  // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
+  struct Hooks {
+    bool fuse = true, graph = true, dw_on_mfma = true;
+    int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
+  };
+  Hooks hooks_;
+  void ReadHooks();
+
   // ---- fused executor: int8 NHWC activations + folded requantisation chains
   void BuildPlan();
   void RunStep(PlanStep& st);

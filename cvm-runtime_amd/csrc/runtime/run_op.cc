@@ -104,6 +104,7 @@ extern "C" int CVMHIPRunOp(const char* op, const char* attr_json, int n_in, cons
       CVM_CHECK(out_data[i] && out_capacity[i] >= cvmrt::shape_size(out[i]))
           << "output " << i << " needs " << cvmrt::shape_size(out[i]) << " elements";
     cvmrt::RegisterHipKernels();
+    cvmhip_set_conv_tuning(0, -1, 0, 0);   // automatic kernel choice, whatever this thread forced before
     const std::string fname = std::string("cvm.runtime.hip.") + op;
     const cvmrt::OpKernel* kernel = cvmrt::OpRegistry::Global().Get(fname);
     CVM_VERIFY(kernel != nullptr) << "function undefined " << fname;

@@ -6,6 +6,7 @@ reference's operators (`cvm.runtime.<dev>.<op>`, src/runtime/cpu/ops), so a
 parity test reads like the reference's tests/test_op.cc cases.
 """
 import ctypes
+import os
 
 import torch
 
@@ -25,7 +26,18 @@ def _ptr(t):
     return ctypes.cast(t.data_ptr(), _i32p)
 
 
+def _apply_conv_tuning():
+    """The library never reads the environment on a launch; this glue turns the test hooks CVM_HIP_CONV
+    (lds | wave), CVM_HIP_WAVECFG (index) and CVM_HIP_TILE ("wm,wn") into the explicit per-thread setting."""
+    kind = os.environ.get("CVM_HIP_CONV", "")
+    cfg = os.environ.get("CVM_HIP_WAVECFG", "")
+    tile = os.environ.get("CVM_HIP_TILE", "")
+    wm, wn = (int(tile[0]), int(tile[2])) if len(tile) >= 3 and tile[1] == "," else (0, 0)
+    check(lib().cvmhip_set_conv_tuning({"l": 1, "w": 2}.get(kind[:1], 0), int(cfg) if cfg.isdigit() else -1, wm, wn))
+
+
 def _stream():
+    _apply_conv_tuning()
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

@@ -196,6 +196,9 @@ int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms);
  * where work is the algorithmic operation (or byte) count of the launches. */
 int cvmhip_kernel_timing_begin(void);
 int cvmhip_kernel_timing_end(char* json_out, int capacity);
+/* The same end call, but the text is a list with one entry per bracketed launch, in launch order:
+ * [{"kernel", "desc" (layer shape and kernel configuration), "work", "bytes" (algorithmic HBM bytes), "ms"}] */
+int cvmhip_kernel_timing_end_launches(char* json_out, int capacity);
 int cvmhip_kernel_timing_active(void);   /* 1 between begin and end */
 
 /* ---- stream capture: the launches issued on `stream` between begin and end
@@ -248,6 +251,10 @@ typedef struct {
 } cvmhip_chain;
 
 int cvmhip_pad_channels(int channels);
+/* Test and tuning hook: forces, for the calling thread's later convolution launches, the implicit-GEMM kernel
+ * (0 automatic, 1 LDS-tiled, 2 wavefront-private), a configuration of the wavefront kernel (-1 automatic) and a
+ * tile of the tiled kernel (wm, wn in 1..2; 0 automatic).  The library never reads the environment on a launch. */
+int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn);
 /* int32 NCHW <-> int8 act layout (narrowing is static_cast<int8_t>) */
 int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream);
 int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void* stream);

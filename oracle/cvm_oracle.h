@@ -8,8 +8,8 @@
  * arrays of length ndim (ndim <= 6).  All functions return 0 on success, a
  * positive code on rejected arguments.
  *
- * Pinned against the compiled reference (oracle/_ref) by tests/test_oracle_vs_ref.py
- * and against closed forms / brute force by tests/test_oracle_math.py.
+ * Pinned by tests/test_oracle.py: against the compiled reference (oracle/_ref) where it is built, against the
+ * golden outputs it wrote (tests/golden/), and against closed forms / brute force.
  */
 #ifndef CVM_ORACLE_H_
 #define CVM_ORACLE_H_
