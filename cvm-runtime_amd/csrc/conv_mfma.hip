@@ -137,7 +137,11 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
       // the block exists (all 32 pixel rows of it are allocated) unless it lies past the tensor
       const bool tile_ok = (px_wave + gj * 32) < P && (oc0 + chb) < ocp;
       const int64_t off = ((int64_t)((px_wave >> 5) + gj) * (ocp >> 5) + ((oc0 + chb) >> 5)) * 1024;
-      const int4 r4 = tile_ok ? *reinterpret_cast<const int4*>(ep.residual + off + lane * 16) : zero4();
+      int4 r4 = zero4();
+      if (tile_ok) {
+        const v4i t4 = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(ep.residual + off + lane * 16));
+        r4 = make_int4(t4[0], t4[1], t4[2], t4[3]);
+      }
       rp[t * 4] = r4.x; rp[t * 4 + 1] = r4.y; rp[t * 4 + 2] = r4.z; rp[t * 4 + 3] = r4.w;
     }
   } else {
@@ -229,7 +233,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int first = tile_first + lgrp * 16;
       if (tile_first + 32 > g.OC) mask_channels(w, first, g.OC);          // only the last tile of a ragged channel count
       const int p = px_wave + gj[t * 4] * 32 + lrow;
-      if (p < P && first < ocp) *reinterpret_cast<int4*>(y8 + block_off(t * 4) + lane * 16) = make_int4(w[0], w[1], w[2], w[3]);
+      if (p < P && first < ocp) {
+        const v4i pk4 = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16));
+      }
     }
   } else if (halves) {
     uint32_t a = pk[0], b = pk[1];
@@ -739,14 +746,21 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   int bias_mine = 0;
   if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
 
-  regs_t R1 = fetch();
-  consume(R0, true);
-  for (int it = 1; it < niter; it += 2) {
-    R0 = fetch();
-    consume(R1, false);
-    if (it + 1 >= niter) break;
-    R1 = fetch();
-    consume(R0, false);
+  if (niter <= 1) {
+    // the whole K range is one batch (a 1x1 layer over 64 channels): no second request.  Every byte a
+    // wavefront asks for, used or not, takes its turn in the CU's memory pipeline, and these layers are
+    // bound by exactly that.
+    consume(R0, true);
+  } else {
+    regs_t R1 = fetch();
+    consume(R0, true);
+    for (int it = 1; it < niter; it += 2) {
+      R0 = fetch();
+      consume(R1, false);
+      if (it + 1 >= niter) break;
+      R1 = fetch();
+      consume(R0, false);
+    }
   }
   if (tid < BM) sBias[tid] = bias_mine;
 
