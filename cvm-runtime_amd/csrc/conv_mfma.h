@@ -53,6 +53,7 @@ struct ConvGeom {
                            //    filter packed by pack_depthwise_diag (OC == C, Cp % 32 == 0)
   int octiles;             // filled by conv_igemm for the wavefront kernel: channel tiles of the grid, and division by it
   FastDiv div_octiles;
+  int p_begin, p_end;      // layer-sequence kernel only: the output pixels [p_begin, p_end) this share of the layer covers
 };
 
 // What happens to an accumulator before it is stored:

@@ -110,6 +110,20 @@ __device__ __forceinline__ void mask_channels(uint32_t (&d)[N], int first, int O
   }
 }
 
+// 16 bytes per lane from a tensor that another workgroup of this kernel may have written (COH): the request
+// carries device scope, so it is answered by the L2 (the point where the compute units of one XCD meet)
+// and never by a line the CU's own L1 kept from an earlier layer.  An offset with its top bit set lies
+// outside every buffer (sizes stay below 2^31) and reads as zeros.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+constexpr unsigned kOutsideBuffer = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t act_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ int4 ld16_l2(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 16 /* sc1: device scope */);
+  return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
+}
+
 // Epilogue shared by both kernels.  A wavefront holds NG groups of 4 values; group
 // u (counted from u0, which is a multiple of NG) belongs to the 32x32 MFMA tile
 // t = u / 4 of the wavefront's TM x TN tiles (t = i * TN + j) and is the 4
@@ -122,7 +136,7 @@ __device__ __forceinline__ void mask_channels(uint32_t (&d)[N], int first, int O
 // they lie in memory: for whole tiles the 16 bytes per lane of each tile's KiB block, otherwise the 4
 // bytes of each group.  Separate from finish_groups so that a kernel can issue these loads before its
 // K loop and find them in registers when the accumulators are ready.
-template <int TN, int NG>
+template <int TN, int NG, bool COH = false>
 __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch_wave, int oc0, int px_wave, int lane,
                                               const ConvGeom& g, const Epilogue& ep) {
   const int lrow = lane & 31, lgrp = lane >> 5;
@@ -138,7 +152,9 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
       const bool tile_ok = (px_wave + gj * 32) < P && (oc0 + chb) < ocp;
       const int64_t off = ((int64_t)((px_wave >> 5) + gj) * (ocp >> 5) + ((oc0 + chb) >> 5)) * 1024;
       int4 r4 = zero4();
-      if (tile_ok) {
+      if constexpr (COH) {
+        r4 = ld16_l2(act_rsrc(ep.residual), tile_ok ? (unsigned)off + (unsigned)lane * 16u : kOutsideBuffer);
+      } else if (tile_ok) {
         const v4i t4 = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(ep.residual + off + lane * 16));
         r4 = make_int4(t4[0], t4[1], t4[2], t4[3]);
       }
@@ -150,17 +166,22 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
       const int u = u0 + m, t = u >> 2;
       const int p = px_wave + (t % TN) * 32 + lrow;
       const int oc = oc0 + ch_wave + (t / TN) * 32 + (u & 3) * 8 + lgrp * 4;
-      rp[m] = *reinterpret_cast<const uint32_t*>(ep.residual + act_offset(p < P ? p : 0, oc < ocp ? oc : 0, ocp));
+      const int64_t roff = act_offset(p < P ? p : 0, oc < ocp ? oc : 0, ocp);
+      if constexpr (COH) rp[m] = __builtin_amdgcn_raw_buffer_load_b32(act_rsrc(ep.residual), (int)roff, 0, 16);
+      else rp[m] = *reinterpret_cast<const uint32_t*>(ep.residual + roff);
     }
   }
 }
 
-template <int TN, int NG, int OUT>
+// RANGE: only the pixels [g.p_begin, g.p_end) are stored (one share of a layer inside the layer-sequence
+// kernel); the stores are then ordinary ones, because the next layer reads the tensor from this L2.
+template <int TN, int NG, int OUT, bool RANGE = false>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
                                               int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
                                               uint32_t (&rp)[NG]) {
   const int lrow = lane & 31, lgrp = lane >> 5;
-  const int P = (int)g.P;
+  const int P = RANGE ? g.p_end : (int)g.P;
+  const int Plo = RANGE ? g.p_begin : 0;
   const int ocp = ep.out_cp;
   const bool blocked = act_blocked(ocp);
   // group m: tile (gi, gj), channel quarter gq; ch = first channel inside the workgroup's BM channels
@@ -207,7 +228,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
 #pragma unroll
     for (int m = 0; m < NG; ++m) {
       const int p = px_wave + gj[m] * 32 + lrow;
-      if (p >= P) continue;
+      if (p >= P || p < Plo) continue;
       const int n = (int)fastdiv((unsigned)p, g.div_ohw);
       const int rem = p - n * OHW;
       const int oc = oc0 + ch[m];
@@ -233,9 +254,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int first = tile_first + lgrp * 16;
       if (tile_first + 32 > g.OC) mask_channels(w, first, g.OC);          // only the last tile of a ragged channel count
       const int p = px_wave + gj[t * 4] * 32 + lrow;
-      if (p < P && first < ocp) {
+      if (p < P && p >= Plo && first < ocp) {
         const v4i pk4 = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-        __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16));
+        if constexpr (RANGE) *reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16) = pk4;
+        else __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16));
       }
     }
   } else if (halves) {
@@ -245,7 +267,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     const int first = oc0 + ch[0] - lgrp * 4 + lgrp * 8;
     mask_channels(w, first, g.OC);
     const int p = px_wave + gj[0] * 32 + lrow;
-    if (p < P && first < ocp) *reinterpret_cast<uint2*>(y8 + act_offset(p, first, ocp)) = make_uint2(w[0], w[1]);
+    if (p < P && p >= Plo && first < ocp) *reinterpret_cast<uint2*>(y8 + act_offset(p, first, ocp)) = make_uint2(w[0], w[1]);
   } else {
 #pragma unroll
     for (int m = 0; m < NG; ++m) {
@@ -253,7 +275,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int first = oc0 + ch[m];
       mask_channels(w, first, g.OC);
       const int p = px_wave + gj[m] * 32 + lrow;
-      if (p < P && first < ocp) *reinterpret_cast<uint32_t*>(y8 + act_offset(p, first, ocp)) = w[0];
+      if (p < P && p >= Plo && first < ocp) *reinterpret_cast<uint32_t*>(y8 + act_offset(p, first, ocp)) = w[0];
     }
   }
 }
@@ -503,10 +525,14 @@ __device__ __forceinline__ unsigned tap_mask_dilated(int x0, int extent, int k, 
 //                    out-of-image granules are read from a zero granule
 enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 
-template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
-__global__ void __launch_bounds__(NW * 64, MINW)
-k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
-            const ConvGeom g, const Epilogue ep) {
+// One tile set of the wavefront-private kernel: workgroup-level tile `pid` (channel tile fastest) of the
+// pixel range [g.p_begin, g.p_end), computed by the NW wavefronts whose thread index is `tid`, with
+// sPart / sBias their LDS.  k_conv_wave is this function over a grid; the layer-sequence kernel calls it
+// from its loop over layers with COH set (operands written earlier in the same launch).
+template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH>
+__device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
+                                               const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
+                                               int* __restrict__ sPart, int* __restrict__ sBias) {
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
   constexpr int BM = 32 * TM;             // output channels per workgroup
   constexpr int WPIX = 32 * TN;           // pixels per wavefront
@@ -514,10 +540,8 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   constexpr int U = TM * TN * 4;          // groups of 4 accumulator registers (4 consecutive channels) per wavefront
   constexpr int NU = U / KSPLIT;          // groups one wavefront finalises
   static_assert(NW % KSPLIT == 0 && U % KSPLIT == 0, "split must divide the work");
-  __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
-  __shared__ __attribute__((aligned(16))) int sBias[BM];
+  static_assert(!(COH && (MODE == WAVE_ROWS || SLICES)), "the layer-sequence kernel has no row-window or K-sliced form");
 
-  const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kw_ = wave % KSPLIT, pw_ = wave / KSPLIT;
@@ -532,9 +556,6 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int X = G >> 2, Q = G & 3;
   const int Xi = X / TN, Xj = X % TN;
 
-  int pid = blockIdx.x;
-  const int nb = gridDim.x;
-  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
   // K sliced over the grid (g.kslices > 1: a layer with very few tiles and a very long K, whose filter stream
   // needs more workgroups than it has tiles): slice index = low bits of the block index (the slices of a tile then share its activation operand in one L2); a slice writes
   // raw int32 partial sums to its own plane of the workspace and a second kernel adds the planes up.
@@ -546,13 +567,15 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   }
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);   // g.octiles = ceil(OC / BM), set by the host for this tile
   const int oc0 = (pid - ptile * g.octiles) * BM;
-  const int px0 = ptile * BN;              // P < 2^31 is checked on the host
+  const int px0 = (COH ? (g.p_begin & ~31) : 0) + ptile * BN;   // P < 2^31 is checked on the host
   const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
   const int P = (int)g.P;
+  __amdgpu_buffer_rsrc_t rs_x = act_rsrc(xp);   // only used by the COH form
 
   // ---- per-lane operand addressing
   const int8_t* xb[TN];                    // WAVE_IDENT: block base + lane * 16
+  unsigned xoff[TN];                       //   ... the same as a byte offset from xp (COH)
   int rowbase[TN];                         // otherwise: linear index of the first input pixel of the receptive field
   unsigned rowmask[TN], colmask[TN];       // WAVE_PAD: filter rows / columns inside the image
 #pragma unroll
@@ -562,10 +585,11 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       const int last = (P - 1) >> 5;
       t = t < last ? t : last;             // blocks past the tensor re-read its last block; their pixels are never stored
       xb[j] = xp + (int64_t)t * ctiles * 1024 + lane * 16;
+      xoff[j] = (unsigned)t * (unsigned)(ctiles * 1024) + (unsigned)lane * 16u;
       rowbase[j] = 0; rowmask[j] = 0; colmask[j] = 0;
     } else {
       const int p = px0 + (pw_ * TN + (j ^ Xj)) * 32 + lrow;
-      const bool ok = p < P;
+      const bool ok = COH ? (p >= g.p_begin && p < g.p_end) : p < P;
       const unsigned pp = ok ? (unsigned)p : 0u;
       const int n = (int)fastdiv(pp, g.div_ohw);
       const int rem = (int)pp - n * OHW;
@@ -575,6 +599,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
       rowbase[j] = (n * g.H + ih0) * g.W + iw0;
       if (MODE == WAVE_ROWS) rowbase[j] *= 4;   // byte offset of the window of filter row 0 (g.H, g.W: stored size, no padding left)
       xb[j] = xp;
+      xoff[j] = 0;
       unsigned rm = 0, cm = 0;
       if (MODE == WAVE_PAD) {
         if (g.DH == 1 && g.DW == 1) {
@@ -620,10 +645,11 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   const int lconst = lgrp * 512;
   const int8_t* tapptr[TN];                // per-lane operand address of the current filter tap
+  unsigned tapoff[TN];                     //   ... as a byte offset from xp, kOutsideBuffer for a tap outside the image (COH)
   int okv[TN];                             // 0: the lane reads the zero granule for this tap
   bool need_tap = true;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) { tapptr[j] = zero; okv[j] = 0; }
+  for (int j = 0; j < TN; ++j) { tapptr[j] = zero; tapoff[j] = kOutsideBuffer; okv[j] = 0; }
 
   v16i acc[TM][TN];   // first written by the first MFMA of each tile, whose addend is the constant 0
 
@@ -654,7 +680,10 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb[d] * 1024));
+        for (int d = 0; d < D; ++d) {
+          if constexpr (COH) put(R, (d * (TM + TN) + TM + j) * 4, ld16_l2(rs_x, xoff[j] + (unsigned)cb[d] * 1024u));
+          else put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb[d] * 1024));
+        }
       cur = cur + D < c_end ? cur + D : c_end;
       return R;
     }
@@ -688,14 +717,17 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
             const unsigned off = __umul24((unsigned)pin >> 5, (unsigned)g.Cp << 5) + (((unsigned)pin & 31u) << 4) + (unsigned)lconst;
             const int8_t* inside = xp + off;
             tapptr[j] = ok ? inside : zero;
+            tapoff[j] = ok ? off : kOutsideBuffer;
             okv[j] = ok ? 1 : 0;
           }
           need_tap = false;
         }
         const int coff = live ? ((ch + ch_first) >> 5) * 1024 : 0;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(tapptr[j] + (okv[j] ? coff : 0)));
+        for (int j = 0; j < TN; ++j) {
+          if constexpr (COH) put(R, (d * (TM + TN) + TM + j) * 4, ld16_l2(rs_x, tapoff[j] + (unsigned)coff));
+          else put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(tapptr[j] + (okv[j] ? coff : 0)));
+        }
       }
       if (live) {
         ++cur;
@@ -741,7 +773,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   // register and staged in LDS after the loop (staging it here would put a full memory latency in
   // front of the first operand request).
   uint32_t rp[NU];
-  if (ep.residual) load_residual<TN, NU>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+  if (ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
   regs_t R0 = fetch();
   int bias_mine = 0;
   if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
@@ -801,7 +833,20 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   }
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp);
+  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp);
+}
+
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
+__global__ void __launch_bounds__(NW * 64, MINW)
+k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
+            const ConvGeom g, const Epilogue ep) {
+  constexpr int U = TM * TN * 4;
+  __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
+  __shared__ __attribute__((aligned(16))) int sBias[32 * TM];
+  int pid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
+  conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
 }
 
 // Second step of a K-sliced convolution: out = chain(sum over slices + bias), stored like the epilogue would
