@@ -53,7 +53,6 @@ struct ConvGeom {
                            //    filter packed by pack_depthwise_diag (OC == C, Cp % 32 == 0)
   int octiles;             // filled by conv_igemm for the wavefront kernel: channel tiles of the grid, and division by it
   FastDiv div_octiles;
-  int p_begin, p_end;      // layer-sequence kernel only: the output pixels [p_begin, p_end) this share of the layer covers
 };
 
 // What happens to an accumulator before it is stored:
@@ -147,6 +146,18 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
 size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep);
 int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, void* ws, size_t ws_bytes,
                   hipStream_t s);
+
+// ---- a run of convolutions in one launch (k_conv_seq), for batches that are a multiple of 8: every XCD computes all
+// layers for its share of the images and layer boundaries are counters in that XCD's L2.  The caller builds a host
+// table with conv_seq_layer (one entry per convolution, in order; each must only read tensors that earlier entries
+// or earlier launches wrote), copies it to the device and launches it; `sync` is conv_seq_sync_bytes() of zeroed
+// device memory, 256-byte aligned, whose last block holds an error flag (non-zero: a wait ran out, results invalid).
+// Two sequence launches must never be in flight at once on one device (each needs every compute unit).
+size_t conv_seq_layer_bytes();
+size_t conv_seq_sync_bytes();
+int conv_seq_shares();
+int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep);
+int conv_seq_launch(const void* dev_table, int nlayers, void* sync, hipStream_t s);
 
 }  // namespace cvmhip
 #endif

@@ -23,6 +23,7 @@
 //                 K and meet in LDS once.  Serves layers whose grid is too small
 //                 to hide the per-step latency of the tiled kernel.
 #include <stdlib.h>
+#include <string.h>
 
 #include <type_traits>
 
@@ -173,15 +174,15 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
   }
 }
 
-// RANGE: only the pixels [g.p_begin, g.p_end) are stored (one share of a layer inside the layer-sequence
+// RANGE: only the pixels [p_begin, p_end) are stored (one share of a layer inside the layer-sequence
 // kernel); the stores are then ordinary ones, because the next layer reads the tensor from this L2.
 template <int TN, int NG, int OUT, bool RANGE = false>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
                                               int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
-                                              uint32_t (&rp)[NG]) {
+                                              uint32_t (&rp)[NG], int p_begin = 0, int p_end = 0) {
   const int lrow = lane & 31, lgrp = lane >> 5;
-  const int P = RANGE ? g.p_end : (int)g.P;
-  const int Plo = RANGE ? g.p_begin : 0;
+  const int P = RANGE ? p_end : (int)g.P;
+  const int Plo = RANGE ? p_begin : 0;
   const int ocp = ep.out_cp;
   const bool blocked = act_blocked(ocp);
   // group m: tile (gi, gj), channel quarter gq; ch = first channel inside the workgroup's BM channels
@@ -526,13 +527,14 @@ __device__ __forceinline__ unsigned tap_mask_dilated(int x0, int extent, int k, 
 enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 
 // One tile set of the wavefront-private kernel: workgroup-level tile `pid` (channel tile fastest) of the
-// pixel range [g.p_begin, g.p_end), computed by the NW wavefronts whose thread index is `tid`, with
+// pixel range [p_begin, p_end) (COH only; otherwise the whole layer), computed by the NW wavefronts whose thread index is `tid`, with
 // sPart / sBias their LDS.  k_conv_wave is this function over a grid; the layer-sequence kernel calls it
 // from its loop over layers with COH set (operands written earlier in the same launch).
 template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
-                                               int* __restrict__ sPart, int* __restrict__ sBias) {
+                                               int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
+                                               const int p_end = 0) {
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
   constexpr int BM = 32 * TM;             // output channels per workgroup
   constexpr int WPIX = 32 * TN;           // pixels per wavefront
@@ -567,7 +569,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   }
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);   // g.octiles = ceil(OC / BM), set by the host for this tile
   const int oc0 = (pid - ptile * g.octiles) * BM;
-  const int px0 = (COH ? (g.p_begin & ~31) : 0) + ptile * BN;   // P < 2^31 is checked on the host
+  const int px0 = (COH ? (p_begin & ~31) : 0) + ptile * BN;   // P < 2^31 is checked on the host
   const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
   const int P = (int)g.P;
@@ -589,7 +591,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       rowbase[j] = 0; rowmask[j] = 0; colmask[j] = 0;
     } else {
       const int p = px0 + (pw_ * TN + (j ^ Xj)) * 32 + lrow;
-      const bool ok = COH ? (p >= g.p_begin && p < g.p_end) : p < P;
+      const bool ok = COH ? (p >= p_begin && p < p_end) : p < P;
       const unsigned pp = ok ? (unsigned)p : 0u;
       const int n = (int)fastdiv(pp, g.div_ohw);
       const int rem = (int)pp - n * OHW;
@@ -833,7 +835,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   }
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp);
+  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
 }
 
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
@@ -847,6 +849,139 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
   conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
+}
+
+// ---------------------------------------------------------------- layer-sequence kernel
+// A run of convolutions of one graph in ONE launch, for batches that divide over the chip's 8 XCDs.
+// Images are independent, so XCD x computes every layer for its own share of the images (pixel range
+// [x * px_per_share, (x + 1) * px_per_share) of every tensor) and never reads what another XCD wrote.  The
+// 32 compute units of an XCD share one L2, which makes a layer boundary cheap and local:
+//   * a producer's ordinary stores are in the L2 once its wavefronts have waited for them (vmcnt);
+//   * the consumers read activations and residuals with device-scope loads (ld16_l2), which the L2 answers;
+//   * the boundary itself is one counter per XCD in that L2 (an atomic add per workgroup, then polling) --
+//     no L2 write-back or invalidation, which is what makes a kernel boundary or an agent-scope
+//     release cost microseconds; the dirty lines leave the L2 when the kernel ends, as after any kernel.
+// One workgroup of 8 wavefronts per compute unit (grid = 256); it learns its XCD from the hardware
+// register, its rank among the workgroups of that XCD from the order of arrival, and walks the tiles
+// rank, rank + 32, ... of every layer (configurations of 4 wavefronts run two tiles side by side).
+// Every wait is bounded: when a counter does not arrive within spin_limit polls the workgroup raises
+// the error flag, which makes every workgroup leave at its next boundary; the host then falls back to one
+// launch per layer.
+struct SeqLayer {
+  const int8_t* xp;
+  const int8_t* wf;
+  void* out;
+  ConvGeom g;
+  Epilogue ep;
+  int kernel;          // configuration * 3 + mode (identity, no padding, padding)
+  int px_per_share;    // output pixels of one share of the images
+  int ptiles;          // pixel tiles that cover a share (its first block may begin before the share)
+  int reserved;
+};
+constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
+enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
+
+template <int TM, int TN, int KSPLIT, int NW, int D, int MODE>
+__device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
+                                                int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
+                                                int p_end) {
+  constexpr int UNITS = 8 / NW;   // tiles a workgroup computes side by side
+  const int half = UNITS == 2 ? (tid >> 8) : 0;
+  const int htid = UNITS == 2 ? (tid & 255) : tid;
+  for (int base = 0; base < ntiles; base += SEQ_WG_PER_SHARE * UNITS) {
+    const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
+    conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
+                                                                         sPart + half * 16384, sBias + half * 64, p_begin, p_end);
+    __syncthreads();   // the next tile reuses the LDS
+  }
+}
+
+template <int MODE>
+__device__ __forceinline__ void seq_layer_cfg(int cfg, const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
+                                              int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
+                                              int p_end) {
+  switch (cfg) {
+    case 0: seq_layer_tiles<2, 2, 8, 8, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 1: seq_layer_tiles<2, 2, 4, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 2: seq_layer_tiles<2, 2, 2, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 3: seq_layer_tiles<2, 2, 1, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 4: seq_layer_tiles<1, 2, 8, 8, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 5: seq_layer_tiles<1, 2, 4, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    default: seq_layer_tiles<1, 2, 1, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+  }
+}
+
+__global__ void __launch_bounds__(512, 1)
+k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit) {
+  __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: one 8-wavefront tile set or two 4-wavefront ones
+  __shared__ __attribute__((aligned(16))) int sBias[128];
+  __shared__ int s_rank, s_stop;
+  // The table never changes during the launch.  It is read through the constant address space, so that a field is
+  // a scalar load wherever it is needed, as a kernel argument would be (a copy in registers would hold ~100 scalar
+  // registers for the whole layer).
+  typedef const SeqLayer __attribute__((address_space(4))) * table_t;
+  const table_t table = (table_t)(uintptr_t)layers_generic;
+  const int tid = threadIdx.x;
+  unsigned xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  xcc &= 15u;
+  unsigned* my = sync + (xcc < SEQ_SHARES ? xcc : 0) * SEQ_SYNC_WORDS;
+  unsigned* error = sync + SEQ_SHARES * SEQ_SYNC_WORDS;
+  if (tid == 0) {
+    const unsigned r = __hip_atomic_fetch_add(my + SEQ_ARRIVE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (xcc >= SEQ_SHARES || r >= SEQ_WG_PER_SHARE) __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // not the chip this kernel is laid out for
+    s_rank = (int)r;
+    s_stop = 0;
+  }
+  __syncthreads();
+  const int rank = s_rank;
+  bool stop = xcc >= SEQ_SHARES || rank >= SEQ_WG_PER_SHARE;
+  for (int l = 0; l < nlayers && !stop; ++l) {
+    const SeqLayer& L = *(const SeqLayer*)(table + l);
+    const ConvGeom& g = L.g;
+    const Epilogue& ep = L.ep;
+    const int8_t* xp = L.xp;
+    const int8_t* wf = L.wf;
+    void* out = L.out;
+    const int kernel = L.kernel;
+    const int p_begin = (int)xcc * L.px_per_share;
+    const int p_end = p_begin + L.px_per_share;
+    const int ntiles = g.octiles * L.ptiles;
+    const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
+    const int cfg = kernel / 3, mode = kernel - cfg * 3;
+    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
+    else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
+    else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
+    if (l + 1 == nlayers) break;
+    // ---- layer boundary inside the XCD: every store of this wavefront is in the L2, then count and wait
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned target = (unsigned)(l + 1) * SEQ_WG_PER_SHARE;
+      int spins = 0, bad = 0;
+      while (__hip_atomic_load(my + SEQ_BAR, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (++spins > spin_limit || __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { bad = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (bad) {
+        __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_stop = 1;
+      }
+    }
+    __syncthreads();
+    stop = s_stop != 0;
+  }
+  // the last workgroup of a share to finish clears the share's counters for the next launch
+  __syncthreads();
+  if (tid == 0 && xcc < SEQ_SHARES) {
+    const unsigned d = __hip_atomic_fetch_add(my + SEQ_DONE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (d == SEQ_WG_PER_SHARE - 1) {
+      __hip_atomic_store(my + SEQ_ARRIVE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(my + SEQ_BAR, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(my + SEQ_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
 }
 
 // Second step of a K-sliced convolution: out = chain(sum over slices + bias), stored like the epilogue would
@@ -1252,22 +1387,23 @@ static int64_t wave_cfg_blocks(const WaveCfg& c, const ConvGeom& g) {
 // wavefront as possible: the deepest K split (at least two chunks per wavefront)
 // of the largest tile whose grid is resident at once.  Larger grids run unsplit
 // in several rounds (the wavefronts of a workgroup then share the filter through L1).
-static int choose_wave_cfg(const ConvGeom& g) {
+// `cus`: compute units the layer runs on (the chip, or one XCD for a share of a layer-sequence launch; g.P is then the share's)
+static int choose_wave_cfg(const ConvGeom& g, int cus = 256) {
   const int nlive = g.K / 32;
   // very few pixels, deep K (fully connected layers, the last stage): even the deepest split of
   // the 64-channel tile leaves SIMDs without a wavefront, so halve the tile instead
-  if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < 128) return 4;
+  if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < cus / 2) return 4;
   const int first = g.OC > 32 ? 0 : 4;
   const int last = g.OC > 32 ? 4 : 7;   // 64-channel tiles: 0..3 (and 7, see below); 32-channel tiles: 4..6
   for (int i = first; i < last; ++i) {
     const WaveCfg& c = kWaveCfgs[i];
     if (c.ksplit > 1 && nlive < 2 * c.ksplit) continue;
-    const int64_t capacity = 256 * (int64_t)c.blocks_per_cu;
+    const int64_t capacity = cus * (int64_t)c.blocks_per_cu;
     if (c.ksplit == 1 || wave_cfg_blocks(c, g) <= capacity) {
       // Unsplit with a grid of many rounds and a long K loop (the large layers of a VGG): the K loop is bound by
       // operand delivery, and a 64 x 128 wavefront tile takes 0.75 KiB per MFMA instead of 1 KiB (measured
       // 1.0 -> 1.2-1.3 POP/s on 28x28x512 and 56x56x256 layers with 3x3 filters).
-      if (c.ksplit == 1 && g.OC > 32 && g.K >= 512 && wave_cfg_blocks(kWaveCfgs[7], g) >= 192) return 7;
+      if (cus == 256 && c.ksplit == 1 && g.OC > 32 && g.K >= 512 && wave_cfg_blocks(kWaveCfgs[7], g) >= 192) return 7;
       return i;
     }
   }
@@ -1330,8 +1466,8 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
   return conv_igemm_ws(xp, wp, out, g, ep_in, nullptr, 0, s);
 }
 
-int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, void* ws, size_t ws_bytes,
-                  hipStream_t s) {
+// Checks a convolution's geometry and fills the derived fields of g and the defaults of the epilogue.
+static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom& g, const Epilogue& ep_in, Epilogue& ep) {
   const Epilogue& ep0 = ep_in;
   if (g.N < 1 || g.H < 1 || g.W < 1 || g.OC < 1 || g.OH < 1 || g.OW < 1 || g.KH < 1 || g.KW < 1 || g.SH < 1 ||
       g.SW < 1 || g.DH < 1 || g.DW < 1 || g.PH < 0 || g.PW < 0)
@@ -1351,7 +1487,7 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
   if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
-  Epilogue ep = ep_in;
+  ep = ep_in;
   ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
   if (ep.o32_img == 0 && ep.o32_ch == 0 && ep.o32_px == 0) {  // int32 output defaults to NCHW
     ep.o32_img = (int64_t)g.OC * g.OH * g.OW;
@@ -1360,6 +1496,18 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   } else if (ep.o32_ch < 1 || ep.o32_px < 1 || ep.o32_img < 0) {
     return arg_error("conv int32 output strides");
   }
+  g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
+  g.div_ow = make_fastdiv((uint32_t)g.OW);
+  g.div_ct = make_fastdiv((uint32_t)(g.dw ? 1 : g.Cp >= 32 ? g.Cp / 32 : 1));
+  g.div_kw = make_fastdiv((uint32_t)g.KW);
+  return CVMHIP_OK;
+}
+
+int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, void* ws, size_t ws_bytes,
+                  hipStream_t s) {
+  Epilogue ep;
+  const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
+  if (prc) return prc;
   const bool wide = (g.Kp % 128) == 0;
   const int gran = g.Cp >= 16 ? 16 : g.Cp;
   // Tile choice: the largest tile that still yields >= 2 workgroups per CU;
@@ -1374,10 +1522,6 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     wm = tune.tile_wm;
     wn = tune.tile_wn;
   }
-  g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
-  g.div_ow = make_fastdiv((uint32_t)g.OW);
-  g.div_ct = make_fastdiv((uint32_t)(g.dw ? 1 : g.Cp >= 32 ? g.Cp / 32 : 1));
-  g.div_kw = make_fastdiv((uint32_t)g.KW);
   // kernel choice: the wavefront-private kernel when the layout allows it and its grid fits the chip,
   // else the LDS-tiled kernel.  The calling thread's tuning (cvmhip_set_conv_tuning) can force one of
   // them or a configuration of the wavefront kernel; nothing is read from the environment here.
@@ -1460,6 +1604,64 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (ep.out_mode == OUT_I8_ACT) launch_out<OUT_I8_ACT>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
   else launch_out<OUT_I32_NCHW>(wm, wn, gran, wide, grid, s, xp, wp, out, g, ep);
   return check_launch("conv_igemm");
+}
+
+
+// ---- layer-sequence launch: host side
+size_t conv_seq_layer_bytes() { return sizeof(SeqLayer); }
+int conv_seq_shares() { return SEQ_SHARES; }
+size_t conv_seq_sync_bytes() { return (SEQ_SHARES + 1) * SEQ_SYNC_WORDS * sizeof(unsigned); }
+
+// Fills entry `index` of a host copy of the table.  CVMHIP_ERR_ARG with "not eligible" when this convolution
+// cannot be one layer of a sequence (the caller then launches it on its own).
+int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in) {
+  Epilogue ep;
+  const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
+  if (prc) return prc;
+  const bool nopad = g.PH == 0 && g.PW == 0;
+  if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT ||
+      !(nopad || (g.KH <= 32 && g.KW <= 32)))
+    return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
+  SeqLayer& L = reinterpret_cast<SeqLayer*>(table)[index];
+  memset(&L, 0, sizeof(L));
+  L.px_per_share = (int)(g.P / SEQ_SHARES);
+  // the configuration is chosen for one share on the 32 compute units of its XCD
+  ConvGeom share = g;
+  share.P = L.px_per_share;
+  int cfg = choose_wave_cfg(share, SEQ_WG_PER_SHARE);
+  const ConvTuning tune = t_conv_tuning;
+  if (tune.wave_cfg >= 0 && tune.wave_cfg <= 6) cfg = tune.wave_cfg;
+  if (cfg > 6) cfg = 3;
+  const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                       ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
+  const WaveCfg& c = kWaveCfgs[cfg];
+  const int bm = 32 * c.tm, bn = 32 * c.tn * (c.nw / c.ksplit);
+  g.octiles = (g.OC + bm - 1) / bm;
+  g.div_octiles = make_fastdiv((uint32_t)g.octiles);
+  // a share begins at a multiple of px_per_share, which need not be a multiple of 32: its first pixel block
+  // may start up to 31 pixels early (those pixels are computed and not stored)
+  int ptiles = 0;
+  for (int x = 0; x < SEQ_SHARES; ++x) {
+    const int lead = (x * L.px_per_share) & 31;
+    const int t = (lead + L.px_per_share + bn - 1) / bn;
+    ptiles = t > ptiles ? t : ptiles;
+  }
+  L.ptiles = ptiles;
+  L.kernel = cfg * 3 + (mode == WAVE_IDENT ? 0 : mode == WAVE_NOPAD ? 1 : 2);
+  L.xp = xp;
+  L.wf = wp;
+  L.out = out;
+  L.g = g;
+  L.ep = ep;
+  return CVMHIP_OK;
+}
+
+int conv_seq_launch(const void* dev_table, int nlayers, void* sync, hipStream_t s) {
+  if (!dev_table || nlayers < 1 || !sync || ((uintptr_t)dev_table & 15) || ((uintptr_t)sync & 255)) return arg_error("conv_seq_launch");
+  KernelTimer timer("k_conv_seq", 0, s, 0, "layer sequence");
+  k_conv_seq<<<SEQ_SHARES * SEQ_WG_PER_SHARE, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers,
+                                                          reinterpret_cast<unsigned*>(sync), 2000000);
+  return check_launch("conv_seq");
 }
 
 }  // namespace cvmhip

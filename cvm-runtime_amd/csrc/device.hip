@@ -233,6 +233,16 @@ int cvmhip_event_record(void* event, void* stream) {
   return CVMHIP_OK;
 }
 
+int cvmhip_device_sync(void) {
+  HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize");
+  return CVMHIP_OK;
+}
+
+int cvmhip_stream_wait_event(void* stream, void* event) {
+  HIP_TRY(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0), "hipStreamWaitEvent");
+  return CVMHIP_OK;
+}
+
 int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms) {
   HIP_TRY(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize");
   HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");

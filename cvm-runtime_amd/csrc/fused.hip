@@ -230,7 +230,8 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
                          const void* residual, const cvmhip_chain* chain2, void* out, int out_is_i8, int64_t nhwc_image_stride,
                          int n, int ic, int h, int wd, int oc, int kh, int kw,
                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream,
-                         void* ws = nullptr, size_t ws_bytes = 0, size_t* ws_query = nullptr) {
+                         void* ws = nullptr, size_t ws_bytes = 0, size_t* ws_query = nullptr, void* seq_table = nullptr,
+                         int seq_index = 0) {
   if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
   if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
       pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
@@ -259,6 +260,8 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
     *ws_query = nhwc_image_stride >= 0 ? 0 : conv_slices_workspace_bytes(g, ep);
     return CVMHIP_OK;
   }
+  if (seq_table)   // describe the launch as one layer of a layer-sequence launch instead of issuing it
+    return conv_seq_layer(seq_table, seq_index, reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep);
   if (nhwc_image_stride >= 0) ws = nullptr;
   return conv_igemm_ws(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep, ws, ws_bytes,
                        as_stream(stream));
@@ -288,6 +291,23 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
   return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, out_is_i8, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
                        pad_h, pad_w, dil_h, dil_w, stream);
+}
+
+size_t cvmhip_conv_seq_layer_bytes(void) { return conv_seq_layer_bytes(); }
+size_t cvmhip_conv_seq_sync_bytes(void) { return conv_seq_sync_bytes(); }
+int cvmhip_conv_seq_shares(void) { return conv_seq_shares(); }
+
+int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          const void* residual, const cvmhip_chain* chain2, void* out,
+                          int n, int ic, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w) {
+  if (!table || index < 0) return arg_error("conv_seq_layer table");
+  return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, 1, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
+                       pad_h, pad_w, dil_h, dil_w, nullptr, nullptr, 0, nullptr, table, index);
+}
+
+int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, void* stream) {
+  return conv_seq_launch(dev_table, nlayers, sync, as_stream(stream));
 }
 
 int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,

@@ -596,6 +596,57 @@ void HipGraphRuntime::BuildPlan() {
   }
   plan_ = std::move(plan);
   fused_ = true;
+  if (hooks_.seq) BuildSequences();
+}
+
+// Runs of at least three consecutive convolution steps that a layer-sequence launch can take (batch a multiple
+// of 8, int8 in and out, channels padded to 32, no K slices) become one launch each.  Consecutive plan steps
+// only depend on earlier ones, which is all a sequence needs.
+void HipGraphRuntime::BuildSequences() {
+  seq_at_.assign(plan_.size(), -1);
+  const size_t entry = cvmhip_conv_seq_layer_bytes();
+  std::vector<char> table;
+  size_t i = 0;
+  while (i < plan_.size()) {
+    table.clear();
+    size_t j = i;
+    for (; j < plan_.size(); ++j) {
+      const PlanStep& st = plan_[j];
+      if (st.kind != PlanStep::CONV || st.stem || st.nhwc || st.ws || !st.out_i8) break;
+      table.resize((j - i + 1) * entry);
+      const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
+      const int rc = cvmhip_conv_seq_layer(table.data(), static_cast<int>(j - i), i8_ptr_[st.src],
+                                           static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res, &st.chain2,
+                                           i8_ptr_[st.dst], st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh, st.sw, st.ph,
+                                           st.pw, st.dh, st.dw);
+      if (rc != CVMHIP_OK) break;
+    }
+    const size_t count = j - i;
+    if (count >= 3) {
+      auto buf = std::make_shared<DeviceBuffer>();
+      Check(cvmhip_alloc(&buf->ptr, count * entry), "layer-sequence table");
+      Check(cvmhip_copy_h2d(buf->ptr, table.data(), count * entry, stream_), "layer-sequence table");
+      Check(cvmhip_stream_sync(stream_), "layer-sequence table");   // the host copy goes away
+      SeqRun r;
+      r.first = i;
+      r.last = j - 1;
+      r.owner = buf;
+      r.table = buf->ptr;
+      r.nlayers = static_cast<int>(count);
+      seq_at_[i] = static_cast<int>(seqs_.size());
+      seqs_.push_back(r);
+    }
+    i = j > i ? j : i + 1;
+  }
+  if (seqs_.empty()) return;
+  const size_t words = cvmhip_conv_seq_sync_bytes() / 4;
+  Check(cvmhip_alloc(&seq_sync_, words * 4), "layer-sequence counters");
+  Check(cvmhip_memset32(seq_sync_, 0, words, stream_), "layer-sequence counters");
+  void* host = nullptr;
+  Check(cvmhip_host_alloc(&host, 64), "layer-sequence status");
+  seq_error_host_ = static_cast<uint32_t*>(host);
+  use_seq_ = true;
+  CountSequenceModel(+1);
 }
 
 void HipGraphRuntime::RunStep(PlanStep& st) {

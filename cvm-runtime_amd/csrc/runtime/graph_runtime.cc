@@ -5,6 +5,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <iostream>
+#include <atomic>
+#include <mutex>
 #include <unordered_set>
 
 #include "../../../include/cvm_hip_ops.h"
@@ -445,6 +447,7 @@ void HipGraphRuntime::ReadHooks() {
   auto env = [](const char* name) { const char* v = std::getenv(name); return std::string(v ? v : ""); };
   hooks_.fuse = env("CVM_HIP_FUSE") != "0";
   hooks_.graph = env("CVM_HIP_GRAPH") != "0";
+  hooks_.seq = env("CVM_HIP_SEQ") != "0";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
   hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : 0;
@@ -458,6 +461,10 @@ void HipGraphRuntime::ReadHooks() {
 void HipGraphRuntime::Release() {
   if (graph_exec_) { cvmhip_graph_destroy(graph_exec_); graph_exec_ = nullptr; }
   plan_.clear();
+  if (!seqs_.empty()) CountSequenceModel(-1);
+  seqs_.clear();
+  if (seq_sync_) { cvmhip_free(seq_sync_); seq_sync_ = nullptr; }
+  if (seq_error_host_) { cvmhip_host_free(seq_error_host_); seq_error_host_ = nullptr; }
   execs_.clear();  // releases per-node device state before the stream goes away
   if (i8_slab_) { cvmhip_free(i8_slab_); i8_slab_ = nullptr; }
   if (in_stage_dev_) { cvmhip_free(in_stage_dev_); in_stage_dev_ = nullptr; }
@@ -649,11 +656,53 @@ void HipGraphRuntime::LoadParams(const std::string& blob) {
 }
 
 // ---------------------------------------------------------------- execution
+// A layer-sequence launch occupies every compute unit and waits, inside the kernel, for all of its workgroups:
+// two of them in flight at once (two models on two streams) could each hold part of the chip and wait for the
+// rest.  So a run that contains one starts only after the previous such run of this process has finished: the
+// stream waits for the event recorded behind that run.  Runs without sequence launches are not affected.
+// A single model needs none of this (its runs are ordered by its stream): the gate acts only while the process
+// holds more than one model with sequence launches.
+namespace {
+std::atomic<int> g_sequence_models{0};
+struct SequenceGate {
+  static std::mutex& Mutex() { static std::mutex m; return m; }
+  static void*& Last() { static void* e = nullptr; return e; }
+  void* stream;
+  bool active;
+  std::unique_lock<std::mutex> lock;
+  explicit SequenceGate(void* s) : stream(s), active(g_sequence_models.load() > 1) {
+    if (!active) return;
+    lock = std::unique_lock<std::mutex>(Mutex());
+    if (Last()) HipCheck(cvmhip_stream_wait_event(stream, Last()), "sequence gate");
+    else HipCheck(cvmhip_event_create(&Last()), "sequence gate");
+  }
+  ~SequenceGate() { if (active) cvmhip_event_record(Last(), stream); }
+};
+}  // namespace
+
+// A second model with sequence launches appears: what the first one has in flight is drained once, from then on
+// every such run goes through the gate.
+void HipGraphRuntime::CountSequenceModel(int delta) {
+  if (delta > 0 && g_sequence_models.fetch_add(1) >= 1) HipCheck(cvmhip_device_sync(), "sequence gate");
+  if (delta < 0) g_sequence_models.fetch_sub(1);
+}
+
 void HipGraphRuntime::Launch() {
   // the kernel choice this model was loaded with, for the launches of this thread
   HipCheck(cvmhip_set_conv_tuning(hooks_.conv_kernel, hooks_.wave_cfg, hooks_.tile_wm, hooks_.tile_wn), "conv tuning");
   if (fused_) {
-    for (PlanStep& st : plan_) RunStep(st);
+    // a kernel-timing session wants one event pair per layer: it sees the steps, not the sequence launch
+    const bool seq = use_seq_ && !cvmhip_kernel_timing_active();
+    for (size_t i = 0; i < plan_.size();) {
+      if (seq && seq_at_[i] >= 0) {
+        const SeqRun& r = seqs_[seq_at_[i]];
+        HipCheck(cvmhip_conv_seq_launch(r.table, r.nlayers, seq_sync_, stream_), "layer-sequence launch");
+        seq_ran_ = true;
+        i = r.last + 1;
+      } else {
+        RunStep(plan_[i++]);
+      }
+    }
   } else {
     for (Exec& ex : execs_) ex.kernel->run(ex.call);
   }
@@ -667,11 +716,21 @@ void HipGraphRuntime::Launch() {
 void HipGraphRuntime::Run() {
   if (graph_state_ == 0) graph_state_ = hooks_.graph ? 1 : -1;
   if (graph_state_ < 0 || cvmhip_kernel_timing_active()) {
-    Launch();
+    if (use_seq_ && !cvmhip_kernel_timing_active()) {
+      SequenceGate gate(stream_);
+      Launch();
+    } else {
+      Launch();
+    }
     return;
   }
   if (graph_state_ == 1) {  // first run: eager (operators may finish lazy set-up)
-    Launch();
+    if (use_seq_) {
+      SequenceGate gate(stream_);
+      Launch();
+    } else {
+      Launch();
+    }
     graph_state_ = 2;
     return;
   }
@@ -699,6 +758,12 @@ void HipGraphRuntime::Run() {
       Launch();
       return;
     }
+  }
+  if (use_seq_) {
+    SequenceGate gate(stream_);
+    HipCheck(cvmhip_graph_launch(graph_exec_, stream_), "graph launch");
+    seq_ran_ = true;
+    return;
   }
   HipCheck(cvmhip_graph_launch(graph_exec_, stream_), "graph launch");
 }
@@ -742,6 +807,29 @@ void HipGraphRuntime::CopyOutputTo(int index, int32_t* host) {
   const uint32_t eid = entry_id(outputs_[index]);
   HipCheck(cvmhip_copy_d2h(host, entry_ptr_[eid], static_cast<size_t>(shape_size(shape_[eid])) * 4, stream_), "copy output");
   HipCheck(cvmhip_stream_sync(stream_), "copy output");
+  if (seq_ran_) {
+    CheckSequences();
+    if (!use_seq_) CopyOutputTo(index, host);   // the run was repeated with one launch per layer
+  }
+}
+
+// A layer-sequence launch whose bounded waits ran out (its workgroups were not all resident at once) leaves its error
+// word set and its results undefined.  Seen after a synchronisation: sequences are switched off for this model for
+// good and the run is repeated with one launch per layer.
+void HipGraphRuntime::CheckSequences() {
+  seq_ran_ = false;
+  if (!use_seq_ || !seq_sync_) return;
+  const size_t words = cvmhip_conv_seq_sync_bytes() / 4;
+  HipCheck(cvmhip_copy_d2h(seq_error_host_, static_cast<uint32_t*>(seq_sync_) + (words - 64), 4, stream_), "sequence status");
+  HipCheck(cvmhip_stream_sync(stream_), "sequence status");
+  if (*seq_error_host_ == 0) return;
+  std::cerr << "cvm hip: a layer-sequence launch could not keep all its workgroups resident; using one launch per layer\n";
+  use_seq_ = false;
+  HipCheck(cvmhip_memset32(seq_sync_, 0, words, stream_), "sequence status");
+  if (graph_exec_) { cvmhip_graph_destroy(graph_exec_); graph_exec_ = nullptr; }
+  graph_state_ = 0;
+  Run();
+  HipCheck(cvmhip_stream_sync(stream_), "repeat run");
 }
 
 const std::vector<const int32_t*>& HipGraphRuntime::FetchOutputs() {
@@ -761,6 +849,10 @@ const std::vector<const int32_t*>& HipGraphRuntime::FetchOutputs() {
                              stream_), "copy output");
   }
   HipCheck(cvmhip_stream_sync(stream_), "copy output");
+  if (seq_ran_) {
+    CheckSequences();
+    if (!use_seq_) return FetchOutputs();   // the run was repeated with one launch per layer
+  }
   return out_host_;
 }
 
@@ -769,7 +861,10 @@ int32_t* HipGraphRuntime::DataDevicePtr() {
   return entry_ptr_[entry_id(input_nodes_[idx], 0)];
 }
 
-void HipGraphRuntime::SyncStream() { HipCheck(cvmhip_stream_sync(stream_), "synchronise"); }
+void HipGraphRuntime::SyncStream() {
+  HipCheck(cvmhip_stream_sync(stream_), "synchronise");
+  if (seq_ran_) CheckSequences();
+}
 
 const Shape& HipGraphRuntime::InputShape() const {
   const int idx = GetInputIndex("data");

@@ -195,11 +195,12 @@ class HipGraphRuntime {
   int graph_state_ = 0;  // 0 undecided, -1 eager for good, 1 before the first run, 2 ready to capture, 3 captured
 
   // Test and tuning hooks, read from the environment once, when the model is constructed (never on the
-  // launch path): CVM_HIP_FUSE=0 no load-time fusion, CVM_HIP_GRAPH=0 no graph replay, CVM_HIP_DW=valu
+  // launch path): CVM_HIP_FUSE=0 no load-time fusion, CVM_HIP_GRAPH=0 no graph replay, CVM_HIP_SEQ=0 no
+  // layer-sequence launches, CVM_HIP_DW=valu
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;
@@ -213,6 +214,25 @@ class HipGraphRuntime {
   std::vector<void*> i8_ptr_;      // per entry: int8 NHWC form (nullptr if never materialised)
   std::vector<std::shared_ptr<void>> own_storage_;  // int32 tensors the planner moved out of the shared storage pool
   void* i8_slab_ = nullptr;
+
+  // ---- runs of consecutive convolution steps issued as one layer-sequence launch (cvmhip_conv_seq_launch).  The
+  // steps stay in plan_: they are what runs when sequences are switched off, when a kernel-timing session wants
+  // one event pair per layer, and after a sequence launch reported that its waits ran out.
+  struct SeqRun {
+    size_t first = 0, last = 0;         // plan_ indices, inclusive
+    std::shared_ptr<void> owner;        // device copy of the layer table
+    void* table = nullptr;
+    int nlayers = 0;
+  };
+  void BuildSequences();
+  static void CountSequenceModel(int delta);   // models with sequence launches alive in this process
+  void CheckSequences();                // after a synchronisation: did a sequence launch give up?
+  std::vector<SeqRun> seqs_;
+  std::vector<int> seq_at_;             // per plan_ index: the run that starts there, or -1
+  void* seq_sync_ = nullptr;            // counters and error word of the sequence launches (device)
+  uint32_t* seq_error_host_ = nullptr;  // pinned copy of the error word
+  bool use_seq_ = false;
+  bool seq_ran_ = false;                // a sequence launch was issued since the last check
 };
 
 }  // namespace cvmrt

@@ -190,6 +190,8 @@ int cvmhip_event_create(void** event);
 int cvmhip_event_destroy(void* event);
 int cvmhip_event_record(void* event, void* stream);
 int cvmhip_event_elapsed_ms(void* start, void* stop, float* ms);
+int cvmhip_device_sync(void);                               /* every stream of the current device */
+int cvmhip_stream_wait_event(void* stream, void* event);   /* work issued to `stream` later waits for `event` */
 /* Per-kernel device time for a measurement harness: between begin and end the
  * implicit-GEMM and packing launches are bracketed by event pairs on their own
  * stream; end synchronises and writes {"kernel": {"launches", "ms", "work"}}
@@ -279,6 +281,25 @@ int cvmhip_conv2d_i8_ws(const void* xp, const void* wp, const int32_t* bias, con
                         int n, int ic, int h, int wd, int oc, int kh, int kw,
                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
                         void* workspace, size_t workspace_bytes, void* stream);
+/* A run of convolutions in ONE launch, for a batch that is a multiple of cvmhip_conv_seq_shares() (8, the XCDs
+ * of the chip).  No counterpart in the reference.  Images are independent, so every XCD computes all layers
+ * of the run for its own share of the images; a layer boundary is then a counter in that XCD's L2 instead of a
+ * kernel boundary (no L2 write-back, the next layer's operands are still in the L2).  Use: fill a host table of
+ * n * cvmhip_conv_seq_layer_bytes() bytes with cvmhip_conv_seq_layer (entry i describes what
+ * cvmhip_conv2d_i8 with the same arguments and an int8 output would compute; it returns 10 when that layer
+ * cannot be part of a run), copy the table to the device, and launch it.  Layer i may read what layers < i of
+ * the run or earlier launches wrote.  `sync` is cvmhip_conv_seq_sync_bytes() of device memory, zeroed once,
+ * 256-byte aligned; its last 256-byte block starts with an error word that is non-zero after a launch whose
+ * bounded waits ran out (results invalid; the caller falls back to one launch per layer).  The launch needs
+ * every compute unit: two of them must never be in flight at the same time on one device. */
+size_t cvmhip_conv_seq_layer_bytes(void);
+size_t cvmhip_conv_seq_sync_bytes(void);
+int cvmhip_conv_seq_shares(void);
+int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                          const void* residual, const cvmhip_chain* chain2, void* out,
+                          int n, int ic, int h, int wd, int oc, int kh, int kw,
+                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, void* stream);
 /* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values
  * are contiguous at out + n*image_stride (elements).  This is what conv2d -> transpose(0,2,3,1) ->
  * reshape -> concatenate produces for a detection head (transpose: ops.cc:743-789, concatenate:
