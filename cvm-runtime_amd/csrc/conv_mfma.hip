@@ -530,11 +530,39 @@ enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 // pixel range [p_begin, p_end) (COH only; otherwise the whole layer), computed by the NW wavefronts whose thread index is `tid`, with
 // sPart / sBias their LDS.  k_conv_wave is this function over a grid; the layer-sequence kernel calls it
 // from its loop over layers with COH set (operands written earlier in the same launch).
+// Layer boundary of the layer-sequence kernel, seen from the layer that follows: its wavefronts compute their
+// addresses and request their filter operands first, and only then wait here until every workgroup of the
+// XCD has counted itself out of the previous layer -- the filter does not depend on that layer, so its trip
+// from memory overlaps the wait.  The wait is bounded; when it runs out, or another one has, the error word is
+// set and the wavefront goes on (the results are then void, and every later wait ends after 1024 polls).
+struct LayerGate {
+  unsigned* counter;   // nullptr: nothing to wait for
+  unsigned target;
+  unsigned* error;
+  int spin_limit;
+};
+__device__ __forceinline__ void gate_wait(const LayerGate& gate) {
+  if (!gate.counter) return;
+  unsigned v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  int spins = 0;
+  while (v < gate.target) {
+    __builtin_amdgcn_s_sleep(1);
+    v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    if ((++spins & 1023) == 0) {
+      const unsigned e = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      if (e != 0 || spins > gate.spin_limit) {
+        __hip_atomic_store(gate.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+    }
+  }
+}
+
 template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
-                                               const int p_end = 0) {
+                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0}) {
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
   constexpr int BM = 32 * TM;             // output channels per workgroup
   constexpr int WPIX = 32 * TN;           // pixels per wavefront
@@ -660,7 +688,15 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   auto put = [](regs_t& R, int b, const int4 v) __attribute__((always_inline)) {
     R[b] = v.x; R[b + 1] = v.y; R[b + 2] = v.z; R[b + 3] = v.w;
   };
-  auto fetch = [&]() __attribute__((always_inline)) -> regs_t {
+  uint32_t rp[NU];
+  // COH: called once, between the filter requests and the activation requests of the first batch
+  auto pass_gate = [&]() __attribute__((always_inline)) {
+    if constexpr (COH) {
+      gate_wait(gate);
+      if (ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+    }
+  };
+  auto fetch = [&](const bool gated) __attribute__((always_inline)) -> regs_t {
     regs_t R;
     if (MODE == WAVE_IDENT) {
       // One path, loads always in the same order (filter blocks, then pixel blocks; the chunks of a
@@ -679,6 +715,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)ca[d] * 1024));
+      if (gated) pass_gate();
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -696,6 +733,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       const int chunk = live ? cur : nch;
 #pragma unroll
       for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024));
+      if (gated && d == 0) pass_gate();
       if (MODE == WAVE_ROWS) {
         // 16-byte unit k16 of K: filter row k16 / (row_bytes/16), part k16 % (row_bytes/16) of its window
         const int k16 = (live ? cur : 0) * 2 + lgrp;
@@ -774,9 +812,8 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // every outstanding load first), the operands of the first batch, then the bias, which is kept in a
   // register and staged in LDS after the loop (staging it here would put a full memory latency in
   // front of the first operand request).
-  uint32_t rp[NU];
-  if (ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
-  regs_t R0 = fetch();
+  if (!COH && ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+  regs_t R0 = fetch(COH);
   int bias_mine = 0;
   if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
 
@@ -786,13 +823,13 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     // bound by exactly that.
     consume(R0, true);
   } else {
-    regs_t R1 = fetch();
+    regs_t R1 = fetch(false);
     consume(R0, true);
     for (int it = 1; it < niter; it += 2) {
-      R0 = fetch();
+      R0 = fetch(false);
       consume(R1, false);
       if (it + 1 >= niter) break;
-      R1 = fetch();
+      R1 = fetch(false);
       consume(R0, false);
     }
   }
@@ -884,14 +921,15 @@ enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
 template <int TM, int TN, int KSPLIT, int NW, int D, int MODE>
 __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                                 int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
-                                                int p_end) {
+                                                int p_end, const LayerGate gate) {
   constexpr int UNITS = 8 / NW;   // tiles a workgroup computes side by side
   const int half = UNITS == 2 ? (tid >> 8) : 0;
   const int htid = UNITS == 2 ? (tid & 255) : tid;
   for (int base = 0; base < ntiles; base += SEQ_WG_PER_SHARE * UNITS) {
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
     conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
-                                                                         sPart + half * 16384, sBias + half * 64, p_begin, p_end);
+                                                                         sPart + half * 16384, sBias + half * 64, p_begin, p_end,
+                                                                         base == 0 ? gate : LayerGate{nullptr, 0, nullptr, 0});
     __syncthreads();   // the next tile reuses the LDS
   }
 }
@@ -899,15 +937,15 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
 template <int MODE>
 __device__ __forceinline__ void seq_layer_cfg(int cfg, const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                               int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
-                                              int p_end) {
+                                              int p_end, const LayerGate gate) {
   switch (cfg) {
-    case 0: seq_layer_tiles<2, 2, 8, 8, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    case 1: seq_layer_tiles<2, 2, 4, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    case 2: seq_layer_tiles<2, 2, 2, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    case 3: seq_layer_tiles<2, 2, 1, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    case 4: seq_layer_tiles<1, 2, 8, 8, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    case 5: seq_layer_tiles<1, 2, 4, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
-    default: seq_layer_tiles<1, 2, 1, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end); break;
+    case 0: seq_layer_tiles<2, 2, 8, 8, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 1: seq_layer_tiles<2, 2, 4, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 2: seq_layer_tiles<2, 2, 2, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 3: seq_layer_tiles<2, 2, 1, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 4: seq_layer_tiles<1, 2, 8, 8, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 5: seq_layer_tiles<1, 2, 4, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    default: seq_layer_tiles<1, 2, 1, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
   }
 }
 
@@ -915,12 +953,18 @@ __global__ void __launch_bounds__(512, 1)
 k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit) {
   __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: one 8-wavefront tile set or two 4-wavefront ones
   __shared__ __attribute__((aligned(16))) int sBias[128];
-  __shared__ int s_rank, s_stop;
-  // The table never changes during the launch.  It is read through the constant address space, so that a field is
-  // a scalar load wherever it is needed, as a kernel argument would be (a copy in registers would hold ~100 scalar
-  // registers for the whole layer).
-  typedef const SeqLayer __attribute__((address_space(4))) * table_t;
-  const table_t table = (table_t)(uintptr_t)layers_generic;
+  __shared__ int s_rank;
+  // The current layer's table entry lives in LDS, where any field is a short read away wherever the code needs
+  // it (a copy in registers would hold ~100 scalar registers for the whole layer, and reading it from memory
+  // would begin every layer with a trip there).  The first wavefront requests the next entry when a layer
+  // begins and stores it to the other LDS slot before the layer boundary.
+  constexpr int LWORDS = (int)(sizeof(SeqLayer) / 4);
+  static_assert(sizeof(SeqLayer) % 16 == 0 && LWORDS <= 128, "a table entry is copied by one wavefront, two words per lane");
+  __shared__ __attribute__((aligned(16))) uint32_t sLayer[2][LWORDS];
+  {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(layers_generic);
+    if ((int)threadIdx.x < LWORDS) sLayer[0][threadIdx.x] = src[threadIdx.x];
+  }
   const int tid = threadIdx.x;
   unsigned xcc;
   asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
@@ -931,13 +975,19 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const unsigned r = __hip_atomic_fetch_add(my + SEQ_ARRIVE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (xcc >= SEQ_SHARES || r >= SEQ_WG_PER_SHARE) __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // not the chip this kernel is laid out for
     s_rank = (int)r;
-    s_stop = 0;
   }
   __syncthreads();
   const int rank = s_rank;
-  bool stop = xcc >= SEQ_SHARES || rank >= SEQ_WG_PER_SHARE;
+  const bool stop = xcc >= SEQ_SHARES || rank >= SEQ_WG_PER_SHARE;
   for (int l = 0; l < nlayers && !stop; ++l) {
-    const SeqLayer& L = *(const SeqLayer*)(table + l);
+    const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer[l & 1]);
+    uint32_t next0 = 0, next1 = 0;
+    const bool fetch_next = tid < 64 && l + 1 < nlayers;
+    if (fetch_next) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(layers_generic + l + 1);
+      next0 = src[tid];
+      if (tid + 64 < LWORDS) next1 = src[tid + 64];
+    }
     const ConvGeom& g = L.g;
     const Epilogue& ep = L.ep;
     const int8_t* xp = L.xp;
@@ -949,28 +999,20 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int ntiles = g.octiles * L.ptiles;
     const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
-    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
-    else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
-    else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end);
+    // layer l may read what layer l - 1 wrote once all 32 workgroups of the XCD have counted themselves out of it
+    const LayerGate gate = {l > 0 ? my + SEQ_BAR : nullptr, (unsigned)l * SEQ_WG_PER_SHARE, error, spin_limit};
+    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
+    else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
+    else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
     if (l + 1 == nlayers) break;
-    // ---- layer boundary inside the XCD: every store of this wavefront is in the L2, then count and wait
+    if (fetch_next) {
+      sLayer[(l + 1) & 1][tid] = next0;
+      if (tid + 64 < LWORDS) sLayer[(l + 1) & 1][tid + 64] = next1;
+    }
+    // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (tid == 0) {
-      __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned target = (unsigned)(l + 1) * SEQ_WG_PER_SHARE;
-      int spins = 0, bad = 0;
-      while (__hip_atomic_load(my + SEQ_BAR, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-        if (++spins > spin_limit || __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { bad = 1; break; }
-        __builtin_amdgcn_s_sleep(1);
-      }
-      if (bad) {
-        __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_stop = 1;
-      }
-    }
-    __syncthreads();
-    stop = s_stop != 0;
+    if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   // the last workgroup of a share to finish clears the share's counters for the next launch
   __syncthreads();
