@@ -129,7 +129,8 @@ def layer_table(args, pkg, L, model, title):
         empties = [d for n, d in seq if n == "k_copy16"]
         if empties:
             empty_us = statistics.median(empties[-50:])
-    print("# %s, batch %d: %d launches per step, %.1f us per step without instrumentation" % (title, args.batch, per_step, plain_us))
+    print("# %s, batch %d, one launch per layer (layer-sequence launches switched off): %d launches per step, %.1f us per step "
+          "without instrumentation" % (title, args.batch, per_step, plain_us))
     print("# durations: %s; sum %.1f us" % (source, sum(dur)))
     if empty_us is not None:
         print("# a launch that does nothing (256-byte copy kernel): %.2f us in the same trace" % empty_us)
@@ -206,7 +207,10 @@ def main():
     js, pb = g.build(heads)
     gmac = g.macs / 1e9
     x = synth.tensor("bench", "data", g.shape((0, 0)), -127, 127).astype(np.int8)
+    if args.layers:
+        os.environ["CVM_HIP_SEQ"] = "0"     # the table is about single layers: one launch each
     model = runtime.HipModel(js, pb)
+    launch_counts = model.launch_counts()
     model.set_input(x.tobytes())            # input resident in HBM from here on
     model.time_run(max(args.warmup, 1))
     torch.cuda.synchronize()
@@ -276,15 +280,15 @@ def main():
                                            ctypes.c_size_t(a.numel()), None))
         torch.cuda.synchronize()
 
-    # The two implicit-GEMM kernels (same arithmetic, chosen per layer); the roofline object is about the
-    # one that takes more of the step.  An event pair makes a launch look longer than it is.  Every launch
+    # The implicit-GEMM kernels (same arithmetic, chosen per layer; k_conv_seq is a run of layers in one launch);
+    # the roofline object is about the one that takes more of the step.  An event pair makes a launch look longer than it is.  Every launch
     # of a step is timed and the un-instrumented step is GPU-bound with its kernels back to back, so the
     # cost of one pair is (sum of all pair times - un-instrumented step time) / launches; it is taken off
     # every launch.  The rocprofv3 kernel trace under profiles/ measures the same durations directly.
     n_timed = sum(v["launches"] for v in kt.values())
     pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall * 1e6) / max(n_timed, 1))
     pair_us = {"empty_us": pair_cost_us}
-    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm")}
+    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq")}
     dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
     conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
     launches = max(conv["launches"], 1)
@@ -311,6 +315,8 @@ def main():
         "config": {"workload": titles[args.workload] % args.batch,
                    "batch": args.batch, "graph_nodes": len(g.nodes), "gmac_per_step": gmac,
                    "device_ms_per_step": dev_ms / args.steps,
+                   "kernel_launches_per_step": launch_counts[0], "layer_sequence_launches": launch_counts[1],
+                   "convolutions_inside_layer_sequences": launch_counts[2],
                    "ms_per_step_with_kernel_events": wall_events / args.steps * 1e3,
                    "images_per_s_through_CVMAPIInference": args.batch / api_s,
                    "images_per_s_two_models_in_flight": two_models_rate,

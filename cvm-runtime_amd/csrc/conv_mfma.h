@@ -157,7 +157,7 @@ size_t conv_seq_layer_bytes();
 size_t conv_seq_sync_bytes();
 int conv_seq_shares();
 int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep);
-int conv_seq_launch(const void* dev_table, int nlayers, void* sync, hipStream_t s);
+int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s);
 
 }  // namespace cvmhip
 #endif

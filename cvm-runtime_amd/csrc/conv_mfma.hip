@@ -1698,9 +1698,11 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   return CVMHIP_OK;
 }
 
-int conv_seq_launch(const void* dev_table, int nlayers, void* sync, hipStream_t s) {
+int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s) {
   if (!dev_table || nlayers < 1 || !sync || ((uintptr_t)dev_table & 15) || ((uintptr_t)sync & 255)) return arg_error("conv_seq_launch");
-  KernelTimer timer("k_conv_seq", 0, s, 0, "layer sequence");
+  char desc[64];
+  snprintf(desc, sizeof(desc), "%d convolutions in one launch", nlayers);
+  KernelTimer timer("k_conv_seq", ops, s, bytes, desc);
   k_conv_seq<<<SEQ_SHARES * SEQ_WG_PER_SHARE, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers,
                                                           reinterpret_cast<unsigned*>(sync), 2000000);
   return check_launch("conv_seq");

@@ -306,8 +306,8 @@ int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp
                        pad_h, pad_w, dil_h, dil_w, nullptr, nullptr, 0, nullptr, table, index);
 }
 
-int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, void* stream) {
-  return conv_seq_launch(dev_table, nlayers, sync, as_stream(stream));
+int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream) {
+  return conv_seq_launch(dev_table, nlayers, sync, ops, bytes, as_stream(stream));
 }
 
 int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,

@@ -143,6 +143,13 @@ int CVMHIPTimeRun(void* net, int iterations, float* elapsed_ms) {
   API_END();
 }
 
+int CVMHIPLaunchCounts(void* net, int* launches_per_run, int* sequence_launches, int* layers_in_sequences) {
+  API_BEGIN();
+  NOT_NULL(net);
+  static_cast<HipModel*>(net)->runtime()->LaunchCounts(launches_per_run, sequence_launches, layers_in_sequences);
+  API_END();
+}
+
 int CVMHIPProfileOps(void* net, char* json_out, int capacity) {
   API_BEGIN();
   NOT_NULL(net);

@@ -633,6 +633,14 @@ void HipGraphRuntime::BuildSequences() {
       r.owner = buf;
       r.table = buf->ptr;
       r.nlayers = static_cast<int>(count);
+      for (size_t k = i; k < j; ++k) {
+        const PlanStep& st = plan_[k];
+        const int oh = (st.h + 2 * st.ph - (st.dh * (st.kh - 1) + 1)) / st.sh + 1, ow = (st.w + 2 * st.pw - (st.dw * (st.kw - 1) + 1)) / st.sw + 1;
+        const double px = static_cast<double>(st.n) * oh * ow;
+        r.ops += 2.0 * px * st.oc * st.c * st.kh * st.kw;
+        r.bytes += static_cast<double>(st.n) * st.h * st.w * st.c + static_cast<double>(st.oc) * st.c * st.kh * st.kw +
+                   px * st.oc * (st.src2 != kNone ? 2.0 : 1.0);
+      }
       seq_at_[i] = static_cast<int>(seqs_.size());
       seqs_.push_back(r);
     }

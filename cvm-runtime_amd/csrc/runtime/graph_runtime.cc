@@ -448,6 +448,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.fuse = env("CVM_HIP_FUSE") != "0";
   hooks_.graph = env("CVM_HIP_GRAPH") != "0";
   hooks_.seq = env("CVM_HIP_SEQ") != "0";
+  hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
   hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : 0;
@@ -653,6 +654,29 @@ void HipGraphRuntime::LoadParams(const std::string& blob) {
   if (hooks_.fuse) BuildPlan();
   HipCheck(cvmhip_stream_sync(stream_), "prepare operators");
   params_loaded_ = true;
+  if (use_seq_ && !hooks_.seq_forced) CalibrateSequences();
+}
+
+// Layer-sequence launches pay for layers that are bound by latency and cost a little where layers are large:
+// which way a model runs faster is measured once, when it is loaded (a few replays each way; timing does not
+// depend on the values in the tensors, so whatever the storage holds will do), unless CVM_HIP_SEQ=1 forces them.
+void HipGraphRuntime::CalibrateSequences() {
+  float ms[2] = {0, 0};
+  for (int with_seq = 0; with_seq < 2; ++with_seq) {
+    use_seq_ = with_seq != 0;
+    if (graph_exec_) { cvmhip_graph_destroy(graph_exec_); graph_exec_ = nullptr; }
+    graph_state_ = 0;
+    for (int i = 0; i < 3; ++i) Run();   // eager, capture, first replay
+    SyncStream();
+    if (with_seq && !use_seq_) {          // the launch could not run here: stay with one launch per layer
+      ms[1] = 1e30f;
+      break;
+    }
+    ms[with_seq] = TimeRuns(8);
+  }
+  use_seq_ = ms[1] < ms[0];
+  if (graph_exec_) { cvmhip_graph_destroy(graph_exec_); graph_exec_ = nullptr; }
+  graph_state_ = 0;
 }
 
 // ---------------------------------------------------------------- execution
@@ -691,12 +715,11 @@ void HipGraphRuntime::Launch() {
   // the kernel choice this model was loaded with, for the launches of this thread
   HipCheck(cvmhip_set_conv_tuning(hooks_.conv_kernel, hooks_.wave_cfg, hooks_.tile_wm, hooks_.tile_wn), "conv tuning");
   if (fused_) {
-    // a kernel-timing session wants one event pair per layer: it sees the steps, not the sequence launch
-    const bool seq = use_seq_ && !cvmhip_kernel_timing_active();
+    const bool seq = use_seq_;
     for (size_t i = 0; i < plan_.size();) {
       if (seq && seq_at_[i] >= 0) {
         const SeqRun& r = seqs_[seq_at_[i]];
-        HipCheck(cvmhip_conv_seq_launch(r.table, r.nlayers, seq_sync_, stream_), "layer-sequence launch");
+        HipCheck(cvmhip_conv_seq_launch(r.table, r.nlayers, seq_sync_, r.ops, r.bytes, stream_), "layer-sequence launch");
         seq_ran_ = true;
         i = r.last + 1;
       } else {
@@ -716,7 +739,7 @@ void HipGraphRuntime::Launch() {
 void HipGraphRuntime::Run() {
   if (graph_state_ == 0) graph_state_ = hooks_.graph ? 1 : -1;
   if (graph_state_ < 0 || cvmhip_kernel_timing_active()) {
-    if (use_seq_ && !cvmhip_kernel_timing_active()) {
+    if (use_seq_) {
       SequenceGate gate(stream_);
       Launch();
     } else {

@@ -148,6 +148,14 @@ class HipGraphRuntime {
   // number of launches per Run(): nodes when unfused, plan steps when fused
   size_t NumSteps() const { return fused_ ? plan_.size() : execs_.size(); }
   bool fused() const { return fused_; }
+  void LaunchCounts(int* launches, int* sequences, int* layers) const {
+    int seq = 0, lay = 0;
+    if (use_seq_)
+      for (const SeqRun& r : seqs_) { ++seq; lay += r.nlayers; }
+    if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq;
+    if (sequences) *sequences = seq;
+    if (layers) *layers = lay;
+  }
 
  private:
   uint32_t entry_id(uint32_t nid, uint32_t index) const { return node_row_ptr_[nid] + index; }
@@ -196,11 +204,11 @@ class HipGraphRuntime {
 
   // Test and tuning hooks, read from the environment once, when the model is constructed (never on the
   // launch path): CVM_HIP_FUSE=0 no load-time fusion, CVM_HIP_GRAPH=0 no graph replay, CVM_HIP_SEQ=0 no
-  // layer-sequence launches, CVM_HIP_DW=valu
+  // layer-sequence launches (=1: always, without measuring), CVM_HIP_DW=valu
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;
@@ -216,15 +224,17 @@ class HipGraphRuntime {
   void* i8_slab_ = nullptr;
 
   // ---- runs of consecutive convolution steps issued as one layer-sequence launch (cvmhip_conv_seq_launch).  The
-  // steps stay in plan_: they are what runs when sequences are switched off, when a kernel-timing session wants
-  // one event pair per layer, and after a sequence launch reported that its waits ran out.
+  // steps stay in plan_: they are what runs when sequences are switched off and after a sequence launch
+  // reported that its waits ran out.
   struct SeqRun {
     size_t first = 0, last = 0;         // plan_ indices, inclusive
     std::shared_ptr<void> owner;        // device copy of the layer table
     void* table = nullptr;
     int nlayers = 0;
+    double ops = 0, bytes = 0;          // algorithmic operations and HBM bytes of its layers (for the measurement harness)
   };
   void BuildSequences();
+  void CalibrateSequences();            // measures a run with and without sequence launches, keeps the faster
   static void CountSequenceModel(int delta);   // models with sequence launches alive in this process
   void CheckSequences();                // after a synchronisation: did a sequence launch give up?
   std::vector<SeqRun> seqs_;

@@ -136,6 +136,12 @@ class HipModel:
         _ck(lib().CVMHIPTimeRun(self.net, ctypes.c_int(iterations), ctypes.byref(ms)), "CVMHIPTimeRun")
         return ms.value
 
+    def launch_counts(self):
+        """(kernel launches per run, layer-sequence launches among them, convolutions inside those)"""
+        a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _ck(lib().CVMHIPLaunchCounts(self.net, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)), "CVMHIPLaunchCounts")
+        return a.value, b.value, c.value
+
     def profile_ops(self):
         buf = ctypes.create_string_buffer(1 << 16)
         _ck(lib().CVMHIPProfileOps(self.net, buf, ctypes.c_int(len(buf))), "CVMHIPProfileOps")

@@ -21,6 +21,9 @@ int CVMHIPGetOutput(void* net, char* output_data);
  * returns the elapsed device time in milliseconds, measured with events
  * recorded on the runtime's own stream. */
 int CVMHIPTimeRun(void* net, int iterations, float* elapsed_ms);
+/* What a run of the model issues: kernel launches per run, how many of them are layer-sequence launches
+ * (cvmhip_conv_seq_launch) and how many convolutions those contain.  Any pointer may be NULL. */
+int CVMHIPLaunchCounts(void* net, int* launches_per_run, int* sequence_launches, int* layers_in_sequences);
 /* Per-operator device time of one run as a JSON object {"op": ms, ...}
  * (the table the reference prints under -DPROFILE, graph_runtime.cc:62-87). */
 int CVMHIPProfileOps(void* net, char* json_out, int capacity);

@@ -299,7 +299,8 @@ int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp
                           const void* residual, const cvmhip_chain* chain2, void* out,
                           int n, int ic, int h, int wd, int oc, int kh, int kw,
                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
-int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, void* stream);
+/* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
+int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream);
 /* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values
  * are contiguous at out + n*image_stride (elements).  This is what conv2d -> transpose(0,2,3,1) ->
  * reshape -> concatenate produces for a detection head (transpose: ops.cc:743-789, concatenate:

@@ -1,0 +1,140 @@
+"""Layer-sequence launches (a run of convolutions in one kernel, every XCD computing all layers for its share
+of the images; include/cvm_hip_ops.h: cvmhip_conv_seq_*) against the CPU oracle executing the same graph node
+by node, and against the same model with one launch per layer.  Bit-exact.  CVM_HIP_SEQ=1 forces the
+sequences (by default a model measures both ways when it is loaded and keeps the faster), =0 switches them off."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle.graph as og
+from cvm_runtime_amd import graphgen, runtime, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(js, pb, x, seq):
+    os.environ["CVM_HIP_SEQ"] = seq
+    try:
+        m = runtime.HipModel(js, pb)
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+    try:
+        launches, sequences, layers = m.launch_counts()
+        assert (sequences >= 1 and layers >= 3) if seq == "1" else (sequences == 0 and layers == 0), (launches, sequences, layers)
+        outs = [m.inference(x.tobytes()) for _ in range(3)]      # eager run, captured run, replay
+        tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+        after = m.launch_counts()
+    finally:
+        m.close()
+    assert outs[0] == outs[1] == outs[2], "runs of one model differ"
+    assert m_counts_unchanged(seq, after), "a sequence launch gave up and the model fell back: %s" % (after,)
+    return np.frombuffer(outs[0], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+
+
+def m_counts_unchanged(seq, after):
+    return after[1] >= 1 if seq == "1" else after[1] == 0
+
+
+def _check(g, heads, cid, oracle_too=True):
+    js, pb = g.build(heads)
+    x = synth.tensor(cid, "data", g.shape((0, 0)), -127, 127).astype(np.int8)
+    with_seq = _run(js, pb, x, "1")
+    without = _run(js, pb, x, "0")
+    assert np.array_equal(with_seq, without), "%d of %d values differ from one launch per layer" % (
+        int((with_seq != without).sum()), without.size)
+    if oracle_too:
+        ref = og.run_graph(js, graphgen.load_params(pb), x.astype(np.int32))
+        want = np.concatenate([r.ravel() for r in ref])
+        assert np.array_equal(with_seq, want), "%d of %d values differ from the oracle" % (int((with_seq != want).sum()), want.size)
+
+
+def _chain(cid, n, c, hw, layers):
+    """data -> a chain of requantised convolutions given as (oc, k, stride, relu, residual_from) -> global sum."""
+    g = graphgen.GraphBuilder(cid)
+    x = g.var("data", (n, c, hw, hw), 8)
+    kept = [g.conv_relu_q(x, layers[0][0], 3, 1, 1)]          # the few-channel input layer stays outside the sequence
+    for oc, k, st, relu, res in layers[1:]:
+        y = g.conv_relu_q(kept[-1], oc, k, st, k // 2, relu=relu)
+        if res is not None and g.shape(kept[res]) == g.shape(y):
+            y = g.rshift(g.relu(g.add(y, kept[res])), 1)
+        kept.append(y)
+    s, _ = g.global_sum(kept[-1])
+    return g, [g.rshift(s, 6)]
+
+
+CHAINS = {
+    # batch 8: one image per XCD; 7x7 and 5x5 maps give shares that are not multiples of 32 (or of 8) pixels
+    "b8_1x1_3x3_residual": (8, 3, 14, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (64, 3, 1, True, None), (256, 1, 1, False, None),
+                                       (64, 1, 1, True, None), (64, 3, 1, True, None), (256, 1, 1, False, 3)]),
+    "b8_strided_no_padding": (8, 3, 15, [(32, 0, 0, 0, None), (64, 1, 2, True, None), (96, 3, 2, True, None), (128, 1, 1, True, None),
+                                         (128, 3, 1, False, None)]),
+    "b16_ragged_shares_7x7": (16, 3, 7, [(128, 0, 0, 0, None), (512, 1, 1, True, None), (128, 1, 1, True, None), (128, 3, 1, True, None),
+                                         (512, 1, 1, False, 1), (1000, 1, 1, True, None)]),
+    "b8_deep_k": (8, 3, 5, [(64, 0, 0, 0, None), (1024, 1, 1, True, None), (256, 1, 1, True, None), (256, 3, 1, True, None),
+                            (2048, 1, 1, True, None), (40, 1, 1, True, None)]),
+    "b24_three_images_per_share": (24, 3, 6, [(32, 0, 0, 0, None), (32, 3, 1, True, None), (64, 1, 1, True, None), (64, 3, 2, True, None),
+                                              (96, 1, 1, False, None)]),
+    "b8_many_tiles_two_rounds": (8, 3, 40, [(64, 0, 0, 0, None), (256, 1, 1, True, None), (64, 1, 1, True, None), (64, 3, 1, True, None),
+                                            (256, 1, 1, False, 1)]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CHAINS))
+def test_chain_of_convolutions_in_one_launch(name, dev):
+    n, c, hw, layers = CHAINS[name]
+    g, heads = _chain("seq-" + name, n, c, hw, layers)
+    _check(g, heads, "seq-" + name)
+
+
+@pytest.mark.parametrize("cfg", range(7))
+def test_every_configuration_of_the_tile_kernel_inside_a_sequence(cfg, dev):
+    """CVM_HIP_WAVECFG forces one configuration for every layer of the sequence (all three addressing modes occur)."""
+    g, heads = _chain("seq-cfg%d" % cfg, 8, 3, 12, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (128, 3, 2, True, None),
+                                                     (128, 1, 2, True, None), (256, 3, 1, False, None), (256, 1, 1, True, None)])
+    os.environ["CVM_HIP_WAVECFG"] = str(cfg)
+    try:
+        _check(g, heads, "seq-cfg%d" % cfg)
+    finally:
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+
+
+def test_resnet50_shrunk_batch16_and_resnet20_batch64(dev):
+    g, heads = graphgen.resnet50(16, width=32, size=64, classes=100, config_id="seq-r50")
+    _check(g, heads, "seq-r50")
+    g, heads = graphgen.resnet20_cifar(64)
+    _check(g, heads, "seq-r20", oracle_too=False)     # the oracle comparison of this model is in test_models_gpu.py
+
+
+def test_resnet50_full_size_batch16_equals_one_launch_per_layer(dev):
+    g, heads = graphgen.resnet50(16)
+    _check(g, heads, "seq-r50-full", oracle_too=False)   # image-wise oracle parity of this model: test_models_gpu.py
+
+
+def test_two_models_with_sequences_on_two_threads(dev):
+    """Two sequence launches must never be in flight at once; the runtime orders the runs of different models."""
+    import threading
+    g, heads = graphgen.resnet50(8, width=16, size=64, classes=50, config_id="seq-two")
+    js, pb = g.build(heads)
+    x = synth.tensor("seq-two", "data", (8, 3, 64, 64), -127, 127).astype(np.int8)
+    want = _run(js, pb, x, "0")
+    os.environ["CVM_HIP_SEQ"] = "1"
+    try:
+        models = [runtime.HipModel(js, pb) for _ in range(2)]
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+    results = [[], []]
+
+    def work(i):
+        for _ in range(20):
+            results[i].append(models[i].inference(x.tobytes()))
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for m in models:
+        m.close()
+    for i in range(2):
+        for out in results[i]:
+            assert np.array_equal(np.frombuffer(out, np.int32), want)
