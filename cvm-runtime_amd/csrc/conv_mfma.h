@@ -106,7 +106,7 @@ __host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c
 
 // Forced kernel choice of the calling thread (thread-local; automatic by default): which implicit-GEMM kernel,
 // which configuration of the wavefront kernel (-1 = automatic), which tile of the tiled kernel (0 = automatic).
-enum { CONV_KERNEL_AUTO = 0, CONV_KERNEL_LDS = 1, CONV_KERNEL_WAVE = 2 };
+enum { CONV_KERNEL_AUTO = 0, CONV_KERNEL_LDS = 1, CONV_KERNEL_WAVE = 2, CONV_KERNEL_BIG = 3 };
 struct ConvTuning { int kernel, wave_cfg, tile_wm, tile_wn; };
 void set_conv_tuning(const ConvTuning& t);
 

@@ -888,6 +888,252 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
 }
 
+// ---------------------------------------------------------------- large-tile kernel
+// Layers with enough output to fill the chip several times over (the 3x3 layers of a VGG) are bound by how
+// many operand bytes an MFMA needs, not by latency.  Here a workgroup of four wavefronts, one per SIMD,
+// owns a tile of up to 256 output channels x 256 pixels; each wavefront keeps a TM x TN block of 32x32
+// MFMA tiles (4x4: 256 accumulator registers), so the 8 fragments it reads from LDS per 32 bytes of K
+// feed 16 MFMAs.  Both operands reach LDS without passing through registers: global_load_lds_dwordx4
+// takes one global address per lane and writes lane l's 16 bytes to (LDS base + 16 l), which is exactly the
+// fragment order, so a wavefront gathers one 1 KiB fragment of the im2col matrix (padding taps read the
+// zero granule) or of the packed filter per instruction.  K advances 64 bytes per step through a ring of
+// NST stage buffers; a step is: wait until this wavefront's requests for the step have landed, one
+// s_barrier, request the step NST-1 ahead into the buffer everyone has just left, then 2 x (TM + TN)
+// ds_read_b128 and 2 x TM x TN MFMAs.  The barrier is the bare instruction and the waits are written by
+// hand: the fence that comes with __syncthreads would wait for every outstanding request, i.e. undo the ring.
+// One request: 16 bytes per lane from `gaddr` (any address per lane) to LDS byte lds_base + 16 * lane.  Written as
+// assembly on purpose: the compiler then neither counts these requests nor protects LDS reads against them (it would
+// wait for every outstanding one before the first ds_read of a step, which undoes the ring); the waits are wait_vm.
+__device__ __forceinline__ void lds_dma16(const void* gaddr, uint32_t lds_base) {
+  // (the s_nop is the wait state an instruction that reads M0 needs after a scalar write to it; inside inline assembly
+  // nobody inserts it for us)
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(lds_base) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int I, int TM, int TN, int OUT>
+__device__ __forceinline__ void big_epilogue_rows(v16i (&acc)[TM][TN], const int* sBias, int ch_wave, int oc0, int px_wave, int lane,
+                                                  void* out, const ConvGeom& g, const Epilogue& ep) {
+  if constexpr (I < TM) {
+    int32_t val[TN * 16];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) val[j * 16 + e] = acc[I][j][e];
+    uint32_t rp[TN * 4];
+    if (ep.residual) load_residual<TN, TN * 4>(rp, I * TN * 4, ch_wave, oc0, px_wave, lane, g, ep);
+    finish_groups<TN, TN * 4, OUT>(val, I * TN * 4, sBias, ch_wave, oc0, px_wave, lane, out, g, ep, rp);
+    big_epilogue_rows<I + 1, TM, TN, OUT>(acc, sBias, ch_wave, oc0, px_wave, lane, out, g, ep);
+  }
+}
+
+template <int WGM, int WGN, int TM, int TN, int OUT>
+__global__ void __launch_bounds__(256, (TM * TN <= 8 ? 2 : 1))
+k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out, const ConvGeom g, const Epilogue ep) {
+  static_assert(WGM * WGN == 4, "four wavefronts");
+  constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+  constexpr int NA = BM / 32, NB = BN / 32;               // 32-row blocks of the two operands
+  constexpr int AF = NA * 2, BF = NB * 2;                  // fragments per stage (two 32-byte chunks of K)
+  constexpr int STAGE = (AF + BF) * 1024;
+  constexpr int NST = TM * TN <= 8 ? 3 : (STAGE * 4 <= 147456 ? 4 : 3);   // two workgroups per CU share the LDS when the tile is small
+  constexpr int LA = AF / 4, LB = BF / 4;                  // requests per wavefront and stage
+  constexpr int LPW = LA + LB;
+  constexpr int PXW = NB / 4;                              // pixel blocks whose rows a wavefront gathers
+  static_assert(NB % 4 == 0 && AF % 4 == 0, "pixel blocks and filter fragments are dealt to the four wavefronts");
+  __shared__ __attribute__((aligned(16))) int8_t smem[NST * STAGE];
+  __shared__ __attribute__((aligned(16))) int sBias[BM];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  int pid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);   // contiguous tile runs per XCD
+  const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);
+  const int oc0 = (pid - ptile * g.octiles) * BM;
+  const int px0 = ptile * BN;
+  const int P = (int)g.P, OHW = g.OH * g.OW;
+  const int ctiles = g.Cp >> 5;
+  const int nch = g.Kp >> 5, nlive = (g.K + 31) >> 5;
+  const int nsteps = g.Kp >> 6;
+  const int last_ot = ((g.OC + 127) / 128) * 4 - 1;       // last 32-row block the packed filter holds
+
+  // ---- what this lane gathers: row (lane & 31) of PXW pixel blocks, bytes (lane >> 5) * 16 .. +15 of a chunk
+  int rowbase[PXW];
+  unsigned rowmask[PXW], colmask[PXW];
+#pragma unroll
+  for (int q = 0; q < PXW; ++q) {
+    const int p = px0 + (wave + 4 * q) * 32 + lrow;
+    const bool ok = p < P;
+    const unsigned pp = ok ? (unsigned)p : 0u;
+    const int n = (int)fastdiv(pp, g.div_ohw);
+    const int rem = (int)pp - n * OHW;
+    const int oh = (int)fastdiv((unsigned)rem, g.div_ow);
+    const int ow = rem - oh * g.OW;
+    const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
+    rowbase[q] = (n * g.H + ih0) * g.W + iw0;
+    unsigned rm, cm;
+    if (g.DH == 1 && g.DW == 1) {
+      rm = tap_mask_dense(ih0, g.H, g.KH);
+      cm = tap_mask_dense(iw0, g.W, g.KW);
+    } else {
+      rm = tap_mask_dilated(ih0, g.H, g.KH, g.DH);
+      cm = tap_mask_dilated(iw0, g.W, g.KW, g.DW);
+    }
+    rowmask[q] = ok ? rm : 0u;
+    colmask[q] = cm;
+  }
+  const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
+  typedef int8_t __attribute__((address_space(3))) * lptr_t;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)smem;   // LDS byte address of the ring
+
+  // ---- the request stream.  Stages are requested in order (the first NST - 1 before the loop, then one per step), so
+  // the position in K is kept as running state instead of being decoded per request: chunk, its channel block and
+  // filter tap (uniform), and per lane the address of the tap's granule for each pixel it gathers plus what one
+  // channel block adds to it -- 1 KiB inside the image, nothing for a padding tap, whose address is the zero granule.
+  // A request then costs one multiply-add per pixel; the address of a tap is worked out once per tap.  Requests past
+  // the end of K (the ring runs NST - 1 stages ahead) read the zero granule and the slack behind the filter.
+  int rq_cblk = 0, rq_r = 0, rq_s = 0, rq_tap = 0;
+  uint64_t tap_addr[PXW];
+  uint32_t tap_inc[PXW];
+  uint64_t flt_addr[LA];      // this lane's 16 bytes of the filter fragments the wavefront requests, at the current step
+#pragma unroll
+  for (int t = 0; t < LA; ++t) {
+    const int a = wave + 4 * t;                    // fragment (block a >> 1, chunk a & 1) of the filter
+    int ot = (oc0 >> 5) + (a >> 1);
+    ot = ot < last_ot ? ot : last_ot;              // blocks past the filter repeat its last one; their channels are never stored
+    flt_addr[t] = (uint64_t)(uintptr_t)wf + ((uint64_t)ot * (nch + 1) + (a & 1)) * 1024 + lane * 16;
+  }
+  // One stage is LPW requests: `prepare` works out their addresses and advances the stream, `issue(i)` sends the
+  // i-th.  They are sent one at a time between groups of MFMAs: a wavefront that sends a request is held until
+  // the CU's address unit has taken all 64 lanes of it (1 KiB at 64 bytes a clock, behind the requests of the
+  // other wavefronts), and eight of them back to back kept the MFMA pipes idle for longer than the MFMAs of a
+  // stage take.
+  uint64_t rq_addr[LPW];
+  uint32_t rq_lds[LPW];
+  auto prepare = [&](int slot) __attribute__((always_inline)) {
+    const uint32_t stage = lds_base + (uint32_t)(slot * STAGE);
+#pragma unroll
+    for (int t = 0; t < LA; ++t) {
+      const int a = wave + 4 * t;
+      rq_addr[t] = flt_addr[t];
+      rq_lds[t] = stage + (uint32_t)a * 1024u;
+      flt_addr[t] += 2048;
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      if (rq_cblk == 0) {       // a new tap (uniform, once per Cp / 32 chunks)
+        const bool tap_ok = rq_tap < g.taps;
+        const int soff = (rq_r * g.DH) * g.W + rq_s * g.DW;
+#pragma unroll
+        for (int q = 0; q < PXW; ++q) {
+          const int pin = rowbase[q] + soff;
+          const bool ok = tap_ok && ((((rowmask[q] >> rq_r) & (colmask[q] >> rq_s)) & 1u) != 0);
+          const unsigned off = __umul24((unsigned)pin >> 5, (unsigned)g.Cp << 5) + (((unsigned)pin & 31u) << 4) + (unsigned)(lgrp * 512);
+          const uint64_t inside = (uint64_t)(uintptr_t)xp + off, outside = (uint64_t)(uintptr_t)zero;
+          tap_addr[q] = outside ^ ((inside ^ outside) & (ok ? ~0ull : 0ull));
+          tap_inc[q] = ok ? 1024u : 0u;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < PXW; ++q) {
+        rq_addr[LA + c * PXW + q] = tap_addr[q];
+        tap_addr[q] += tap_inc[q];             // the next channel block of the tap
+        rq_lds[LA + c * PXW + q] = stage + (uint32_t)(AF + (wave + 4 * q) * 2 + c) * 1024u;
+      }
+      if (++rq_cblk == ctiles) {
+        rq_cblk = 0;
+        ++rq_tap;
+        if (++rq_s == g.KW) { rq_s = 0; ++rq_r; }
+      }
+    }
+  };
+  auto issue = [&](int i) __attribute__((always_inline)) {
+    lds_dma16(reinterpret_cast<const void*>((uintptr_t)rq_addr[i]), rq_lds[i]);
+  };
+
+  v16i acc[TM][TN];
+  const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = zero16;
+
+  // ---- the ring.  A step multiplies the fragments of its first chunk while those of its second chunk are read from
+  // LDS, then meets the other wavefronts once (its own requests for the next step have landed, it has read the last
+  // fragment of this step's slot), and multiplies the second chunk while the first chunk of the next step is read.
+  // The slot just left is refilled with the step NST ahead: H1 of its requests go out among the MFMAs of this
+  // step's second half, the other H2 among those of the next step's first half -- so LDS reads and requests always
+  // run under MFMAs, the requests one at a time, and there is one barrier per step.
+  constexpr int H1 = LPW / 2, H2 = LPW - H1, NM = TM * TN;
+  auto mfma_group = [&](const v4i (&fa)[TM], const v4i (&fb)[TN], int first, int count) __attribute__((always_inline)) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+      if (m >= first && m < first + count)
+        acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[m / TN], fb[m % TN], acc[m / TN][m % TN], 0, 0, 0);
+  };
+#pragma unroll
+  for (int st = 0; st < NST; ++st) {
+    prepare(st);
+#pragma unroll
+    for (int i = 0; i < (st < NST - 1 ? LPW : H1); ++i) issue(i);   // the last slot's other requests go out in the first step
+  }
+  stage_bias<BM>(sBias, ep, g.OC, oc0, tid);
+  v4i a0[TM], b0[TN], a1[TM], b1[TN];
+  wait_vm<(NST - 2) * LPW + H1>();
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a0[i] = *reinterpret_cast<const v4i*>(smem + ((wm * TM + i) * 2) * 1024 + lane * 16);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b0[j] = *reinterpret_cast<const v4i*>(smem + (AF + (wn * TN + j) * 2) * 1024 + lane * 16);
+  int slot = 0;
+  for (int kt = 0; kt < nsteps; ++kt) {
+    const int8_t* stage = smem + slot * STAGE;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a1[i] = *reinterpret_cast<const v4i*>(stage + ((wm * TM + i) * 2 + 1) * 1024 + lane * 16);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b1[j] = *reinterpret_cast<const v4i*>(stage + (AF + (wn * TN + j) * 2 + 1) * 1024 + lane * 16);
+    // first half: chunk 0, with the H2 requests still owed to the slot refilled in the previous step
+#pragma unroll
+    for (int r = 0; r < H2; ++r) {
+      issue(H1 + r);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_group(a0, b0, r * NM / H2, (r + 1) * NM / H2 - r * NM / H2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    prepare(slot);                                          // addresses of step kt + NST, which goes into the slot being left
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot has been read completely
+    wait_vm<(NST - 2) * LPW>();                             // own requests of the next step have landed
+    __builtin_amdgcn_s_barrier();
+    const int next = slot + 1 == NST ? 0 : slot + 1;
+    const int8_t* nstage = smem + next * STAGE;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a0[i] = *reinterpret_cast<const v4i*>(nstage + ((wm * TM + i) * 2) * 1024 + lane * 16);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b0[j] = *reinterpret_cast<const v4i*>(nstage + (AF + (wn * TN + j) * 2) * 1024 + lane * 16);
+    // second half: chunk 1, with the first H1 requests of the refill
+#pragma unroll
+    for (int r = 0; r < H1; ++r) {
+      issue(r);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_group(a1, b1, r * NM / H1, (r + 1) * NM / H1 - r * NM / H1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    slot = next;
+  }
+  wait_vm<0>();      // the requests that ran past the end of K
+  __syncthreads();   // bias staged (all requests have landed by now)
+
+  // ---- epilogue, one row of TN tiles at a time (the row index is a template argument: an accumulator indexed by a
+  // loop variable that the compiler does not unroll would be moved to scratch memory as a whole)
+  big_epilogue_rows<0, TM, TN, OUT>(acc, sBias, wm * TM * 32, oc0, px0 + wn * TN * 32, lane, out, g, ep);
+}
+
 // ---------------------------------------------------------------- layer-sequence kernel
 // A run of convolutions of one graph in ONE launch, for batches that divide over the chip's 8 XCDs.
 // Images are independent, so XCD x computes every layer for its own share of the images (pixel range
@@ -1452,6 +1698,31 @@ static int choose_wave_cfg(const ConvGeom& g, int cus = 256) {
   return last - 1;
 }
 
+// ---- large-tile kernel: tile shapes and choice
+struct BigCfg { int wgm, wgn, tm, tn; };
+static const BigCfg kBigCfgs[] = {{2, 2, 4, 4}, {2, 2, 2, 4}, {1, 4, 2, 4}};   // 256x256, 128x256, 64x512 (channels x pixels)
+static int64_t big_cfg_blocks(const BigCfg& c, const ConvGeom& g) {
+  const int bm = c.wgm * c.tm * 32, bn = c.wgn * c.tn * 32;
+  return (int64_t)((g.OC + bm - 1) / bm) * ((g.P + bn - 1) / bn);
+}
+// The largest tile that does not reach past the layer's channels and still gives most compute units a tile; -1 when
+// the layer is too small for this kernel (fewer than 160 tiles of the smallest fitting shape, or a short K).
+static int choose_big_cfg(const ConvGeom& g) {
+  if (g.dw || g.row_bytes || (g.Cp % 32) != 0 || g.KH > 32 || g.KW > 32 || g.K < 256) return -1;
+  // 128 x 256 tiles, two workgroups per compute unit, measured best (1.4-1.6 POP/s on the 3x3 layers of a VGG against
+  // 1.05-1.2 for the wavefront kernel); the 256 x 256 tile (one workgroup, 1.4) and the 64 x 512 one (0.65, below the
+  // wavefront kernel's 0.96 on 64 -> 64 channels) are kept for forced use
+  if (g.OC <= 64) return -1;
+  return big_cfg_blocks(kBigCfgs[1], g) >= 160 ? 1 : -1;
+}
+template <int OUT>
+static void launch_big_out(int cfg, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out, const ConvGeom& g,
+                           const Epilogue& ep) {
+  if (cfg == 0) k_conv_big<2, 2, 4, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  else if (cfg == 1) k_conv_big<2, 2, 2, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+  else k_conv_big<1, 4, 2, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+}
+
 static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out,
                         const ConvGeom& g, const Epilogue& ep) {
   switch (cfg) {
@@ -1617,6 +1888,28 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
       k_slices_finish<OUT_I32_NCHW><<<grid_for(total, 256), 256, 0, s>>>(reinterpret_cast<const int32_t*>(ws), out, kslices, g.slice_stride, g, ep);
     return check_launch("conv K-slice finish");
   }
+  // layers that fill the chip several times over: the large-tile kernel (CONV_KERNEL_BIG forces it where it applies,
+  // a forced wavefront or tiled kernel keeps it away)
+  {
+    const int big = (tune.kernel == CONV_KERNEL_AUTO || tune.kernel == CONV_KERNEL_BIG) && wave_forced < 0 ? choose_big_cfg(g) : -1;
+    int bcfg = big;
+    if (tune.kernel == CONV_KERNEL_BIG && bcfg < 0 && !g.dw && !rows && (g.Cp % 32) == 0 && g.KH <= 32 && g.KW <= 32)
+      bcfg = g.OC > 128 ? 0 : g.OC > 64 ? 1 : 2;   // forced: any size
+    if (tune.kernel == CONV_KERNEL_BIG && tune.tile_wm >= 1 && tune.tile_wm <= 3 && bcfg >= 0) bcfg = tune.tile_wm - 1;
+    if (bcfg >= 0 && kslices <= 1) {
+      const BigCfg& c = kBigCfgs[bcfg];
+      const int64_t nbig = big_cfg_blocks(c, g);
+      if (nbig > 0x7fffffff) return arg_error("conv grid too large");
+      g.octiles = (g.OC + c.wgm * c.tm * 32 - 1) / (c.wgm * c.tm * 32);
+      g.div_octiles = make_fastdiv((uint32_t)g.octiles);
+      const ConvDesc desc(g, ep, "big", bcfg, 0, (long)nbig);
+      KernelTimer timer("k_conv_big", 2.0 * (double)g.P * g.OC * (double)g.taps * (double)(g.C ? g.C : g.Cp), s, conv_bytes(g, ep),
+                        desc.text);
+      if (ep.out_mode == OUT_I8_ACT) launch_big_out<OUT_I8_ACT>(bcfg, (unsigned)nbig, s, xp, wp, out, g, ep);
+      else launch_big_out<OUT_I32_NCHW>(bcfg, (unsigned)nbig, s, xp, wp, out, g, ep);
+      return check_launch("conv_big");
+    }
+  }
   if (cfg >= 0) {
     const int mode = rows ? WAVE_ROWS
                           : (!g.dw && g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
@@ -1715,7 +2008,7 @@ using namespace cvmhip;
 extern "C" {
 
 int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn) {
-  if (kernel < CONV_KERNEL_AUTO || kernel > CONV_KERNEL_WAVE) return arg_error("set_conv_tuning kernel");
+  if (kernel < CONV_KERNEL_AUTO || kernel > CONV_KERNEL_BIG) return arg_error("set_conv_tuning kernel");
   set_conv_tuning(ConvTuning{kernel, wave_cfg, tile_wm, tile_wn});
   return CVMHIP_OK;
 }

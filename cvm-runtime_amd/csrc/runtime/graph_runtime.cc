@@ -451,7 +451,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
-  hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : 0;
+  hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : kind.rfind("b", 0) == 0 ? 3 : 0;
   if (!cfg.empty() && cfg[0] >= '0' && cfg[0] <= '9') hooks_.wave_cfg = std::atoi(cfg.c_str());
   if (tile.size() >= 3 && tile[1] == ',') {
     hooks_.tile_wm = tile[0] - '0';
@@ -682,25 +682,22 @@ void HipGraphRuntime::CalibrateSequences() {
 // ---------------------------------------------------------------- execution
 // A layer-sequence launch occupies every compute unit and waits, inside the kernel, for all of its workgroups:
 // two of them in flight at once (two models on two streams) could each hold part of the chip and wait for the
-// rest.  So a run that contains one starts only after the previous such run of this process has finished: the
-// stream waits for the event recorded behind that run.  Runs without sequence launches are not affected.
-// A single model needs none of this (its runs are ordered by its stream): the gate acts only while the process
-// holds more than one model with sequence launches.
+// rest.  So while the process holds more than one model with sequence launches, a run that contains one is
+// issued under a process-wide lock and the lock is kept until the stream has drained.  (Ordering the streams with
+// an event instead would leave the host free, but a wait on an event that another thread records while this
+// thread's stream is being captured is refused by the runtime.)  A single model needs none of this: its runs
+// are ordered by its stream.
 namespace {
 std::atomic<int> g_sequence_models{0};
 struct SequenceGate {
   static std::mutex& Mutex() { static std::mutex m; return m; }
-  static void*& Last() { static void* e = nullptr; return e; }
   void* stream;
   bool active;
   std::unique_lock<std::mutex> lock;
   explicit SequenceGate(void* s) : stream(s), active(g_sequence_models.load() > 1) {
-    if (!active) return;
-    lock = std::unique_lock<std::mutex>(Mutex());
-    if (Last()) HipCheck(cvmhip_stream_wait_event(stream, Last()), "sequence gate");
-    else HipCheck(cvmhip_event_create(&Last()), "sequence gate");
+    if (active) lock = std::unique_lock<std::mutex>(Mutex());
   }
-  ~SequenceGate() { if (active) cvmhip_event_record(Last(), stream); }
+  ~SequenceGate() { if (active) cvmhip_stream_sync(stream); }
 };
 }  // namespace
 

@@ -28,12 +28,13 @@ def _ptr(t):
 
 def _apply_conv_tuning():
     """The library never reads the environment on a launch; this glue turns the test hooks CVM_HIP_CONV
-    (lds | wave), CVM_HIP_WAVECFG (index) and CVM_HIP_TILE ("wm,wn") into the explicit per-thread setting."""
+    (lds | wave | big), CVM_HIP_WAVECFG (index) and CVM_HIP_TILE ("wm,wn"; with big: "t,0" picks tile t = 1..3)
+    into the explicit per-thread setting."""
     kind = os.environ.get("CVM_HIP_CONV", "")
     cfg = os.environ.get("CVM_HIP_WAVECFG", "")
     tile = os.environ.get("CVM_HIP_TILE", "")
     wm, wn = (int(tile[0]), int(tile[2])) if len(tile) >= 3 and tile[1] == "," else (0, 0)
-    check(lib().cvmhip_set_conv_tuning({"l": 1, "w": 2}.get(kind[:1], 0), int(cfg) if cfg.isdigit() else -1, wm, wn))
+    check(lib().cvmhip_set_conv_tuning({"l": 1, "w": 2, "b": 3}.get(kind[:1], 0), int(cfg) if cfg.isdigit() else -1, wm, wn))
 
 
 def _stream():

@@ -254,8 +254,9 @@ typedef struct {
 
 int cvmhip_pad_channels(int channels);
 /* Test and tuning hook: forces, for the calling thread's later convolution launches, the implicit-GEMM kernel
- * (0 automatic, 1 LDS-tiled, 2 wavefront-private), a configuration of the wavefront kernel (-1 automatic) and a
- * tile of the tiled kernel (wm, wn in 1..2; 0 automatic).  The library never reads the environment on a launch. */
+ * (0 automatic, 1 LDS-tiled, 2 wavefront-private, 3 large-tile wherever the layout allows it), a configuration of the
+ * wavefront kernel (-1 automatic) and a tile of the tiled kernel (wm, wn in 1..2; 0 automatic; with kernel 3, wm = 1..3
+ * picks the 256x256, 128x256 or 64x512 tile).  The library never reads the environment on a launch. */
 int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn);
 /* int32 NCHW <-> int8 act layout (narrowing is static_cast<int8_t>) */
 int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream);

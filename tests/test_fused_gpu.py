@@ -95,7 +95,7 @@ FUSED_CONV = [
 ]
 
 
-@pytest.fixture(params=["auto", "lds", "wave"])
+@pytest.fixture(params=["auto", "lds", "wave", "big"])
 def conv_kernel(request):
     """Both implicit-GEMM kernels must give the same bits: force each in turn (the library reads the hook per call)."""
     if request.param == "auto":
@@ -171,7 +171,7 @@ def test_conv2d_i8_random_geometries(case, dev):
         ref = run_chain(oracle.elemwise("elemwise_add", ref, r), ch2)
         res_t = hipops.pack_act_i8(T(r, dev))
     xp, wp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev))
-    for kind in ("lds", "wave"):
+    for kind in ("lds", "wave", "big"):
         os.environ["CVM_HIP_CONV"] = kind
         try:
             out = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1), res_t,
@@ -306,6 +306,48 @@ def test_conv_wave_kernel_every_configuration(case, cfg, dev):
         os.environ.pop("CVM_HIP_WAVECFG", None)
     eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), ref8, "wave cfg %d int8" % cfg)
     eq(out32.cpu().numpy(), conv, "wave cfg %d int32" % cfg)
+
+
+BIG_TILE_CASES = [
+    # n, ic, h, w, oc, k, stride, pad, dilation, bias
+    (2, 64, 20, 20, 160, 3, 1, 1, 1, True),     # channels past one 128-row tile, ragged pixel count
+    (1, 96, 17, 15, 300, 3, 1, 1, 1, True),     # 300 channels: blocks past the packed filter are repeated, never stored
+    (3, 32, 9, 9, 64, 5, 2, 2, 1, False),       # 25 taps over one channel block, stride 2
+    (1, 128, 12, 12, 128, 3, 1, 2, 2, True),    # dilated
+    (2, 256, 7, 7, 96, 1, 1, 0, 1, True),       # 1x1: eight channel blocks per tap
+    (1, 64, 33, 31, 40, 3, 1, 0, 1, True),      # no padding, few channels
+    (4, 160, 14, 14, 256, 3, 1, 1, 1, True),    # five channel blocks per tap (odd: a step of K straddles two taps)
+]
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("case", BIG_TILE_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%dd%d" % c[:9])
+def test_large_tile_kernel_every_tile(case, tile, dev):
+    """The large-tile kernel (operands through a ring of LDS stages filled by global -> LDS requests), forced for
+    layers of any size, for each of its three tiles: int8 output with a residual, and int32 output."""
+    n, ic, h, w, oc, k, st, pd, dl, bias = case
+    cid = "bigtile-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768) if bias else None
+    ch1, ch2 = [("cvm_right_shift", 8, 12)], [("relu",), ("cvm_right_shift", 8, 1)]
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (dl, dl), 1)
+    r = synth.tensor(cid, "r", conv.shape, -127, 127)
+    ref8 = run_chain(oracle.elemwise("elemwise_add", run_chain(conv, ch1), r), ch2)
+    xp, wp, rp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev)), hipops.pack_act_i8(T(r, dev))
+    os.environ["CVM_HIP_CONV"] = "big"
+    os.environ["CVM_HIP_TILE"] = "%d,0" % tile
+    try:
+        out8 = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1), rp,
+                                hipops.chain(*ch2), True, (st, st), (pd, pd), (dl, dl))
+        out32 = hipops.conv2d_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, None, None, None, False,
+                                 (st, st), (pd, pd), (dl, dl))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_CONV", None)
+        os.environ.pop("CVM_HIP_TILE", None)
+    eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), ref8, "large tile %d int8" % tile)
+    eq(out32.cpu().numpy(), conv, "large tile %d int32" % tile)
 
 
 DW_MFMA_CASES = [

@@ -124,10 +124,14 @@ def test_two_models_with_sequences_on_two_threads(dev):
     finally:
         os.environ.pop("CVM_HIP_SEQ", None)
     results = [[], []]
+    errors = []
 
     def work(i):
-        for _ in range(20):
-            results[i].append(models[i].inference(x.tobytes()))
+        try:
+            for _ in range(20):
+                results[i].append(models[i].inference(x.tobytes()))
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(repr(e))
     threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
     for t in threads:
         t.start()
@@ -135,6 +139,8 @@ def test_two_models_with_sequences_on_two_threads(dev):
         t.join()
     for m in models:
         m.close()
+    assert not errors, errors
     for i in range(2):
+        assert len(results[i]) == 20
         for out in results[i]:
             assert np.array_equal(np.frombuffer(out, np.int32), want)
