@@ -20,10 +20,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
-# HBM bytes per k_conv_wave launch of the batch-16 workload, from the FETCH_SIZE and WRITE_SIZE counter
-# passes summarised in profiles/k_conv_wave_resnet50_b16_traffic.txt (a counter pass cannot run inside
-# this program, so the figure is carried here; it is reported only for the workload it was measured on)
-TRAFFIC_BYTES_PER_LAUNCH = {("k_conv_wave", 16): 12.84e6}
+# HBM bytes per launch of the dominant kernel of a batch-16 workload, from the FETCH_SIZE and WRITE_SIZE counter
+# passes summarised in the named file under profiles/ (a counter pass cannot run inside this program, so the
+# figures are carried here; each is reported only for the workload and kernel it was measured on)
+TRAFFIC_BYTES_PER_LAUNCH = {
+    ("resnet50", "k_conv_seq", 16): (553.4e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt"),
+    ("vgg16", "k_conv_big", 16): (37.4e6, "profiles/k_conv_big_vgg16_b16_traffic.txt"),
+}
 
 
 def cpu_baseline(js1, pb1, x1, budget_s=20.0):
@@ -140,20 +143,27 @@ def layer_table(args, pkg, L, model, title):
     print("# durations: %s; sum %.1f us" % (source, sum(dur)))
     if empty_us is not None:
         print("# a launch that does nothing (256-byte copy kernel): %.2f us in the same trace" % empty_us)
-    print("# floors: ops / 5 POP/s, bytes / 8 TB/s; excess = duration - max(floors)")
-    print("%3s %-14s %-78s %8s %8s %7s %7s %7s %7s %7s" % ("#", "kernel", "launch", "GOP", "MB", "us", "mfma_us", "hbm_us", "TOP/s", "TB/s"))
+    print("# floors: ops / 5 POP/s, bytes / 8 TB/s, the launch that does nothing; excess = duration - the largest floor")
+    print("%3s %-14s %-78s %8s %8s %7s %7s %7s %7s %7s %7s" % ("#", "kernel", "launch", "GOP", "MB", "us", "mfma_us", "hbm_us", "TOP/s", "TB/s",
+                                                                "excess"))
     tot_ops = tot_bytes = 0.0
+    excess = []
     for i, (e, u) in enumerate(zip(step, dur)):
         is_conv = e["kernel"].startswith("k_conv")
         ops = e["work"] if is_conv else 0.0
         byts = e["bytes"] if is_conv else e["work"]
         tot_ops += ops
         tot_bytes += byts
-        print("%3d %-14s %-78s %8.3f %8.2f %7.2f %7.2f %7.2f %7.0f %7.2f" % (
+        floor = max(ops / 5e15 * 1e6, byts / 8e12 * 1e6, empty_us or 0.0)
+        excess.append((u - floor, i, e["kernel"], e["desc"]))
+        print("%3d %-14s %-78s %8.3f %8.2f %7.2f %7.2f %7.2f %7.0f %7.2f %7.2f" % (
             i, e["kernel"], e["desc"][:78], ops / 1e9, byts / 1e6, u, ops / 5e15 * 1e6, byts / 8e12 * 1e6,
-            ops / max(u, 1e-3) / 1e6, byts / max(u, 1e-3) / 1e6))
+            ops / max(u, 1e-3) / 1e6, byts / max(u, 1e-3) / 1e6, u - floor))
     print("# step: %.1f GOP = %.1f us at 5 POP/s; %.1f MB = %.1f us at 8 TB/s" % (
         tot_ops / 1e9, tot_ops / 5e15 * 1e6, tot_bytes / 1e6, tot_bytes / 8e12 * 1e6))
+    print("# sum of the floors %.1f us; the ten launches furthest above their floor:" % (sum(dur) - sum(x[0] for x in excess)))
+    for x in sorted(excess, reverse=True)[:10]:
+        print("#   %6.2f us  %3d %-14s %s" % (x[0], x[1], x[2], x[3][:78]))
 
 
 def main():
@@ -305,6 +315,7 @@ def main():
     all_ops = sum(v["work"] for v in convs.values())
     all_s = sum(v["ms"] / 1e3 - v["launches"] * pair_us["empty_us"] * 1e-6 for v in convs.values())
     step_s = wall / args.steps
+    traffic = TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dom, args.batch), (None, None))
     line = {
         "metric": "images/sec int8 %s, one MI355X, input resident in HBM" % names[args.workload],
         "value": args.batch / step_s,
@@ -329,10 +340,9 @@ def main():
                    "output_checksum": int(np.bitwise_xor.reduce(out.view(np.uint32)))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_I8_TOPS, "unit": "TOP/s",
                      "frac": achieved / PEAK_I8_TOPS,
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((dom, args.batch)) if args.workload == "resnet50" else None,
-                     "traffic_unit": "bytes per launch",
-                     "traffic_source": "recorded from the FETCH_SIZE / WRITE_SIZE counter passes summarised in "
-                                       "profiles/k_conv_wave_resnet50_b16_traffic.txt, not measured by this run",
+                     "traffic": traffic[0], "traffic_unit": "bytes per launch",
+                     "traffic_source": ("recorded from the FETCH_SIZE / WRITE_SIZE counter passes summarised in "
+                                        + traffic[1] + ", not measured by this run") if traffic[0] else None,
                      "kernel": dom, "launches_per_step": conv["launches"] / args.steps,
                      "avg_launch_us": avg_s * 1e6, "avg_launch_us_with_event_pair": raw_avg_s * 1e6,
                      "event_pair_cost_us": pair_cost_us, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
