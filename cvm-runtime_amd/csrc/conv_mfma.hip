@@ -1016,7 +1016,7 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   // stage take.
   uint64_t rq_addr[LPW];
   uint32_t rq_lds[LPW];
-  auto prepare = [&](int slot) __attribute__((always_inline)) {
+  auto prepare_filter = [&](int slot) __attribute__((always_inline)) {
     const uint32_t stage = lds_base + (uint32_t)(slot * STAGE);
 #pragma unroll
     for (int t = 0; t < LA; ++t) {
@@ -1025,8 +1025,10 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
       rq_lds[t] = stage + (uint32_t)a * 1024u;
       flt_addr[t] += 2048;
     }
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
+  };
+  auto prepare_chunk = [&](int slot, int c) __attribute__((always_inline)) {
+    const uint32_t stage = lds_base + (uint32_t)(slot * STAGE);
+    {
       if (rq_cblk == 0) {       // a new tap (uniform, once per Cp / 32 chunks)
         const bool tap_ok = rq_tap < g.taps;
         const int soff = (rq_r * g.DH) * g.W + rq_s * g.DW;
@@ -1053,6 +1055,11 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
       }
     }
   };
+  auto prepare = [&](int slot) __attribute__((always_inline)) {
+    prepare_filter(slot);
+    prepare_chunk(slot, 0);
+    prepare_chunk(slot, 1);
+  };
   auto issue = [&](int i) __attribute__((always_inline)) {
     lds_dma16(reinterpret_cast<const void*>((uintptr_t)rq_addr[i]), rq_lds[i]);
   };
@@ -1067,16 +1074,15 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   // ---- the ring.  A step multiplies the fragments of its first chunk while those of its second chunk are read from
   // LDS, then meets the other wavefronts once (its own requests for the next step have landed, it has read the last
   // fragment of this step's slot), and multiplies the second chunk while the first chunk of the next step is read.
-  // The slot just left is refilled with the step NST ahead: H1 of its requests go out among the MFMAs of this
-  // step's second half, the other H2 among those of the next step's first half -- so LDS reads and requests always
-  // run under MFMAs, the requests one at a time, and there is one barrier per step.
+  // The slot just left is refilled with the step NST ahead: H1 of its requests go out during this step's second
+  // half, the other H2 during the next step's first half.  Everything that is not an MFMA -- an LDS read, a
+  // request, a piece of the address arithmetic -- is placed behind one particular MFMA, a few instructions at a
+  // time: a wavefront issues in order, an MFMA keeps the matrix pipe busy for 32 clocks, and only what is issued
+  // inside those 32 clocks is free.  (In blocks between groups of MFMAs the same instructions left the pipe idle
+  // for half of a step when the workgroup had the CU to itself.)
   constexpr int H1 = LPW / 2, H2 = LPW - H1, NM = TM * TN;
-  auto mfma_group = [&](const v4i (&fa)[TM], const v4i (&fb)[TN], int first, int count) __attribute__((always_inline)) {
-#pragma unroll
-    for (int m = 0; m < NM; ++m)
-      if (m >= first && m < first + count)
-        acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[m / TN], fb[m % TN], acc[m / TN][m % TN], 0, 0, 0);
-  };
+  static_assert(H2 <= NM - 3 && TM + TN <= NM, "a half step has an MFMA for every request, LDS read and piece of address arithmetic");
+  auto lds16 = [&](const int8_t* p) __attribute__((always_inline)) { return *reinterpret_cast<const v4i*>(p + lane * 16); };
 #pragma unroll
   for (int st = 0; st < NST; ++st) {
     prepare(st);
@@ -1088,40 +1094,41 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   wait_vm<(NST - 2) * LPW + H1>();
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int i = 0; i < TM; ++i) a0[i] = *reinterpret_cast<const v4i*>(smem + ((wm * TM + i) * 2) * 1024 + lane * 16);
+  for (int i = 0; i < TM; ++i) a0[i] = lds16(smem + ((wm * TM + i) * 2) * 1024);
 #pragma unroll
-  for (int j = 0; j < TN; ++j) b0[j] = *reinterpret_cast<const v4i*>(smem + (AF + (wn * TN + j) * 2) * 1024 + lane * 16);
+  for (int j = 0; j < TN; ++j) b0[j] = lds16(smem + (AF + (wn * TN + j) * 2) * 1024);
   int slot = 0;
   for (int kt = 0; kt < nsteps; ++kt) {
     const int8_t* stage = smem + slot * STAGE;
+    // first half: chunk 0; behind its MFMAs the reads of chunk 1, the H2 requests still owed to the slot refilled in
+    // the previous step, and then the addresses of step kt + NST, which goes into the slot being left
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a1[i] = *reinterpret_cast<const v4i*>(stage + ((wm * TM + i) * 2 + 1) * 1024 + lane * 16);
+    for (int m = 0; m < NM; ++m) {
+      acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0[m / TN], b0[m % TN], acc[m / TN][m % TN], 0, 0, 0);
+      if (m < TM) a1[m] = lds16(stage + ((wm * TM + m) * 2 + 1) * 1024);
+      else if (m < TM + TN) b1[m - TM] = lds16(stage + (AF + (wn * TN + (m - TM)) * 2 + 1) * 1024);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) b1[j] = *reinterpret_cast<const v4i*>(stage + (AF + (wn * TN + j) * 2 + 1) * 1024 + lane * 16);
-    // first half: chunk 0, with the H2 requests still owed to the slot refilled in the previous step
-#pragma unroll
-    for (int r = 0; r < H2; ++r) {
-      issue(H1 + r);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_group(a0, b0, r * NM / H2, (r + 1) * NM / H2 - r * NM / H2);
+      for (int r = 0; r < H2; ++r)
+        if (m == r * (NM - 3) / H2) issue(H1 + r);
+      if (m == NM - 3) prepare_filter(slot);
+      if (m == NM - 2) prepare_chunk(slot, 0);
+      if (m == NM - 1) prepare_chunk(slot, 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    prepare(slot);                                          // addresses of step kt + NST, which goes into the slot being left
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot has been read completely
     wait_vm<(NST - 2) * LPW>();                             // own requests of the next step have landed
     __builtin_amdgcn_s_barrier();
     const int next = slot + 1 == NST ? 0 : slot + 1;
     const int8_t* nstage = smem + next * STAGE;
+    // second half: chunk 1; behind its MFMAs the reads of the next step's chunk 0 and the first H1 requests of the refill
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a0[i] = *reinterpret_cast<const v4i*>(nstage + ((wm * TM + i) * 2) * 1024 + lane * 16);
+    for (int m = 0; m < NM; ++m) {
+      acc[m / TN][m % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1[m / TN], b1[m % TN], acc[m / TN][m % TN], 0, 0, 0);
+      if (m < TM) a0[m] = lds16(nstage + ((wm * TM + m) * 2) * 1024);
+      else if (m < TM + TN) b0[m - TM] = lds16(nstage + (AF + (wn * TN + (m - TM)) * 2) * 1024);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) b0[j] = *reinterpret_cast<const v4i*>(nstage + (AF + (wn * TN + j) * 2) * 1024 + lane * 16);
-    // second half: chunk 1, with the first H1 requests of the refill
-#pragma unroll
-    for (int r = 0; r < H1; ++r) {
-      issue(r);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_group(a1, b1, r * NM / H1, (r + 1) * NM / H1 - r * NM / H1);
+      for (int r = 0; r < H1; ++r)
+        if (m == r * NM / H1) issue(r);
       __builtin_amdgcn_sched_barrier(0);
     }
     slot = next;
