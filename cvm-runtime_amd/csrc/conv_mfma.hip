@@ -814,8 +814,14 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // front of the first operand request).
   if (!COH && ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
   regs_t R0 = fetch(COH);
+  // Without a K split no wavefront needs anything from another one, so each stages its own copy of the bias in its
+  // own part of sBias and the tile needs no barrier at all: the wavefronts of a workgroup drift apart, and one's
+  // epilogue runs under another's operand requests (with a barrier per tile they all wait for memory together
+  // and then all do arithmetic together).
   int bias_mine = 0;
-  if (tid < BM) bias_mine = (ep.bias && oc0 + tid < g.OC) ? ep.bias[oc0 + tid] : 0;
+  const int bias_lane = KSPLIT == 1 ? lane : tid;
+  if (bias_lane < BM) bias_mine = (ep.bias && oc0 + bias_lane < g.OC) ? ep.bias[oc0 + bias_lane] : 0;
+  int* bias_lds = KSPLIT == 1 ? sBias + wave * BM : sBias;
 
   if (niter <= 1) {
     // the whole K range is one batch (a 1x1 layer over 64 channels): no second request.  Every byte a
@@ -833,7 +839,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       consume(R0, false);
     }
   }
-  if (tid < BM) sBias[tid] = bias_mine;
+  if (bias_lane < BM) bias_lds[bias_lane] = bias_mine;
 
   // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
   // wavefront kw_ then finalises the groups kw_*NU .. kw_*NU + NU-1 of the tile set
@@ -862,7 +868,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
     }
   } else {
-    __syncthreads();   // bias staged
+    __builtin_amdgcn_wave_barrier();   // bias staged: written and read by this wavefront only, and LDS serves a wavefront in order
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -872,7 +878,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   }
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, sBias, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
+  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
 }
 
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
@@ -881,7 +887,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
             const ConvGeom g, const Epilogue ep) {
   constexpr int U = TM * TN * 4;
   __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
-  __shared__ __attribute__((aligned(16))) int sBias[32 * TM];
+  __shared__ __attribute__((aligned(16))) int sBias[32 * TM * (KSPLIT == 1 ? NW : 1)];
   int pid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
@@ -1181,9 +1187,9 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
   for (int base = 0; base < ntiles; base += SEQ_WG_PER_SHARE * UNITS) {
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
     conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
-                                                                         sPart + half * 16384, sBias + half * 64, p_begin, p_end,
+                                                                         sPart + half * 16384, sBias + half * 256, p_begin, p_end,
                                                                          base == 0 ? gate : LayerGate{nullptr, 0, nullptr, 0});
-    __syncthreads();   // the next tile reuses the LDS
+    if (KSPLIT > 1) __syncthreads();   // the next tile reuses the LDS of the partial sums
   }
 }
 
@@ -1205,7 +1211,7 @@ __device__ __forceinline__ void seq_layer_cfg(int cfg, const int8_t* xp, const i
 __global__ void __launch_bounds__(512, 1)
 k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit) {
   __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: one 8-wavefront tile set or two 4-wavefront ones
-  __shared__ __attribute__((aligned(16))) int sBias[128];
+  __shared__ __attribute__((aligned(16))) int sBias[512];    // per half: one copy, or one per wavefront of an unsplit tile
   __shared__ int s_rank;
   // The current layer's table entry lives in LDS, where any field is a short read away wherever the code needs
   // it (a copy in registers would hold ~100 scalar registers for the whole layer, and reading it from memory
