@@ -693,7 +693,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   auto pass_gate = [&]() __attribute__((always_inline)) {
     if constexpr (COH) {
       gate_wait(gate);
-      if (ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
     }
   };
   auto fetch = [&](const bool gated) __attribute__((always_inline)) -> regs_t {
@@ -823,13 +822,22 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   if (bias_lane < BM) bias_mine = (ep.bias && oc0 + bias_lane < g.OC) ? ep.bias[oc0 + bias_lane] : 0;
   int* bias_lds = KSPLIT == 1 ? sBias + wave * BM : sBias;
 
+  // (COH) the residual is not needed before the epilogue: requested behind the operand batches that are in flight
+  // at the start, it does not stand between the layer boundary and the first MFMA
+  auto residual_coh = [&]() __attribute__((always_inline)) {
+    if constexpr (COH) {
+      if (ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
+    }
+  };
   if (niter <= 1) {
     // the whole K range is one batch (a 1x1 layer over 64 channels): no second request.  Every byte a
     // wavefront asks for, used or not, takes its turn in the CU's memory pipeline, and these layers are
     // bound by exactly that.
+    residual_coh();
     consume(R0, true);
   } else {
     regs_t R1 = fetch(false);
+    residual_coh();
     consume(R0, true);
     for (int it = 1; it < niter; it += 2) {
       R0 = fetch(false);
