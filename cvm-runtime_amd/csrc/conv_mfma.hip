@@ -120,6 +120,11 @@ constexpr unsigned kOutsideBuffer = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t act_rsrc(const void* base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
 }
+template <bool COH>
+__device__ __forceinline__ int4 ld16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off) {
+  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, COH ? 16 : 0);
+  return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
+}
 __device__ __forceinline__ int4 ld16_l2(__amdgpu_buffer_rsrc_t rs, unsigned off) {
   const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 16 /* sc1: device scope */);
   return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
@@ -601,11 +606,10 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
   const int P = (int)g.P;
-  __amdgpu_buffer_rsrc_t rs_x = act_rsrc(xp);   // only used by the COH form
+  __amdgpu_buffer_rsrc_t rs_x = act_rsrc(xp);   // activations are read through a buffer descriptor: 32-bit offsets, zeros past the end
 
   // ---- per-lane operand addressing
-  const int8_t* xb[TN];                    // WAVE_IDENT: block base + lane * 16
-  unsigned xoff[TN];                       //   ... the same as a byte offset from xp (COH)
+  unsigned xoff[TN];                       // WAVE_IDENT: byte offset (from xp) of the block's row of this lane
   int rowbase[TN];                         // otherwise: linear index of the first input pixel of the receptive field
   unsigned rowmask[TN], colmask[TN];       // WAVE_PAD: filter rows / columns inside the image
 #pragma unroll
@@ -614,7 +618,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       int t = (px0 >> 5) + pw_ * TN + (j ^ Xj);
       const int last = (P - 1) >> 5;
       t = t < last ? t : last;             // blocks past the tensor re-read its last block; their pixels are never stored
-      xb[j] = xp + (int64_t)t * ctiles * 1024 + lane * 16;
       xoff[j] = (unsigned)t * (unsigned)(ctiles * 1024) + (unsigned)lane * 16u;
       rowbase[j] = 0; rowmask[j] = 0; colmask[j] = 0;
     } else {
@@ -628,7 +631,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
       rowbase[j] = (n * g.H + ih0) * g.W + iw0;
       if (MODE == WAVE_ROWS) rowbase[j] *= 4;   // byte offset of the window of filter row 0 (g.H, g.W: stored size, no padding left)
-      xb[j] = xp;
       xoff[j] = 0;
       unsigned rm = 0, cm = 0;
       if (MODE == WAVE_PAD) {
@@ -672,14 +674,12 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   const int8_t* wa[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + (i ^ Xi)) * (nch + 1)) * 1024 + (lane ^ (Q << 3)) * 16;
-  const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
   const int lconst = lgrp * 512;
-  const int8_t* tapptr[TN];                // per-lane operand address of the current filter tap
-  unsigned tapoff[TN];                     //   ... as a byte offset from xp, kOutsideBuffer for a tap outside the image (COH)
-  int okv[TN];                             // 0: the lane reads the zero granule for this tap
+  unsigned tapoff[TN];                     // per-lane byte offset (from xp) of the current filter tap's granule; kOutsideBuffer
+                                           // for a tap outside the image: a buffer load past the end reads zeros
   bool need_tap = true;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) { tapptr[j] = zero; tapoff[j] = kOutsideBuffer; okv[j] = 0; }
+  for (int j = 0; j < TN; ++j) tapoff[j] = kOutsideBuffer;
 
   v16i acc[TM][TN];   // first written by the first MFMA of each tile, whose addend is the constant 0
 
@@ -719,8 +719,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-          if constexpr (COH) put(R, (d * (TM + TN) + TM + j) * 4, ld16_l2(rs_x, xoff[j] + (unsigned)cb[d] * 1024u));
-          else put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(xb[j] + (int64_t)cb[d] * 1024));
+          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, xoff[j] + (unsigned)cb[d] * 1024u));
         }
       cur = cur + D < c_end ? cur + D : c_end;
       return R;
@@ -754,18 +753,14 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
             // tap outside the image the offset is meaningless and the select below discards it -- a select, not
             // a branch, so that the two pointers cost a dozen instructions per tap instead of fifty.
             const unsigned off = __umul24((unsigned)pin >> 5, (unsigned)g.Cp << 5) + (((unsigned)pin & 31u) << 4) + (unsigned)lconst;
-            const int8_t* inside = xp + off;
-            tapptr[j] = ok ? inside : zero;
             tapoff[j] = ok ? off : kOutsideBuffer;
-            okv[j] = ok ? 1 : 0;
           }
           need_tap = false;
         }
         const int coff = live ? ((ch + ch_first) >> 5) * 1024 : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          if constexpr (COH) put(R, (d * (TM + TN) + TM + j) * 4, ld16_l2(rs_x, tapoff[j] + (unsigned)coff));
-          else put(R, (d * (TM + TN) + TM + j) * 4, *reinterpret_cast<const int4*>(tapptr[j] + (okv[j] ? coff : 0)));
+          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, tapoff[j] + (unsigned)coff));
         }
       }
       if (live) {
@@ -1822,7 +1817,8 @@ static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom&
   g.K = g.row_bytes ? g.KH * g.row_bytes : g.dw ? g.taps * 32 : g.taps * g.Cp;
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
-  if ((int64_t)g.N * g.H * g.W * g.Cp > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
+  // operands are addressed with 32-bit offsets from the tensor's base
+  if (act_bytes((int64_t)g.N * g.H * g.W, g.Cp) > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
   ep = ep_in;
   ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
   if (ep.o32_img == 0 && ep.o32_ch == 0 && ep.o32_px == 0) {  // int32 output defaults to NCHW
