@@ -120,9 +120,11 @@ constexpr unsigned kOutsideBuffer = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t act_rsrc(const void* base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
 }
+// `off` is the lane's own offset (the one the descriptor's range check sees), `uni` a wave-uniform one that the
+// instruction adds from a scalar register: it costs no vector instruction
 template <bool COH>
-__device__ __forceinline__ int4 ld16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off) {
-  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, COH ? 16 : 0);
+__device__ __forceinline__ int4 ld16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned uni = 0) {
+  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)uni, COH ? 16 : 0);
   return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
 }
 __device__ __forceinline__ int4 ld16_l2(__amdgpu_buffer_rsrc_t rs, unsigned off) {
@@ -671,9 +673,10 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   const int cp_k = g.dw ? 32 : g.Cp;       // channels of one tap in K
   const int ch_first = g.dw ? oc0 : 0;     // first input channel this workgroup reads
 
-  const int8_t* wa[TM];
+  const __amdgpu_buffer_rsrc_t rs_w = act_rsrc(wf);   // the packed filter is smaller than 2^31 bytes (checked by the host)
+  unsigned wa[TM];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) wa[i] = wf + ((int64_t)(oc0 / 32 + (i ^ Xi)) * (nch + 1)) * 1024 + (lane ^ (Q << 3)) * 16;
+  for (int i = 0; i < TM; ++i) wa[i] = (unsigned)(oc0 / 32 + (i ^ Xi)) * (unsigned)(nch + 1) * 1024u + (unsigned)((lane ^ (Q << 3)) * 16);
   const int lconst = lgrp * 512;
   unsigned tapoff[TN];                     // per-lane byte offset (from xp) of the current filter tap's granule; kOutsideBuffer
                                            // for a tap outside the image: a buffer load past the end reads zeros
@@ -713,13 +716,13 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)ca[d] * 1024));
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, ld16_buf<false>(rs_w, wa[i], (unsigned)ca[d] * 1024u));
       if (gated) pass_gate();
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, xoff[j] + (unsigned)cb[d] * 1024u));
+          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, xoff[j], (unsigned)cb[d] * 1024u));
         }
       cur = cur + D < c_end ? cur + D : c_end;
       return R;
@@ -730,7 +733,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       // a chunk past the end multiplies the all-zero filter chunk with a valid activation address
       const int chunk = live ? cur : nch;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, *reinterpret_cast<const int4*>(wa[i] + (int64_t)chunk * 1024));
+      for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, ld16_buf<false>(rs_w, wa[i], (unsigned)chunk * 1024u));
       if (gated && d == 0) pass_gate();
       if (MODE == WAVE_ROWS) {
         // 16-byte unit k16 of K: filter row k16 / (row_bytes/16), part k16 % (row_bytes/16) of its window
@@ -760,7 +763,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
         const int coff = live ? ((ch + ch_first) >> 5) * 1024 : 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, tapoff[j] + (unsigned)coff));
+          put(R, (d * (TM + TN) + TM + j) * 4, ld16_buf<COH>(rs_x, tapoff[j], (unsigned)coff));
         }
       }
       if (live) {
@@ -1818,7 +1821,9 @@ static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom&
   g.Kp = (g.K + KSTEP - 1) / KSTEP * KSTEP;
   g.P = (int64_t)g.N * g.OH * g.OW;
   // operands are addressed with 32-bit offsets from the tensor's base
-  if (act_bytes((int64_t)g.N * g.H * g.W, g.Cp) > INT32_MAX || g.P > INT32_MAX) return arg_error("conv tensor too large");
+  if (act_bytes((int64_t)g.N * g.H * g.W, g.Cp) > INT32_MAX || g.P > INT32_MAX ||
+      (int64_t)((g.OC + 127) / 128 * 4) * (g.Kp / 32 + 1) * 1024 > INT32_MAX)
+    return arg_error("conv tensor too large");
   ep = ep_in;
   ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
   if (ep.o32_img == 0 && ep.o32_ch == 0 && ep.o32_px == 0) {  // int32 output defaults to NCHW
