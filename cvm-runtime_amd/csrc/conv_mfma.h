@@ -104,6 +104,50 @@ __host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c
   }
 }
 
+// ---- max_pool2d on int8 activations: one 16-byte granule (16 channels of one output pixel).  The window's taps are
+// all requested before the first one is used (KH, KW are compile-time: with a loop over a run-time window every
+// tap waits for its own trip to memory, nine in a row for a 3x3 window).  A tap outside the image reads the nearest
+// pixel inside it instead, which belongs to the same window because every window touches the image (checked by the
+// host), so it changes no maximum and the loads need no predicate.  Bytes are compared two at a time as 16-bit
+// lanes (even bytes shifted up, odd bytes in place, low halves zero: the order of the signed bytes is kept).
+#if defined(__HIPCC__)
+typedef short pool_v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pool_max16(uint32_t a, uint32_t b) {
+  const pool_v2s r = __builtin_elementwise_max(__builtin_bit_cast(pool_v2s, a), __builtin_bit_cast(pool_v2s, b));
+  return __builtin_bit_cast(uint32_t, r);
+}
+template <int KH, int KW, typename Load>
+__device__ __forceinline__ void max_pool_request(int4 (&v)[KH * KW], Load load, int n, int p, int q, int c0, int cp, int h, int w, int sh,
+                                                 int sw, int ph, int pw) {
+#pragma unroll
+  for (int r = 0; r < KH; ++r) {
+    int ih = p * sh + r - ph;
+    ih = ih < 0 ? 0 : (ih > h - 1 ? h - 1 : ih);
+#pragma unroll
+    for (int c = 0; c < KW; ++c) {
+      int iw = q * sw + c - pw;
+      iw = iw < 0 ? 0 : (iw > w - 1 ? w - 1 : iw);
+      v[r * KW + c] = load(act_offset((int64_t)(n * h + ih) * w + iw, c0, cp));
+    }
+  }
+}
+template <int NT>
+__device__ __forceinline__ int4 max_pool_reduce(const int4 (&v)[NT]) {
+  uint32_t ev[4], od[4];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const uint32_t d[4] = {(uint32_t)v[t].x, (uint32_t)v[t].y, (uint32_t)v[t].z, (uint32_t)v[t].w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t e = (d[k] << 8) & 0xff00ff00u, o = d[k] & 0xff00ff00u;
+      ev[k] = t == 0 ? e : pool_max16(ev[k], e);
+      od[k] = t == 0 ? o : pool_max16(od[k], o);
+    }
+  }
+  return make_int4((int)(od[0] | (ev[0] >> 8)), (int)(od[1] | (ev[1] >> 8)), (int)(od[2] | (ev[2] >> 8)), (int)(od[3] | (ev[3] >> 8)));
+}
+#endif
+
 // Forced kernel choice of the calling thread (thread-local; automatic by default): which implicit-GEMM kernel,
 // which configuration of the wavefront kernel (-1 = automatic), which tile of the tiled kernel (0 = automatic).
 enum { CONV_KERNEL_AUTO = 0, CONV_KERNEL_LDS = 1, CONV_KERNEL_WAVE = 2, CONV_KERNEL_BIG = 3 };

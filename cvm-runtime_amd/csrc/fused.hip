@@ -75,10 +75,38 @@ k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t 
 }
 
 // max_pool2d for Cp >= 16: one thread per 16 channels of one output pixel (16-byte loads and stores)
+// The common windows (KH, KW > 0: 3x3 and 2x2): every tap of a granule requested before the first is used, G granules
+// per thread in flight (see max_pool_request); KH = 0: any window, tap by tap.
+template <int KH, int KW>
 __global__ void __launch_bounds__(256)
 k_max_pool_i8x16(const int8_t* __restrict__ x, int8_t* __restrict__ y, int64_t total, int64_t npix_out, int cp, int h,
                  int w, int oh, int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  if constexpr (KH > 0) {
+    constexpr int G = 2;
+    auto load = [&](int64_t off) __attribute__((always_inline)) { return *reinterpret_cast<const int4*>(x + off); };
+    for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < total; i0 += G * stride) {
+      int4 v[G][KH * KW];
+      bool ok[G];
+#pragma unroll
+      for (int k = 0; k < G; ++k) {
+        const int64_t i = i0 + k * stride;
+        int64_t t;
+        int c0;
+        act_decode((i < total ? i : i0) * 4, cp, &t, &c0);
+        ok[k] = i < total && t < npix_out;
+        if (t >= npix_out) t = npix_out - 1;
+        const int q = (int)(t % ow);
+        t /= ow;
+        const int p = (int)(t % oh);
+        max_pool_request<KH, KW>(v[k], load, (int)(t / oh), p, q, c0, cp, h, w, sh, sw, ph, pw);
+      }
+#pragma unroll
+      for (int k = 0; k < G; ++k)
+        if (ok[k]) *reinterpret_cast<int4*>(y + (i0 + k * stride) * 16) = max_pool_reduce<KH * KW>(v[k]);
+    }
+    return;
+  }
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
     int64_t t;
     int c0;
@@ -112,24 +140,34 @@ k_max_pool_i8x16(const int8_t* __restrict__ x, int8_t* __restrict__ y, int64_t t
 }
 
 // out[n][c] = chain(sum_hw x[n][hw][c]); the result is a tensor of n "pixels"
-// Eight consecutive lanes share one output dword (4 channels of one image): each
-// sums every eighth pixel, a butterfly over the 8 lanes adds the parts.
+// Sixteen consecutive lanes share one output dword (4 channels of one image): each sums every sixteenth pixel,
+// four requests at a time (a lane's requests would otherwise wait for one another: the layer is a handful of
+// round trips to memory and nothing else), and a butterfly over the 16 lanes adds the parts.
+constexpr int SUM_LANES = 16;
 __global__ void __launch_bounds__(256)
 k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i8, int64_t total, int nimg, int c, int cp,
             int hw, DevChain chain) {
-  const int64_t stride = ((int64_t)gridDim.x * blockDim.x) >> 3;
-  const int part = threadIdx.x & 7;
-  // all 8 lanes of a group run the same number of iterations (total is rounded up by the launch)
-  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 3; i < total; i += stride) {
+  const int64_t stride = ((int64_t)gridDim.x * blockDim.x) / SUM_LANES;
+  const int part = threadIdx.x & (SUM_LANES - 1);
+  // all lanes of a group run the same number of iterations (total is rounded up by the launch)
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SUM_LANES; i < total; i += stride) {
     int64_t n;
     int c0;
     act_decode(i, cp, &n, &c0);
     int32_t acc[4] = {0, 0, 0, 0};
     if (n < nimg) {
-      for (int t = part; t < hw; t += 8) {
-        const uint32_t v = x[act_offset(n * hw + t, c0, cp) >> 2];
+      for (int t = part; t < hw; t += 4 * SUM_LANES) {
+        uint32_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += byte_of(v, e);
+        for (int k = 0; k < 4; ++k) {
+          const int tt = t + SUM_LANES * k;
+          v[k] = x[act_offset(n * hw + (tt < hw ? tt : t), c0, cp) >> 2];
+          if (tt >= hw) v[k] = 0;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] += byte_of(v[k], e);
       }
     }
 #pragma unroll
@@ -137,6 +175,7 @@ k_sum_hw_i8(const uint32_t* __restrict__ x, void* __restrict__ out, int out_is_i
       acc[e] += __shfl_xor(acc[e], 1, 64);
       acc[e] += __shfl_xor(acc[e], 2, 64);
       acc[e] += __shfl_xor(acc[e], 4, 64);
+      acc[e] += __shfl_xor(acc[e], 8, 64);
     }
     if (part != 0 || n >= nimg) continue;
 #pragma unroll
@@ -474,9 +513,19 @@ int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, i
   KernelTimer timer("k_max_pool_i8", (double)n * c * ((double)h * w + (double)oh * ow), s);
   if (cp >= 16) {
     if (((uintptr_t)xp | (uintptr_t)yp) & 15) return arg_error("max_pool2d_i8 alignment");
-    k_max_pool_i8x16<<<grid_for(total / 4, 256, 1 << 16), 256, 0, s>>>(
-        reinterpret_cast<const int8_t*>(xp), reinterpret_cast<int8_t*>(yp), total / 4, npix, cp, h, w, oh, ow, kh, kw,
-        stride_h, stride_w, pad_h, pad_w);
+    const int8_t* x8 = reinterpret_cast<const int8_t*>(xp);
+    int8_t* y8 = reinterpret_cast<int8_t*>(yp);
+    if ((int64_t)n * h * w >= 0x7fffffff) return arg_error("max_pool2d_i8 size");
+    if ((kh == 3 && kw == 3) || (kh == 2 && kw == 2)) {
+      const unsigned grid = grid_for((total / 4 + 1) / 2, 256, 1 << 16);   // two granules per thread
+      if (kh == 3)
+        k_max_pool_i8x16<3, 3><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
+      else
+        k_max_pool_i8x16<2, 2><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
+    } else {
+      k_max_pool_i8x16<0, 0><<<grid_for(total / 4, 256, 1 << 16), 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw,
+                                                                                stride_h, stride_w, pad_h, pad_w);
+    }
   } else {
     k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
                                                               reinterpret_cast<uint32_t*>(yp), total, npix, cp, h, w, oh, ow,
@@ -495,7 +544,7 @@ int cvmhip_sum_hw_i8(const void* xp, const cvmhip_chain* chain, void* out, int o
   const int64_t total = act_bytes(n, cp) / 4;
   hipStream_t s = as_stream(stream);
   KernelTimer timer("k_sum_hw_i8", (double)n * c * hw + (double)n * c, s);  // bytes in + out
-  k_sum_hw_i8<<<grid_for(total * 8, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
+  k_sum_hw_i8<<<grid_for(total * SUM_LANES, 256), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp), out, out_is_i8, total, n, c, cp,
                                                    hw, ch);
   return check_launch("sum_hw_i8");
 }
