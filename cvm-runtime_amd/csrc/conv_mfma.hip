@@ -1981,6 +1981,10 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT ||
       !(nopad || (g.KH <= 32 && g.KW <= 32)))
     return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
+  // a layer that fills the chip several times over is faster as a launch of the large-tile kernel than as a layer of a
+  // sequence (whose tile is the wavefront kernel's); a run of layers ends there
+  if (t_conv_tuning.kernel == CONV_KERNEL_AUTO && t_conv_tuning.wave_cfg < 0 && choose_big_cfg(g) >= 0)
+    return arg_error("conv_seq_layer: not eligible (a layer for the large-tile kernel)");
   SeqLayer& L = reinterpret_cast<SeqLayer*>(table)[index];
   memset(&L, 0, sizeof(L));
   L.px_per_share = (int)(g.P / SEQ_SHARES);
