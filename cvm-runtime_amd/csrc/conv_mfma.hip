@@ -1392,13 +1392,15 @@ __global__ void __launch_bounds__(256) k_pack_weights(const int32_t* __restrict_
 
 // int32 NCHW -> row-window input int8 [N][hp][wp][4], zero outside the image (conv_mfma.h: StemGeom)
 __global__ void __launch_bounds__(256) k_pack_stem(const int32_t* __restrict__ x, uint32_t* __restrict__ xs, int64_t total,
-                                                   int nimg, int c, int h, int w, int hp, int wp, int ph, int pw) {
+                                                   int nimg, int c, int h, int w, int hp, int wp, int ph, int pw,
+                                                   FastDiv div_wp, FastDiv div_hp) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int q = (int)(i % wp);
-    const int64_t t = i / wp;
-    const int p = (int)(t % hp);
-    const int64_t n = t / hp;
+    // total < 2^31 (checked by the host): 32-bit multiply-high divisions, three instructions each
+    const unsigned t = fastdiv((unsigned)i, div_wp);
+    const int q = (int)((unsigned)i - t * (unsigned)wp);
+    const int64_t n = fastdiv(t, div_hp);
+    const int p = (int)(t - (unsigned)n * (unsigned)hp);
     const int ih = p - ph, iw = q - pw;
     uint32_t pack = 0;
     if (n < nimg && ih >= 0 && ih < h && iw >= 0 && iw < w) {   // the slack behind the last image is cleared
@@ -1605,7 +1607,9 @@ int pack_stem_input(const int32_t* x, int8_t* xs, int n, int c, int h, int w, in
   const StemGeom sg = stem_geom(n, h, w, kh, kw, sh, sw, ph, pw);
   const int64_t total = (int64_t)sg.bytes / 4;   // the slack behind the last row is cleared too
   KernelTimer timer("k_pack_stem", (double)n * c * h * w * 5.0, s);
-  k_pack_stem<<<grid_for(total, 256), 256, 0, s>>>(x, reinterpret_cast<uint32_t*>(xs), total, n, c, h, w, sg.hp, sg.wp, ph, pw);
+  if (total > INT32_MAX) return arg_error("pack_stem size");
+  k_pack_stem<<<grid_for(total, 256), 256, 0, s>>>(x, reinterpret_cast<uint32_t*>(xs), total, n, c, h, w, sg.hp, sg.wp, ph, pw,
+                                                   make_fastdiv((uint32_t)sg.wp), make_fastdiv((uint32_t)sg.hp));
   return check_launch("pack_stem");
 }
 
