@@ -98,7 +98,13 @@ __host__ __device__ inline void act_decode(int64_t i, int cp, int64_t* p, int* c
     const int ctiles = cp >> 5;
     const int64_t blk = i >> 8;
     const int w = (int)(i & 255);
-    const int64_t ptile = blk / ctiles;
+    // one division per element of a bandwidth kernel: a shift when the channel tile count is a power of two (the usual
+    // case), a 32-bit division when the block index fits, the 64-bit one (some sixty instructions) only otherwise
+    const unsigned ct = (unsigned)ctiles;
+    int64_t ptile;
+    if ((ct & (ct - 1)) == 0) ptile = blk >> (31 - __builtin_clz(ct));
+    else if (blk <= 0xffffffffll) ptile = (int64_t)((uint32_t)blk / ct);
+    else ptile = blk / ctiles;
     *p = ptile * 32 + ((w >> 2) & 31);
     *c = (int)(blk - ptile * ctiles) * 32 + (w >> 7) * 16 + (w & 3) * 4;
   }

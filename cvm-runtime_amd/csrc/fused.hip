@@ -80,7 +80,7 @@ k_max_pool_i8(const uint32_t* __restrict__ x, uint32_t* __restrict__ y, int64_t 
 template <int KH, int KW>
 __global__ void __launch_bounds__(256)
 k_max_pool_i8x16(const int8_t* __restrict__ x, int8_t* __restrict__ y, int64_t total, int64_t npix_out, int cp, int h,
-                 int w, int oh, int ow, int kh, int kw, int sh, int sw, int ph, int pw) {
+                 int w, int oh, int ow, int kh, int kw, int sh, int sw, int ph, int pw, FastDiv div_ow, FastDiv div_oh) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   if constexpr (KH > 0) {
     constexpr int G = 2;
@@ -96,10 +96,11 @@ k_max_pool_i8x16(const int8_t* __restrict__ x, int8_t* __restrict__ y, int64_t t
         act_decode((i < total ? i : i0) * 4, cp, &t, &c0);
         ok[k] = i < total && t < npix_out;
         if (t >= npix_out) t = npix_out - 1;
-        const int q = (int)(t % ow);
-        t /= ow;
-        const int p = (int)(t % oh);
-        max_pool_request<KH, KW>(v[k], load, (int)(t / oh), p, q, c0, cp, h, w, sh, sw, ph, pw);
+        const unsigned row = fastdiv((unsigned)t, div_ow);          // npix_out < 2^31 (checked by the host)
+        const int q = (int)((unsigned)t - row * (unsigned)ow);
+        const unsigned n = fastdiv(row, div_oh);
+        const int p = (int)(row - n * (unsigned)oh);
+        max_pool_request<KH, KW>(v[k], load, (int)n, p, q, c0, cp, h, w, sh, sw, ph, pw);
       }
 #pragma unroll
       for (int k = 0; k < G; ++k)
@@ -515,16 +516,17 @@ int cvmhip_max_pool2d_i8(const void* xp, void* yp, int n, int c, int h, int w, i
     if (((uintptr_t)xp | (uintptr_t)yp) & 15) return arg_error("max_pool2d_i8 alignment");
     const int8_t* x8 = reinterpret_cast<const int8_t*>(xp);
     int8_t* y8 = reinterpret_cast<int8_t*>(yp);
-    if ((int64_t)n * h * w >= 0x7fffffff) return arg_error("max_pool2d_i8 size");
+    if ((int64_t)n * h * w >= 0x7fffffff || npix >= 0x7fffffff) return arg_error("max_pool2d_i8 size");
+    const FastDiv dow = make_fastdiv((uint32_t)ow), doh = make_fastdiv((uint32_t)oh);
     if ((kh == 3 && kw == 3) || (kh == 2 && kw == 2)) {
       const unsigned grid = grid_for((total / 4 + 1) / 2, 256, 1 << 16);   // two granules per thread
       if (kh == 3)
-        k_max_pool_i8x16<3, 3><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
+        k_max_pool_i8x16<3, 3><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, dow, doh);
       else
-        k_max_pool_i8x16<2, 2><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w);
+        k_max_pool_i8x16<2, 2><<<grid, 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, dow, doh);
     } else {
       k_max_pool_i8x16<0, 0><<<grid_for(total / 4, 256, 1 << 16), 256, 0, s>>>(x8, y8, total / 4, npix, cp, h, w, oh, ow, kh, kw,
-                                                                                stride_h, stride_w, pad_h, pad_w);
+                                                                                stride_h, stride_w, pad_h, pad_w, dow, doh);
     }
   } else {
     k_max_pool_i8<<<grid_for(total, 256, 1 << 16), 256, 0, s>>>(reinterpret_cast<const uint32_t*>(xp),
