@@ -1715,6 +1715,13 @@ static int choose_wave_cfg(const ConvGeom& g, int cus = 256) {
       // operand delivery, and a 64 x 128 wavefront tile takes 0.75 KiB per MFMA instead of 1 KiB (measured
       // 1.0 -> 1.2-1.3 POP/s on 28x28x512 and 56x56x256 layers with 3x3 filters).
       if (cus == 256 && c.ksplit == 1 && g.OC > 32 && g.K >= 512 && wave_cfg_blocks(kWaveCfgs[7], g) >= 192) return 7;
+      // Unsplit, short K, between one and two rounds of 64 x 64 tiles (ResNet's input layer: 784 workgroups for 512
+      // places): the second round is half empty, while the 64 x 128 tile fits one round (10.0 against 11.9 us)
+      if (cus == 256 && c.ksplit == 1 && g.OC > 32 && i == 3) {
+        const int64_t small = wave_cfg_blocks(c, g), big = wave_cfg_blocks(kWaveCfgs[7], g);
+        const int64_t places = capacity;
+        if (small > places && small <= 2 * places && big <= places) return 7;
+      }
       return i;
     }
   }
