@@ -1703,7 +1703,10 @@ static int choose_wave_cfg(const ConvGeom& g, int cus = 256) {
   const int nlive = g.K / 32;
   // very few pixels, deep K (fully connected layers, the last stage): even the deepest split of
   // the 64-channel tile leaves SIMDs without a wavefront, so halve the tile instead
-  if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < cus / 2) return 4;
+  // (one XCD's share of a layer-sequence launch: also when the 64-channel tiles would fill exactly half of its 32 CUs --
+  // the 512-channel layers of a ResNet's last stage, 16 tiles -- where the 32 tiles of the halved tile give every CU
+  // 0.75 of the operand bytes instead of every second CU all of them: 363 -> 355 us for the ResNet-50 sequence)
+  if (g.OC > 32 && nlive >= 16 && wave_cfg_blocks(kWaveCfgs[0], g) < cus / 2 + (cus == 32 ? 1 : 0)) return 4;
   const int first = g.OC > 32 ? 0 : 4;
   const int last = g.OC > 32 ? 4 : 7;   // 64-channel tiles: 0..3 (and 7, see below); 32-channel tiles: 4..6
   for (int i = first; i < last; ++i) {
