@@ -278,6 +278,42 @@ def test_conv2d_stem_i8(case, dev):
 
 
 @pytest.mark.parametrize("cfg", range(8))
+def test_conv2d_stem_i8_every_configuration(cfg, dev):
+    """The row-window input layer under every tile / K-split configuration of the wavefront kernel."""
+    n, c, h, w, oc, kh, kw, st, pd = (2, 3, 40, 36, 64, 7, 7, 2, 3)
+    cid = "stem-cfg"
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, c, kh, kw), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1)
+    stages = [("relu",), ("cvm_right_shift", 8, 9)]
+    os.environ["CVM_HIP_WAVECFG"] = str(cfg)
+    try:
+        out32 = hipops.conv2d_stem_i8(T(x, dev), T(wt, dev), T(b, dev), None, False, (st, st), (pd, pd))
+        out8 = hipops.conv2d_stem_i8(T(x, dev), T(wt, dev), T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+    eq(out32.cpu().numpy(), conv, "stem cfg %d int32" % cfg)
+    eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), run_chain(conv, stages), "stem cfg %d int8" % cfg)
+
+
+def test_conv2d_stem_i8_benchmark_shape(dev):
+    """ResNet-50's input layer at the benchmark's batch 16 (the shape for which the 64 x 128 tile is chosen
+    automatically: 784 workgroups of 64 x 64 tiles for 512 places)."""
+    n, c, h, w, oc, kh, kw, st, pd = (16, 3, 224, 224, 64, 7, 7, 2, 3)
+    cid = "stem-b16"
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, c, kh, kw), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    conv = oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1)
+    stages = [("relu",), ("cvm_right_shift", 8, 9)]
+    out8 = hipops.conv2d_stem_i8(T(x, dev), T(wt, dev), T(b, dev), hipops.chain(*stages), True, (st, st), (pd, pd))
+    torch.cuda.synchronize()
+    eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), run_chain(conv, stages), "stem batch 16 int8")
+
+
+@pytest.mark.parametrize("cfg", range(8))
 @pytest.mark.parametrize("case", [(3, 96, 11, 13, 100, 3, 1, 1, True), (2, 256, 9, 9, 72, 1, 2, 0, False),
                                   (1, 64, 8, 8, 40, 3, 2, 1, True)],
                          ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%d" % c[:8])
