@@ -1908,12 +1908,6 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (force_lds && !rows) cfg = -1;
   if (wave_ok && force_wave && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced >= 0 && wave_forced < kNumWaveCfgs) cfg = wave_forced;
-  if (const char* e = getenv("WAVECFG_DBG")) {   // "KH,SH,C,OC,N,H:cfg;..."
-    char sig[64];
-    snprintf(sig, sizeof(sig), "%d,%d,%d,%d,%d,%d:", g.KH, g.SH, g.C ? g.C : g.Cp, g.OC, g.N, g.H);
-    const char* hit = strstr(e, sig);
-    if (hit && wave_ok && cfg >= 0 && !g.dw) { const int c2 = atoi(hit + strlen(sig)); if (c2 >= 0 && c2 < kNumWaveCfgs) cfg = c2; }
-  }
   const int kslices = ws ? conv_slices(g, ep) : 1;
   if (kslices > 1 && wave_ok) {
     const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
