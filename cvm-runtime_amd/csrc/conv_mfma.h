@@ -70,6 +70,12 @@ struct Epilogue {
   // out + n*stride, e.g. straight into its slice of a concatenated tensor.
   int64_t o32_img;
   int o32_ch, o32_px;
+  // 1: max_pool2d with a 2x2 window, stride 2 and no padding follows the chain (ops.cc:466-523 for such a window: the
+  // maximum of four values that all exist) and is taken before the store: the output tensor is (N, OC, OH/2, OW/2),
+  // int8, OH and OW even.  The wavefront and large-tile kernels then enumerate the convolution's pixels window by
+  // window (pixel index = 4 * window + 2 * (oh % 2) + ow % 2), so the four values of a window sit in four
+  // neighbouring lanes.  Set through conv_igemm_ws only where conv_pool_eligible says so.
+  int pool;
 };
 
 // ---- int8 activation layout.  Channels are padded to Cp = 4, 8, 16 or a
@@ -194,6 +200,10 @@ int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const 
 // several workgroups per tile (partial sums in the workspace, a second kernel finishes).  Without a workspace, or for
 // any other layer, identical to conv_igemm.  conv_slices_workspace_bytes() gives the size (0 = not applicable).
 size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep);
+// Whether a convolution with this geometry (N, H, W, Cp, OC, OH, OW, filter, strides, padding, dilation set) can take
+// Epilogue::pool: int8 pixel-blocked input and output (channels padded to 32 on both sides), an even output extent,
+// a filter side of at most 32.
+bool conv_pool_eligible(const ConvGeom& g);
 int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, void* ws, size_t ws_bytes,
                   hipStream_t s);
 

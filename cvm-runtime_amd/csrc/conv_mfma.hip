@@ -248,6 +248,23 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     return;
   }
   int8_t* y8 = reinterpret_cast<int8_t*>(out);
+  // Fused 2x2 max-pool (host: only with a pixel-blocked output): the four pixels of a window are the four lanes of a
+  // quad, so two quad permutes leave the window's maximum in each of them; lane 0 of the quad stores it as pixel
+  // p / 4 of the pooled tensor.
+  bool pool = false;
+  if constexpr (!RANGE) pool = blocked && ep.pool != 0;
+  const bool store_lane = !pool || (lrow & 3) == 0;
+  const int pshift = pool ? 2 : 0;
+  if (pool) {
+#pragma unroll
+    for (int e = 0; e < NG * 4; ++e) {
+      int32_t v = val[e];
+      const int32_t a = __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
+      v = v > a ? v : a;
+      const int32_t b = __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);   // quad_perm [2, 3, 0, 1]
+      val[e] = v > b ? v : b;
+    }
+  }
   uint32_t pk[NG];
 #pragma unroll
   for (int m = 0; m < NG; ++m) pk[m] = pack_bytes(val[m * 4], val[m * 4 + 1], val[m * 4 + 2], val[m * 4 + 3]);
@@ -264,8 +281,13 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int p = px_wave + gj[t * 4] * 32 + lrow;
       if (p < P && p >= Plo && first < ocp) {
         const v4i pk4 = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-        if constexpr (RANGE) *reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16) = pk4;
-        else __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16));
+        if constexpr (RANGE) {
+          *reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16) = pk4;
+        } else if (pool) {   // window p / 4 of the pooled tensor, the 16 channels this lane holds
+          if ((lrow & 3) == 0) __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + act_offset(p >> 2, first, ocp)));
+        } else {
+          __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16));
+        }
       }
     }
   } else if (halves) {
@@ -275,7 +297,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     const int first = oc0 + ch[0] - lgrp * 4 + lgrp * 8;
     mask_channels(w, first, g.OC);
     const int p = px_wave + gj[0] * 32 + lrow;
-    if (p < P && p >= Plo && first < ocp) *reinterpret_cast<uint2*>(y8 + act_offset(p, first, ocp)) = make_uint2(w[0], w[1]);
+    if (p < P && p >= Plo && first < ocp && store_lane) *reinterpret_cast<uint2*>(y8 + act_offset(p >> pshift, first, ocp)) = make_uint2(w[0], w[1]);
   } else {
 #pragma unroll
     for (int m = 0; m < NG; ++m) {
@@ -283,7 +305,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int first = oc0 + ch[m];
       mask_channels(w, first, g.OC);
       const int p = px_wave + gj[m] * 32 + lrow;
-      if (p < P && p >= Plo && first < ocp) *reinterpret_cast<uint32_t*>(y8 + act_offset(p, first, ocp)) = w[0];
+      if (p < P && p >= Plo && first < ocp && store_lane) *reinterpret_cast<uint32_t*>(y8 + act_offset(p >> pshift, first, ocp)) = w[0];
     }
   }
 }
@@ -495,6 +517,27 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 // Bit t set when filter tap t (of k <= 32) of a receptive field that starts at input coordinate x0
 // lies inside [0, extent).  Without dilation the valid taps are the run max(0, -x0) ..
 // min(k - 1, extent - 1 - x0), which needs no loop and no branch.
+// Image and output coordinates of output pixel index p.  Ordinary order: p = (n * OH + oh) * OW + ow.  With a fused 2x2
+// max-pool (Epilogue::pool) the pixels are numbered window by window, p = 4 * window + 2 * (oh % 2) + ow % 2 with
+// window = (n * OH/2 + oh/2) * OW/2 + ow/2, and the host has set div_ohw and div_ow to divide by OH*OW/4 and OW/2.
+__device__ __forceinline__ void conv_out_pixel(const ConvGeom& g, const bool pool, const unsigned p, int& n, int& oh, int& ow) {
+  const int OHW = g.OH * g.OW;
+  if (!pool) {
+    n = (int)fastdiv(p, g.div_ohw);
+    const int rem = (int)p - n * OHW;
+    oh = (int)fastdiv((unsigned)rem, g.div_ow);
+    ow = rem - oh * g.OW;
+  } else {
+    const unsigned q = p >> 2;
+    n = (int)fastdiv(q, g.div_ohw);
+    const int rem = (int)q - n * (OHW >> 2);
+    const int qh = (int)fastdiv((unsigned)rem, g.div_ow);
+    const int qw = rem - qh * (g.OW >> 1);
+    oh = 2 * qh + (int)((p >> 1) & 1u);
+    ow = 2 * qw + (int)(p & 1u);
+  }
+}
+
 __device__ __forceinline__ unsigned tap_mask_dense(int x0, int extent, int k) {
   int lo = x0 < 0 ? -x0 : 0;
   int hi = extent - 1 - x0;
@@ -605,7 +648,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);   // g.octiles = ceil(OC / BM), set by the host for this tile
   const int oc0 = (pid - ptile * g.octiles) * BM;
   const int px0 = (COH ? (p_begin & ~31) : 0) + ptile * BN;   // P < 2^31 is checked on the host
-  const int OHW = g.OH * g.OW;
   const int ctiles = g.Cp >> 5;
   const int P = (int)g.P;
   __amdgpu_buffer_rsrc_t rs_x = act_rsrc(xp);   // activations are read through a buffer descriptor: 32-bit offsets, zeros past the end
@@ -626,10 +668,8 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       const int p = px0 + (pw_ * TN + (j ^ Xj)) * 32 + lrow;
       const bool ok = COH ? (p >= p_begin && p < p_end) : p < P;
       const unsigned pp = ok ? (unsigned)p : 0u;
-      const int n = (int)fastdiv(pp, g.div_ohw);
-      const int rem = (int)pp - n * OHW;
-      const int oh = (int)fastdiv((unsigned)rem, g.div_ow);
-      const int ow = rem - oh * g.OW;
+      int n, oh, ow;
+      conv_out_pixel(g, !COH && MODE != WAVE_ROWS && ep.pool != 0, pp, n, oh, ow);
       const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
       rowbase[j] = (n * g.H + ih0) * g.W + iw0;
       if (MODE == WAVE_ROWS) rowbase[j] *= 4;   // byte offset of the window of filter row 0 (g.H, g.W: stored size, no padding left)
@@ -969,7 +1009,7 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);
   const int oc0 = (pid - ptile * g.octiles) * BM;
   const int px0 = ptile * BN;
-  const int P = (int)g.P, OHW = g.OH * g.OW;
+  const int P = (int)g.P;
   const int ctiles = g.Cp >> 5;
   const int nch = g.Kp >> 5, nlive = (g.K + 31) >> 5;
   const int nsteps = g.Kp >> 6;
@@ -983,10 +1023,8 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
     const int p = px0 + (wave + 4 * q) * 32 + lrow;
     const bool ok = p < P;
     const unsigned pp = ok ? (unsigned)p : 0u;
-    const int n = (int)fastdiv(pp, g.div_ohw);
-    const int rem = (int)pp - n * OHW;
-    const int oh = (int)fastdiv((unsigned)rem, g.div_ow);
-    const int ow = rem - oh * g.OW;
+    int n, oh, ow;
+    conv_out_pixel(g, ep.pool != 0, pp, n, oh, ow);
     const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
     rowbase[q] = (n * g.H + ih0) * g.W + iw0;
     unsigned rm, cm;
@@ -1178,7 +1216,7 @@ struct SeqLayer {
   int kernel;          // configuration * 3 + mode (identity, no padding, padding)
   int px_per_share;    // output pixels of one share of the images
   int ptiles;          // pixel tiles that cover a share (its first block may begin before the share)
-  int reserved;
+  int reserved[3];     // keeps the entry a multiple of 16 bytes
 };
 constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
 enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
@@ -1812,7 +1850,7 @@ static double conv_bytes(const ConvGeom& g, const Epilogue& ep) {
   const double c = g.C ? g.C : g.Cp;
   const double in = (double)g.N * g.H * g.W * (g.row_bytes ? 4.0 : c);
   const double flt = (double)g.OC * (g.dw ? 1.0 : c) * g.taps;
-  const double outb = (double)g.P * g.OC * (ep.out_mode == OUT_I8_ACT ? 1.0 : 4.0);
+  const double outb = (double)g.P * g.OC * (ep.out_mode == OUT_I8_ACT ? 1.0 : 4.0) / (ep.pool ? 4.0 : 1.0);
   return in + flt + outb + (ep.residual ? (double)g.P * g.OC : 0.0);
 }
 struct ConvDesc {
@@ -1821,13 +1859,18 @@ struct ConvDesc {
     text[0] = 0;
     if (!kernel_timing_enabled()) return;
     snprintf(text, sizeof(text), "%s%dx%d/%d %d->%d in %dx%dx%d out %dx%d%s%s %s cfg %d mode %d grid %ld", g.dw ? "dw " : "",
-             g.KH, g.KW, g.SH, g.C ? g.C : g.Cp, g.OC, g.N, g.H, g.W, g.OH, g.OW, ep.residual ? " +res" : "",
+             g.KH, g.KW, g.SH, g.C ? g.C : g.Cp, g.OC, g.N, g.H, g.W, g.OH, g.OW, ep.residual ? " +res" : ep.pool ? " +pool" : "",
              ep.out_mode == OUT_I8_ACT ? " i8" : " i32", kernel, cfg, mode, grid);
   }
 };
 
 int conv_igemm(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep_in, hipStream_t s) {
   return conv_igemm_ws(xp, wp, out, g, ep_in, nullptr, 0, s);
+}
+
+bool conv_pool_eligible(const ConvGeom& g) {
+  return !g.dw && g.row_bytes == 0 && (g.Cp % 32) == 0 && (pad_channels(g.OC) % 32) == 0 && g.KH <= 32 && g.KW <= 32 &&
+         g.OH >= 2 && g.OW >= 2 && (g.OH % 2) == 0 && (g.OW % 2) == 0;
 }
 
 // Checks a convolution's geometry and fills the derived fields of g and the defaults of the epilogue.
@@ -1863,8 +1906,15 @@ static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom&
   } else if (ep.o32_ch < 1 || ep.o32_px < 1 || ep.o32_img < 0) {
     return arg_error("conv int32 output strides");
   }
-  g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
-  g.div_ow = make_fastdiv((uint32_t)g.OW);
+  if (ep.pool) {   // pixels are numbered window by window (conv_out_pixel)
+    if (!conv_pool_eligible(g) || ep.out_mode != OUT_I8_ACT || ep.residual)
+      return arg_error("conv with fused 2x2 max-pool: not eligible (int8 pixel-blocked tensors, even output extent, no residual)");
+    g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW / 4));
+    g.div_ow = make_fastdiv((uint32_t)(g.OW / 2));
+  } else {
+    g.div_ohw = make_fastdiv((uint32_t)(g.OH * g.OW));
+    g.div_ow = make_fastdiv((uint32_t)g.OW);
+  }
   g.div_ct = make_fastdiv((uint32_t)(g.dw ? 1 : g.Cp >= 32 ? g.Cp / 32 : 1));
   g.div_kw = make_fastdiv((uint32_t)g.KW);
   return CVMHIP_OK;
@@ -1908,7 +1958,8 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (force_lds && !rows) cfg = -1;
   if (wave_ok && force_wave && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced >= 0 && wave_forced < kNumWaveCfgs) cfg = wave_forced;
-  const int kslices = ws ? conv_slices(g, ep) : 1;
+  if (ep.pool && cfg < 0) cfg = g.OC > 32 ? 3 : 6;   // the tiled kernel has no pooled form
+  const int kslices = ws && !ep.pool ? conv_slices(g, ep) : 1;
   if (kslices > 1 && wave_ok) {
     const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
     if (ws_bytes < need || ((uintptr_t)ws & 15)) return arg_error("conv K-slice workspace");
@@ -1965,8 +2016,9 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     }
   }
   if (cfg >= 0) {
+    // (with a fused max-pool the pixels are renumbered, so output block t is no longer input block t)
     const int mode = rows ? WAVE_ROWS
-                          : (!g.dw && g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                          : (!g.dw && !ep.pool && g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
                                 ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
@@ -2008,7 +2060,7 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
   if (prc) return prc;
   const bool nopad = g.PH == 0 && g.PW == 0;
-  if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT ||
+  if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT || ep.pool ||
       !(nopad || (g.KH <= 32 && g.KW <= 32)))
     return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
   // a layer that fills the chip several times over is faster as a launch of the large-tile kernel than as a layer of a

@@ -271,7 +271,7 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
                          int n, int ic, int h, int wd, int oc, int kh, int kw,
                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream,
                          void* ws = nullptr, size_t ws_bytes = 0, size_t* ws_query = nullptr, void* seq_table = nullptr,
-                         int seq_index = 0) {
+                         int seq_index = 0, int pool = 0, int* pool_query = nullptr) {
   if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
   if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
       pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
@@ -295,6 +295,11 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
     ep.o32_img = nhwc_image_stride;
     ep.o32_ch = 1;
     ep.o32_px = oc;
+  }
+  ep.pool = pool;
+  if (pool_query) {   // eligibility question only
+    *pool_query = conv_pool_eligible(g) ? 1 : 0;
+    return CVMHIP_OK;
   }
   if (ws_query) {   // size question only
     *ws_query = nhwc_image_stride >= 0 ? 0 : conv_slices_workspace_bytes(g, ep);
@@ -331,6 +336,22 @@ int cvmhip_conv2d_i8(const void* xp, const void* wp, const int32_t* bias, const 
                      int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
   return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, out_is_i8, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
                        pad_h, pad_w, dil_h, dil_w, stream);
+}
+
+int cvmhip_conv2d_pool2_i8_eligible(int n, int ic, int h, int wd, int oc, int kh, int kw,
+                                    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w) {
+  int yes = 0;
+  const int dummy = 0;
+  const int rc = conv2d_i8_any(&dummy, &dummy, nullptr, nullptr, nullptr, nullptr, const_cast<int*>(&dummy), 1, -1, n, ic, h, wd, oc, kh,
+                               kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, nullptr, nullptr, 0, nullptr, nullptr, 0, 1, &yes);
+  return rc == CVMHIP_OK ? yes : 0;
+}
+
+int cvmhip_conv2d_pool2_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain, void* out,
+                           int n, int ic, int h, int wd, int oc, int kh, int kw,
+                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  return conv2d_i8_any(xp, wp, bias, chain, nullptr, nullptr, out, 1, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w,
+                       pad_h, pad_w, dil_h, dil_w, stream, nullptr, 0, nullptr, nullptr, 0, 1);
 }
 
 size_t cvmhip_conv_seq_layer_bytes(void) { return conv_seq_layer_bytes(); }

@@ -484,7 +484,24 @@ void HipGraphRuntime::BuildPlan() {
         b.lo = -128;
         b.hi = 127;
         finish_output(&st, out0, b);
-        if (st.out_i8) {
+        // A 2x2 window with stride 2 and no padding over an even extent, fed by a convolution that nobody else reads:
+        // the convolution takes the maximum itself and writes the pooled tensor (the full-resolution one is never stored).
+        const int ps = producer_step[xe];
+        if (st.out_i8 && hooks_.pool_fuse && ps >= 0 && plan[ps].kind == PlanStep::CONV && plan[ps].dst == xe &&
+            plan[ps].out_i8 && !plan[ps].stem && !plan[ps].nhwc && plan[ps].src2 == kNone && !plan[ps].pool2 &&
+            uses[xe].size() == 1 && !is_head[xe] && st.kh == 2 && st.kw == 2 && st.sh == 2 && st.sw == 2 && st.ph == 0 &&
+            st.pw == 0 && st.h % 2 == 0 && st.w % 2 == 0 && st.oh == st.h / 2 && st.ow == st.w / 2 &&
+            cvmhip_conv2d_pool2_i8_eligible(plan[ps].n, plan[ps].c, plan[ps].h, plan[ps].w, plan[ps].oc, plan[ps].kh,
+                                            plan[ps].kw, plan[ps].sh, plan[ps].sw, plan[ps].ph, plan[ps].pw, plan[ps].dh,
+                                            plan[ps].dw)) {
+          PlanStep& cs = plan[ps];
+          cs.pool2 = true;
+          cs.label += "+pool";
+          cs.dst = out0;
+          has_i8[xe] = false;
+          producer_step[out0] = ps;
+          done = true;
+        } else if (st.out_i8) {
           plan.push_back(st);
           done = true;
         } else {  // nobody downstream reads int8: leave the node to the int32 kernel
@@ -612,7 +629,7 @@ void HipGraphRuntime::BuildSequences() {
     size_t j = i;
     for (; j < plan_.size(); ++j) {
       const PlanStep& st = plan_[j];
-      if (st.kind != PlanStep::CONV || st.stem || st.nhwc || st.ws || !st.out_i8) break;
+      if (st.kind != PlanStep::CONV || st.stem || st.nhwc || st.ws || !st.out_i8 || st.pool2) break;
       table.resize((j - i + 1) * entry);
       const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
       const int rc = cvmhip_conv_seq_layer(table.data(), static_cast<int>(j - i), i8_ptr_[st.src],
@@ -686,6 +703,12 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
         Check(cvmhip_conv2d_i8_nhwc(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain,
                                     entry_ptr_[st.dst] + st.dst_off, st.img_stride, st.n, st.c, st.h, st.w, st.oc, st.kh,
                                     st.kw, st.sh, st.sw, st.ph, st.pw, st.dh, st.dw, stream_), "conv2d_i8_nhwc");
+        break;
+      }
+      if (st.pool2) {
+        Check(cvmhip_conv2d_pool2_i8(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, out,
+                                     st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw, st.dh, st.dw,
+                                     stream_), "conv2d_pool2_i8");
         break;
       }
       const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];

@@ -103,6 +103,7 @@ struct PlanStep {
   std::shared_ptr<void> ws;       // CONV: workspace of a K-sliced launch (cvmhip_conv2d_i8_ws), or empty
   size_t ws_bytes = 0;
   bool dw_mfma = false;           // DWCONV through the implicit-GEMM kernel (filter packed as diagonal blocks)
+  bool pool2 = false;             // CONV also takes the 2x2 stride-2 max_pool2d that follows it (cvmhip_conv2d_pool2_i8); dst is the pooled tensor
   bool nhwc = false;              // CONV writes int32 pixel-major rows into a slice of entry dst (a fused detection head)
   int64_t dst_off = 0, img_stride = 0;  // that slice: first element, and elements from one image to the next
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;
@@ -208,7 +209,7 @@ class HipGraphRuntime {
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;

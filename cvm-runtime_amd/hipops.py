@@ -403,6 +403,21 @@ def conv2d_i8(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=
     return out
 
 
+def conv2d_pool2_eligible(n, ic, h, w, oc, kh, kw, strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    return bool(lib().cvmhip_conv2d_pool2_i8_eligible(n, ic, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                                      dilation[0], dilation[1]))
+
+
+def conv2d_pool2_i8(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """conv2d + chain + max_pool2d(2x2, stride 2) in one launch; returns the pooled int8 act tensor."""
+    oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+    out = _act_buffer(n * (oh // 2) * (ow // 2), oc, xp.device)
+    check(lib().cvmhip_conv2d_pool2_i8(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None, _vp(out),
+                                       n, ic, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                       dilation[0], dilation[1], _stream()))
+    return out
+
+
 def conv2d_i8_ws(xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, out_is_i8=True,
                  strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
     """conv2d_i8 with the workspace the library asks for (K slices over the grid for small-batch dense

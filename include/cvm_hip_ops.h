@@ -282,6 +282,18 @@ int cvmhip_conv2d_i8_ws(const void* xp, const void* wp, const int32_t* bias, con
                         int n, int ic, int h, int wd, int oc, int kh, int kw,
                         int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
                         void* workspace, size_t workspace_bytes, void* stream);
+/* conv2d + chain followed by max_pool2d with a 2x2 window, stride 2 and no padding (ops.cc:466-523: the maximum of the
+ * four values of a window, all of which exist when the convolution's output extent is even) in ONE launch: the
+ * kernel numbers the convolution's output pixels window by window, takes the maximum of the four requantised
+ * values across lanes and stores only that.  out is the int8 act tensor of the POOLED result (n, oc, OH/2, OW/2);
+ * the full-resolution tensor is never written.  Eligible (..._eligible returns 1): input and output channels
+ * padded to a multiple of 32 (ic, oc > 16), OH and OW even, filter side <= 32; otherwise the call fails with
+ * CVMHIP_ERR_ARG and the caller runs cvmhip_conv2d_i8 and cvmhip_max_pool2d_i8. */
+int cvmhip_conv2d_pool2_i8_eligible(int n, int ic, int h, int wd, int oc, int kh, int kw,
+                                    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+int cvmhip_conv2d_pool2_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain, void* out,
+                           int n, int ic, int h, int wd, int oc, int kh, int kw,
+                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
 /* A run of convolutions in ONE launch, for a batch that is a multiple of cvmhip_conv_seq_shares() (8, the XCDs
  * of the chip).  No counterpart in the reference.  Images are independent, so every XCD computes all layers
  * of the run for its own share of the images; a layer boundary is then a counter in that XCD's L2 instead of a

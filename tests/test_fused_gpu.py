@@ -9,7 +9,7 @@ import torch
 
 import oracle
 import oracle.graph as og
-from cvm_runtime_amd import graphgen, hipops, runtime, synth
+from cvm_runtime_amd import CvmHipError, graphgen, hipops, runtime, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -386,6 +386,67 @@ def test_large_tile_kernel_every_tile(case, tile, dev):
     eq(out32.cpu().numpy(), conv, "large tile %d int32" % tile)
 
 
+POOL_FUSED_CASES = [
+    # n, ic, h, w, oc, k, stride, pad, dilation, bias
+    (2, 64, 20, 20, 160, 3, 1, 1, 1, True),     # 3x3 with padding, channels past one tile
+    (1, 96, 18, 14, 300, 3, 1, 1, 1, True),     # ragged channel count, windows that straddle pixel tiles
+    (3, 32, 9, 9, 64, 5, 2, 2, 1, False),       # stride 2; the 5x5 output has no whole 2x2 windows: refused
+    (1, 128, 12, 12, 128, 3, 1, 2, 2, True),    # dilated
+    (2, 256, 8, 6, 96, 1, 1, 0, 1, True),       # 1x1 without padding (the identity addressing must not be used)
+    (1, 64, 34, 30, 40, 3, 1, 0, 1, True),      # no padding, few channels
+    (4, 160, 14, 14, 256, 3, 1, 1, 1, True),    # five channel blocks per tap
+    (1, 32, 4, 4, 32, 3, 1, 1, 1, True),        # a single pixel tile, mostly empty
+]
+# kernel, wavefront configuration, large tile
+POOL_FUSED_KERNELS = [("auto", None, None)] + [("wave", str(c), None) for c in range(8)] + [("big", None, t) for t in (1, 2, 3)]
+
+
+@pytest.mark.parametrize("kern", POOL_FUSED_KERNELS, ids=lambda k: "%s%s%s" % (k[0], "-cfg" + k[1] if k[1] else "", "-tile%d" % k[2] if k[2] else ""))
+@pytest.mark.parametrize("case", POOL_FUSED_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%ds%dp%dd%d" % c[:9])
+def test_conv2d_with_fused_max_pool(case, kern, dev):
+    """conv2d -> requantisation -> max_pool2d(2x2, stride 2) in one launch equals the oracle's three operators, for
+    the automatic choice, every configuration of the wavefront kernel and every tile of the large-tile kernel."""
+    n, ic, h, w, oc, k, st, pd, dl, bias = case
+    cid = "poolfused-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768) if bias else None
+    ch1 = [("relu",), ("cvm_right_shift", 8, 12)] if n % 2 else [("cvm_right_shift", 8, 12)]
+    conv = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (dl, dl), 1), ch1)
+    oh, ow = conv.shape[2:]
+    eligible = hipops.conv2d_pool2_eligible(n, ic, h, w, oc, k, k, (st, st), (pd, pd), (dl, dl))
+    assert eligible == (oh % 2 == 0 and ow % 2 == 0)
+    xp, wp = hipops.pack_act_i8(T(x, dev)), hipops.pack_weights(T(wt, dev))
+    if kern[0] != "auto":
+        os.environ["CVM_HIP_CONV"] = kern[0]
+    if kern[1]:
+        os.environ["CVM_HIP_WAVECFG"] = kern[1]
+    if kern[2]:
+        os.environ["CVM_HIP_TILE"] = "%d,0" % kern[2]
+    try:
+        if not eligible:
+            with pytest.raises(CvmHipError):
+                hipops.conv2d_pool2_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1),
+                                       (st, st), (pd, pd), (dl, dl))
+            return
+        out = hipops.conv2d_pool2_i8(xp, n, ic, h, w, wp, oc, k, k, T(b, dev) if bias else None, hipops.chain(*ch1),
+                                     (st, st), (pd, pd), (dl, dl))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_CONV", None)
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+        os.environ.pop("CVM_HIP_TILE", None)
+    ref = oracle.max_pool2d(conv, (2, 2), (2, 2), (0, 0), False)
+    eq(act_to_nchw(out, n, oc, oh // 2, ow // 2), ref, "conv + max_pool, %s" % (kern,))
+
+
+def test_conv2d_with_fused_max_pool_refuses_small_channel_counts(dev):
+    assert not hipops.conv2d_pool2_eligible(1, 16, 8, 8, 64, 3, 3, (1, 1), (1, 1))    # input not pixel-blocked
+    assert not hipops.conv2d_pool2_eligible(1, 64, 8, 8, 16, 3, 3, (1, 1), (1, 1))    # output not pixel-blocked
+    assert not hipops.conv2d_pool2_eligible(1, 64, 9, 8, 64, 3, 3, (1, 1), (1, 1))    # odd extent
+    assert hipops.conv2d_pool2_eligible(1, 64, 8, 8, 64, 3, 3, (1, 1), (1, 1))
+
+
 DW_MFMA_CASES = [
     # n, c, h, w, k, stride, pad, dilation
     (2, 32, 19, 17, 3, 1, 1, 1),
@@ -526,6 +587,30 @@ def test_fused_executor_equals_node_by_node(name, dev):
         finally:
             os.environ.pop("CVM_HIP_FUSE", None)
     assert outs["1"] == outs["0"]
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
+def test_planner_folds_2x2_max_pools_into_their_convolutions(dev):
+    """A VGG whose pooled layers have at least 32 channels: the planner lets those convolutions take their max-pool
+    (fewer launches), CVM_HIP_POOLFUSE=0 keeps the two launches, and both equal the oracle."""
+    g, heads = graphgen.vgg16(2, size=32, width=32, fc=64, classes=20, config_id="poolfuse-vgg")
+    js, pb = g.build(heads)
+    x = synth.tensor("poolfuse-vgg", "data", g.shape((0, 0)), -127, 127)
+    outs, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_POOLFUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(x.astype(np.int8).tobytes())
+            launches[mode] = m.launch_counts()[0]
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_POOLFUSE", None)
+    assert outs["1"] == outs["0"]
+    assert launches["1"] == launches["0"] - 5, launches   # all five pools of a VGG-16 follow an eligible convolution here
     ref = og.run_graph(js, graphgen.load_params(pb), x)
     got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
