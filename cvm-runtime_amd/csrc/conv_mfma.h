@@ -187,6 +187,11 @@ size_t packed_stem_weight_bytes(int oc, int kp);
 int pack_stem_input(const int32_t* x, int8_t* xs, int n, int c, int h, int w, int kh, int kw, int sh, int sw, int ph,
                     int pw, hipStream_t s);
 int pack_stem_weights(const int32_t* w, int8_t* wp, int oc, int c, int kh, int kw, hipStream_t s);
+// Row-window convolution + chain + max_pool2d(3x3, stride 2, padding 1) in one launch (k_stem_pool): xs from
+// pack_stem_input, wp from pack_stem_weights, out the pooled int8 tensor (n, oc, qh, qw); oc 32 or 64.
+bool stem_pool_eligible(int c, int oc, int kh, int kw, int oh, int ow, int qh, int qw);
+int stem_pool(const int8_t* xs, const int8_t* wp, const int32_t* bias, const DevChain& chain, int8_t* out, int n, int c, int h,
+              int w, int oc, int kh, int kw, int sh, int sw, int ph, int pw, int qh, int qw, hipStream_t s);
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp);
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw);
 

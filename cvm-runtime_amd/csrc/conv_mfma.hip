@@ -1191,6 +1191,123 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   big_epilogue_rows<0, TM, TN, OUT>(acc, sBias, wm * TM * 32, oc0, px0 + wn * TN * 32, lane, out, g, ep);
 }
 
+// ---------------------------------------------------------------- row-window convolution + 3x3 stride-2 max-pool
+// The head of a ResNet: a convolution over a few input channels (row-window form, see StemGeom) whose only reader
+// is max_pool2d with a 3x3 window, stride 2 and padding 1 (ops.cc:466-523).  A workgroup computes a patch of
+// 4 x 8 pooled pixels of one image for up to 64 output channels: the 9 x 17 convolution pixels under it (windows
+// overlap, so neighbouring patches share a row and a column: 1.2 x the multiply-adds, which are a small part of a
+// launch that is all latency) go through the requantisation chain into LDS as int8, pixels outside the
+// convolution's output as -128 (every window holds at least one real pixel, so the padding never wins), and a
+// second phase takes the maxima.  The convolution's output never reaches memory and the pool's launch goes away.
+// A workgroup's chain of steps is long (0.6 us of addresses, 2 us of requests and MFMAs, 1.8 us of requantisation
+// into LDS, 0.6 us of maxima at one workgroup per CU), so this pays while the grid is a single round of workgroups
+// (a ResNet's head at batch 1: 8.0 against 4.0 + 4.7 us and a launch gap); at batch 16 its three rounds take 22 us
+// against 17 us for the two launches, and the caller keeps those.
+struct StemPool {
+  int N, Hs, Ws;         // stored (zero padded) input extent in pixels of 4 bytes
+  int OH, OW, QH, QW;    // extent of the convolution's and of the pool's output
+  int SH, SW, OC, ocp;
+  int nch, nlive, sh16;  // chunks per row of the packed filter (zero chunk at nch), chunks of the true K, row_bytes >> 5
+  int tiles_x, tiles_y;
+  DevChain chain;
+  const int32_t* bias;
+};
+constexpr int SP_PH = 4, SP_PW = 8, SP_CH = 2 * SP_PH + 1, SP_CW = 2 * SP_PW + 1, SP_PIX = SP_CH * SP_CW;
+constexpr int SP_BLOCKS = (SP_PIX + 31) / 32, SP_SLOTS = (SP_BLOCKS + 1) / 2, SP_BATCH = 8;
+
+__global__ void __launch_bounds__(256, 2)
+k_stem_pool(const int8_t* __restrict__ xs, const int8_t* __restrict__ wf, int8_t* __restrict__ out, const StemPool a) {
+  __shared__ __attribute__((aligned(16))) int8_t sTile[SP_BLOCKS * 32 * 64];   // [convolution pixel of the patch][64 channels]
+  __shared__ int sBias[64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int tx = blockIdx.x, ty = blockIdx.y, n = blockIdx.z;
+  const int cy0 = 2 * ty * SP_PH - 1, cx0 = 2 * tx * SP_PW - 1;   // first convolution row / column of the patch
+  if (tid < 64) sBias[tid] = (a.bias && tid < a.OC) ? a.bias[tid] : 0;
+  // wavefront: channel tile (wave & 1), pixel blocks (wave >> 1), + 2, + 4
+  const int ot = wave & 1, bg = wave >> 1;
+  const bool has_tile = ot * 32 < a.OC;   // uniform
+  unsigned rowbase[SP_SLOTS];
+  bool inside[SP_SLOTS];
+#pragma unroll
+  for (int j = 0; j < SP_SLOTS; ++j) {
+    int p = (bg + 2 * j) * 32 + lrow;
+    const bool in_patch = p < SP_PIX;
+    p = in_patch ? p : SP_PIX - 1;
+    const int py = p / SP_CW, px = p - py * SP_CW;
+    const int oh = cy0 + py, ow = cx0 + px;
+    inside[j] = in_patch && oh >= 0 && oh < a.OH && ow >= 0 && ow < a.OW;
+    const int ohc = oh < 0 ? 0 : (oh > a.OH - 1 ? a.OH - 1 : oh), owc = ow < 0 ? 0 : (ow > a.OW - 1 ? a.OW - 1 : ow);
+    rowbase[j] = (unsigned)(((n * a.Hs + ohc * a.SH) * a.Ws + owc * a.SW) * 4);   // a pixel outside computes a neighbour's value, unused
+  }
+  const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  v16i acc[SP_SLOTS];
+#pragma unroll
+  for (int j = 0; j < SP_SLOTS; ++j) acc[j] = zero16;
+  if (has_tile) {
+    // all chunks of a 7-row filter are requested before the first is used: one trip to memory instead of two
+    for (int c0 = 0; c0 < a.nlive; c0 += SP_BATCH) {
+      v4i f[SP_BATCH], x[SP_BATCH][SP_SLOTS];
+#pragma unroll
+      for (int d = 0; d < SP_BATCH; ++d) {
+        const int c = c0 + d;
+        const bool live = c < a.nlive;   // a chunk past the end multiplies the filter's all-zero chunk
+        f[d] = *reinterpret_cast<const v4i*>(wf + ((size_t)(ot * (a.nch + 1) + (live ? c : a.nch)) * 1024 + lane * 16));
+        // 16-byte unit k16 of K: filter row k16 >> sh16, part k16 & sh16 of its window
+        const int k16 = (live ? c : 0) * 2 + lgrp;
+        const unsigned off = (unsigned)((k16 >> a.sh16) * (a.Ws * 4) + (k16 & a.sh16) * 16);
+#pragma unroll
+        for (int j = 0; j < SP_SLOTS; ++j)
+          if (bg + 2 * j < SP_BLOCKS) x[d][j] = *reinterpret_cast<const v4i*>(xs + rowbase[j] + off);
+      }
+#pragma unroll
+      for (int d = 0; d < SP_BATCH; ++d)
+#pragma unroll
+        for (int j = 0; j < SP_SLOTS; ++j)
+          if (bg + 2 * j < SP_BLOCKS) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[d], x[d][j], acc[j], 0, 0, 0);
+    }
+  }
+  __syncthreads();   // bias staged
+  if (has_tile) {
+#pragma unroll
+    for (int j = 0; j < SP_SLOTS; ++j) {
+      if (bg + 2 * j >= SP_BLOCKS) continue;
+      int32_t val[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int4 bv = *reinterpret_cast<const int4*>(sBias + ot * 32 + q * 8 + lgrp * 4);
+        val[q * 4] = wadd(acc[j][q * 4], bv.x); val[q * 4 + 1] = wadd(acc[j][q * 4 + 1], bv.y);
+        val[q * 4 + 2] = wadd(acc[j][q * 4 + 2], bv.z); val[q * 4 + 3] = wadd(acc[j][q * 4 + 3], bv.w);
+      }
+      run_chain(a.chain, val);
+      const int p = (bg + 2 * j) * 32 + lrow;   // < SP_BLOCKS * 32: inside sTile
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t pk = inside[j] ? pack_bytes(val[q * 4], val[q * 4 + 1], val[q * 4 + 2], val[q * 4 + 3]) : 0x80808080u;
+        *reinterpret_cast<uint32_t*>(sTile + p * 64 + ot * 32 + q * 8 + lgrp * 4) = pk;
+      }
+    }
+  }
+  __syncthreads();
+  // ---- the maxima: one thread per pooled pixel and 16 channels
+  if (tid < SP_PH * SP_PW * 4) {
+    const int g16 = tid & 3, q = tid >> 2;
+    const int qy = q / SP_PW, qx = q - qy * SP_PW;
+    const int QY = ty * SP_PH + qy, QX = tx * SP_PW + qx;
+    if (QY < a.QH && QX < a.QW && g16 * 16 < a.ocp) {
+      int4 v[9];
+#pragma unroll
+      for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < 3; ++dx)
+          v[dy * 3 + dx] = *reinterpret_cast<const int4*>(sTile + ((2 * qy + dy) * SP_CW + 2 * qx + dx) * 64 + g16 * 16);
+      const int4 m = max_pool_reduce<9>(v);
+      *reinterpret_cast<int4*>(out + act_offset((int64_t)(n * a.QH + QY) * a.QW + QX, g16 * 16, a.ocp)) = m;
+    }
+  }
+}
+
 // ---------------------------------------------------------------- layer-sequence kernel
 // A run of convolutions of one graph in ONE launch, for batches that divide over the chip's 8 XCDs.
 // Images are independent, so XCD x computes every layer for its own share of the images (pixel range
@@ -2047,6 +2164,39 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   return check_launch("conv_igemm");
 }
 
+
+// ---- row-window convolution + 3x3 stride-2 max-pool: host side
+// Pool geometry is fixed (3x3, stride 2, padding 1); qh, qw are the pool's output extent as the graph gives it.
+bool stem_pool_eligible(int c, int oc, int kh, int kw, int oh, int ow, int qh, int qw) {
+  return stem_eligible(c, kh, kw, 1, 1) && oc >= 32 && oc <= 64 && (oc % 32) == 0 && oh >= 1 && ow >= 1 && qh >= 1 && qw >= 1 &&
+         2 * (qh - 1) - 1 <= oh - 1 && 2 * (qw - 1) - 1 <= ow - 1;   // every window touches the convolution's output
+}
+int stem_pool(const int8_t* xs, const int8_t* wp, const int32_t* bias, const DevChain& chain, int8_t* out, int n, int c, int h,
+              int w, int oc, int kh, int kw, int sh, int sw, int ph, int pw, int qh, int qw, hipStream_t s) {
+  const int oh = (h + 2 * ph - kh) / sh + 1, ow = (w + 2 * pw - kw) / sw + 1;
+  if (!stem_pool_eligible(c, oc, kh, kw, oh, ow, qh, qw)) return arg_error("conv2d_stem_pool3_i8: not eligible");
+  if (((uintptr_t)xs | (uintptr_t)wp | (uintptr_t)out) & 15) return arg_error("conv2d_stem_pool3_i8 alignment");
+  const StemGeom sg = stem_geom(n, h, w, kh, kw, sh, sw, ph, pw);
+  StemPool a = {};
+  a.N = n; a.Hs = sg.hp; a.Ws = sg.wp;
+  a.OH = oh; a.OW = ow; a.QH = qh; a.QW = qw;
+  a.SH = sh; a.SW = sw; a.OC = oc; a.ocp = pad_channels(oc);
+  a.nch = sg.kp / 32;
+  a.nlive = (sg.k + 31) / 32;
+  a.sh16 = sg.row_bytes >> 5;
+  a.tiles_x = (qw + SP_PW - 1) / SP_PW;
+  a.tiles_y = (qh + SP_PH - 1) / SP_PH;
+  a.chain = chain;
+  a.bias = bias;
+  if (n > 65535 || a.tiles_y > 65535 || sg.bytes > INT32_MAX) return arg_error("conv2d_stem_pool3_i8: tensor too large");
+  char desc[128] = "";
+  if (kernel_timing_enabled())
+    snprintf(desc, sizeof(desc), "%dx%d/%d %d->%d in %dx%dx%d out %dx%d + 3x3/2 max-pool -> %dx%d", kh, kw, sh, c, oc, n, h, w, oh, ow, qh, qw);
+  KernelTimer timer("k_conv_stem_pool", 2.0 * n * (double)oh * ow * oc * c * kh * kw, s,
+                    4.0 * n * sg.hp * sg.wp + (double)oc * c * kh * kw + (double)n * qh * qw * oc, desc);
+  k_stem_pool<<<dim3((unsigned)a.tiles_x, (unsigned)a.tiles_y, (unsigned)n), 256, 0, s>>>(xs, wp, out, a);
+  return check_launch("conv2d_stem_pool3_i8");
+}
 
 // ---- layer-sequence launch: host side
 size_t conv_seq_layer_bytes() { return sizeof(SeqLayer); }

@@ -430,6 +430,25 @@ int cvmhip_conv2d_stem_i8(const void* xs, const void* wp, const int32_t* bias, c
   return conv_igemm(reinterpret_cast<const int8_t*>(xs), reinterpret_cast<const int8_t*>(wp), out, g, ep, as_stream(stream));
 }
 
+int cvmhip_conv2d_stem_pool3_i8_eligible(int n, int c, int h, int wd, int oc, int kh, int kw, int stride_h, int stride_w,
+                                         int pad_h, int pad_w, int pool_oh, int pool_ow) {
+  if (n < 1 || h < 1 || wd < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0 || kh < 1 || kw < 1 ||
+      cvmhip_stem_input_bytes(n, h, wd, kh, kw, stride_h, stride_w, pad_h, pad_w) == 0)
+    return 0;
+  return stem_pool_eligible(c, oc, kh, kw, (h + 2 * pad_h - kh) / stride_h + 1, (wd + 2 * pad_w - kw) / stride_w + 1, pool_oh, pool_ow) ? 1 : 0;
+}
+
+int cvmhip_conv2d_stem_pool3_i8(const void* xs, const void* wp, const int32_t* bias, const cvmhip_chain* chain, void* out,
+                                int n, int c, int h, int wd, int oc, int kh, int kw, int stride_h, int stride_w,
+                                int pad_h, int pad_w, int pool_oh, int pool_ow, void* stream) {
+  if (!xs || !wp || !out || !cvmhip_conv2d_stem_pool3_i8_eligible(n, c, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, pool_oh, pool_ow))
+    return arg_error("conv2d_stem_pool3_i8: not eligible");
+  DevChain ch;
+  if (!make_chain(chain, &ch)) return arg_error("conv2d_stem_pool3_i8 chain");
+  return stem_pool(reinterpret_cast<const int8_t*>(xs), reinterpret_cast<const int8_t*>(wp), bias, ch, reinterpret_cast<int8_t*>(out),
+                   n, c, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w, pool_oh, pool_ow, as_stream(stream));
+}
+
 size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw) {
   return ((size_t)pad_channels(c) * kh * kw + 255) / 256 * 256;
 }

@@ -487,6 +487,25 @@ void HipGraphRuntime::BuildPlan() {
         // A 2x2 window with stride 2 and no padding over an even extent, fed by a convolution that nobody else reads:
         // the convolution takes the maximum itself and writes the pooled tensor (the full-resolution one is never stored).
         const int ps = producer_step[xe];
+        // The head of a ResNet: a 3x3 window with stride 2 and padding 1 behind a row-window convolution with 32 or 64
+        // output channels that nobody else reads becomes part of that convolution's launch (at small batches).
+        if (st.out_i8 && hooks_.pool_fuse && ps >= 0 && plan[ps].kind == PlanStep::CONV && plan[ps].dst == xe &&
+            plan[ps].out_i8 && plan[ps].stem && !plan[ps].pool3 && uses[xe].size() == 1 && !is_head[xe] && st.kh == 3 &&
+            st.kw == 3 && st.sh == 2 && st.sw == 2 && st.ph == 1 && st.pw == 1 &&
+            // one workgroup per 4 x 8 pooled pixels: worth it while they all run at once (small batches)
+            (int64_t)plan[ps].n * ((st.oh + 3) / 4) * ((st.ow + 7) / 8) <= 512 &&
+            cvmhip_conv2d_stem_pool3_i8_eligible(plan[ps].n, plan[ps].c, plan[ps].h, plan[ps].w, plan[ps].oc, plan[ps].kh,
+                                                 plan[ps].kw, plan[ps].sh, plan[ps].sw, plan[ps].ph, plan[ps].pw, st.oh, st.ow)) {
+          PlanStep& cs = plan[ps];
+          cs.pool3 = true;
+          cs.oh = st.oh;
+          cs.ow = st.ow;
+          cs.label += "+pool";
+          cs.dst = out0;
+          has_i8[xe] = false;
+          producer_step[out0] = ps;
+          done = true;
+        } else
         if (st.out_i8 && hooks_.pool_fuse && ps >= 0 && plan[ps].kind == PlanStep::CONV && plan[ps].dst == xe &&
             plan[ps].out_i8 && !plan[ps].stem && !plan[ps].nhwc && plan[ps].src2 == kNone && !plan[ps].pool2 &&
             uses[xe].size() == 1 && !is_head[xe] && st.kh == 2 && st.kw == 2 && st.sh == 2 && st.sw == 2 && st.ph == 0 &&
@@ -693,6 +712,12 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
       break;
     case PlanStep::CONV: {
       void* out = st.out_i8 ? i8_ptr_[st.dst] : static_cast<void*>(entry_ptr_[st.dst]);
+      if (st.stem && st.pool3) {
+        Check(cvmhip_conv2d_stem_pool3_i8(static_cast<DeviceBuffer*>(st.aux.get())->ptr, static_cast<DeviceBuffer*>(st.weights.get())->ptr,
+                                          st.bias, &st.chain, out, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh, st.sw, st.ph,
+                                          st.pw, st.oh, st.ow, stream_), "conv2d_stem_pool3_i8");
+        break;
+      }
       if (st.stem) {
         Check(cvmhip_conv2d_stem_i8(static_cast<DeviceBuffer*>(st.aux.get())->ptr, static_cast<DeviceBuffer*>(st.weights.get())->ptr,
                                     st.bias, &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw,

@@ -104,6 +104,8 @@ struct PlanStep {
   size_t ws_bytes = 0;
   bool dw_mfma = false;           // DWCONV through the implicit-GEMM kernel (filter packed as diagonal blocks)
   bool pool2 = false;             // CONV also takes the 2x2 stride-2 max_pool2d that follows it (cvmhip_conv2d_pool2_i8); dst is the pooled tensor
+  bool pool3 = false;             // CONV (stem) also takes the 3x3 stride-2 padding-1 max_pool2d that follows it (cvmhip_conv2d_stem_pool3_i8);
+                                  // dst is the pooled tensor, oh x ow its extent
   bool nhwc = false;              // CONV writes int32 pixel-major rows into a slice of entry dst (a fused detection head)
   int64_t dst_off = 0, img_stride = 0;  // that slice: first element, and elements from one image to the next
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;

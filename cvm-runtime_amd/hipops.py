@@ -449,6 +449,30 @@ def conv2d_i8_nhwc(xp, n, ic, h, w, wp, oc, kh, kw, out, offset, image_stride, b
     return out
 
 
+def conv2d_stem_pool3_eligible(n, c, h, w, oc, kh, kw, strides, padding, pool_oh, pool_ow):
+    return bool(lib().cvmhip_conv2d_stem_pool3_i8_eligible(n, c, h, w, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                                           pool_oh, pool_ow))
+
+
+def conv2d_stem_pool3_i8(x, w, bias, chain1, strides, padding, pool_oh, pool_ow):
+    """Row-window convolution + chain + max_pool2d(3x3, stride 2, padding 1) in one launch; x and w are int32 NCHW / OIHW
+    device tensors; returns the pooled int8 act tensor."""
+    L = lib()
+    n, c, h, wd = x.shape
+    oc, _, kh, kw = w.shape
+    L.cvmhip_stem_input_bytes.restype = ctypes.c_size_t
+    L.cvmhip_packed_stem_weight_bytes.restype = ctypes.c_size_t
+    xs = _workspace(L.cvmhip_stem_input_bytes(n, h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1]), x.device)
+    wp = _workspace(L.cvmhip_packed_stem_weight_bytes(oc, kh, kw), x.device)
+    check(L.cvmhip_pack_stem_input(_ptr(x), _vp(xs), n, c, h, wd, kh, kw, strides[0], strides[1], padding[0], padding[1], _stream()))
+    check(L.cvmhip_pack_stem_weights(_ptr(w), _vp(wp), oc, c, kh, kw, _stream()))
+    out = _act_buffer(n * pool_oh * pool_ow, oc, x.device)
+    check(L.cvmhip_conv2d_stem_pool3_i8(_vp(xs), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None, _vp(out),
+                                        n, c, h, wd, oc, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                        pool_oh, pool_ow, _stream()))
+    return out
+
+
 def pack_depthwise_weights(w):
     c, one, kh, kw = w.shape
     wp = _workspace(lib().cvmhip_packed_depthwise_bytes(c, kh, kw), w.device)

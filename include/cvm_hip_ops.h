@@ -334,6 +334,17 @@ int cvmhip_pack_stem_weights(const int32_t* w, void* wp, int oc, int c, int kh, 
 int cvmhip_conv2d_stem_i8(const void* xs, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                           void* out, int out_is_i8, int n, int c, int h, int wd, int oc, int kh, int kw,
                           int stride_h, int stride_w, int pad_h, int pad_w, void* stream);
+/* The same convolution followed by max_pool2d with a 3x3 window, stride 2 and padding 1 (ops.cc:466-523; the head of a
+ * ResNet) in ONE launch: a workgroup computes the convolution pixels under a patch of 4 x 8 pooled pixels into LDS
+ * (requantised to int8; pixels outside the convolution's output count as the smallest value, like the reference's
+ * INT32_MIN padding) and takes the maxima there.  out: the pooled int8 act tensor (n, oc, pool_oh, pool_ow), with
+ * pool_oh, pool_ow as the graph's shape inference gives them.  Eligible: the convolution is (cvmhip_stem_eligible),
+ * oc is 32 or 64, and every window touches the convolution's output. */
+int cvmhip_conv2d_stem_pool3_i8_eligible(int n, int c, int h, int wd, int oc, int kh, int kw, int stride_h, int stride_w,
+                                         int pad_h, int pad_w, int pool_oh, int pool_ow);
+int cvmhip_conv2d_stem_pool3_i8(const void* xs, const void* wp, const int32_t* bias, const cvmhip_chain* chain, void* out,
+                                int n, int c, int h, int wd, int oc, int kh, int kw, int stride_h, int stride_w,
+                                int pad_h, int pad_w, int pool_oh, int pool_ow, void* stream);
 /* depthwise conv2d (groups == channels == out channels) on int8 act tensors, filter packed by
  * cvmhip_pack_depthwise_weights into [kh*kw][cp] int8 */
 size_t cvmhip_packed_depthwise_bytes(int c, int kh, int kw);

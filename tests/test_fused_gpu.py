@@ -277,6 +277,65 @@ def test_conv2d_stem_i8(case, dev):
     eq(act_to_nchw(out8, n, oc, conv.shape[2], conv.shape[3]), run_chain(conv, stages), "stem int8")
 
 
+STEM_POOL_CASES = [
+    # n, c, h, w, oc, kh, kw, stride, pad, ceil_mode
+    (2, 3, 64, 64, 64, 7, 7, 2, 3, False),    # ResNet stem shape, shrunk: 32x32 -> 16x16, two patches by four
+    (1, 3, 224, 224, 64, 7, 7, 2, 3, False),  # the real one
+    (3, 3, 30, 42, 32, 3, 3, 1, 1, False),    # one channel tile, ragged patches on both axes
+    (1, 1, 19, 23, 64, 5, 3, 1, 0, True),     # odd convolution extent, ceil mode: the last windows hang over the edge
+    (2, 4, 12, 12, 64, 3, 8, 1, 4, False),    # the widest window
+    (1, 3, 9, 9, 64, 3, 3, 2, 1, True),       # 5x5 -> 3x3
+]
+
+
+@pytest.mark.parametrize("case", STEM_POOL_CASES, ids=lambda c: "n%dc%dh%dw%d_o%dk%dx%ds%dp%dceil%d" % c)
+def test_conv2d_stem_with_fused_3x3_max_pool(case, dev):
+    """Row-window convolution -> requantisation -> max_pool2d(3x3, stride 2, padding 1) in one launch against the oracle."""
+    n, c, h, w, oc, kh, kw, st, pd, ceil = case
+    cid = "stempool-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, c, h, w), -127, 127)
+    wt = synth.tensor(cid, "w", (oc, c, kh, kw), -127, 127)
+    b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+    stages = [("relu",), ("cvm_right_shift", 8, 9)] if n != 3 else [("cvm_right_shift", 8, 9)]   # with and without negative values
+    conv = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (1, 1), 1), stages)
+    ref = oracle.max_pool2d(conv, (3, 3), (2, 2), (1, 1), ceil)
+    qh, qw = ref.shape[2:]
+    assert hipops.conv2d_stem_pool3_eligible(n, c, h, w, oc, kh, kw, (st, st), (pd, pd), qh, qw)
+    out = hipops.conv2d_stem_pool3_i8(T(x, dev), T(wt, dev), T(b, dev), hipops.chain(*stages), (st, st), (pd, pd), qh, qw)
+    torch.cuda.synchronize()
+    eq(act_to_nchw(out, n, oc, qh, qw), ref, "stem + 3x3 max-pool")
+
+
+def test_conv2d_stem_pool_eligibility(dev):
+    assert not hipops.conv2d_stem_pool3_eligible(1, 3, 32, 32, 16, 3, 3, (1, 1), (1, 1), 16, 16)    # too few output channels
+    assert not hipops.conv2d_stem_pool3_eligible(1, 3, 32, 32, 96, 3, 3, (1, 1), (1, 1), 16, 16)    # too many
+    assert not hipops.conv2d_stem_pool3_eligible(1, 8, 32, 32, 64, 3, 3, (1, 1), (1, 1), 16, 16)    # not a few-channel input
+    assert not hipops.conv2d_stem_pool3_eligible(1, 3, 32, 32, 64, 3, 3, (1, 1), (1, 1), 18, 16)    # a window past the output
+
+
+def test_planner_folds_the_resnet_head_max_pool(dev):
+    """conv 7x7/2 -> relu -> shift -> max_pool 3x3/2 at the head of a ResNet-50 is one launch; CVM_HIP_POOLFUSE=0 keeps two."""
+    g, heads = graphgen.resnet50(2, width=64, blocks=(1, 1, 1, 1), size=64, classes=20, config_id="stempool-r50")
+    js, pb = g.build(heads)
+    x = synth.tensor("stempool-r50", "data", g.shape((0, 0)), -127, 127)
+    outs, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_POOLFUSE"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = m.inference(x.astype(np.int8).tobytes())
+            launches[mode] = m.launch_counts()[0]
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_POOLFUSE", None)
+    assert outs["1"] == outs["0"]
+    assert launches["1"] == launches["0"] - 1, launches
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
 @pytest.mark.parametrize("cfg", range(8))
 def test_conv2d_stem_i8_every_configuration(cfg, dev):
     """The row-window input layer under every tile / K-split configuration of the wavefront kernel."""
