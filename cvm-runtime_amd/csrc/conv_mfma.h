@@ -76,6 +76,14 @@ struct Epilogue {
   // window (pixel index = 4 * window + 2 * (oh % 2) + ow % 2), so the four values of a window sit in four
   // neighbouring lanes.  Set through conv_igemm_ws only where conv_pool_eligible says so.
   int pool;
+  // int32 output over two destinations: two convolutions over the same input with the same geometry and chain (the
+  // class and box heads of a detector's feature map) computed as one, the second one's filter rows behind the
+  // first one's, which are padded to a multiple of 32.  Output channels [0, split) go to `out` as described above
+  // (oc_a of them exist), channels split .. split + oc_b - 1 to out_b with strides of their own.  split == 0: one destination.
+  int split, oc_a, oc_b;
+  int o32_ch_b, o32_px_b;
+  int64_t o32_img_b;
+  int32_t* out_b;
 };
 
 // ---- int8 activation layout.  Channels are padded to Cp = 4, 8, 16 or a
@@ -194,6 +202,9 @@ int stem_pool(const int8_t* xs, const int8_t* wp, const int32_t* bias, const Dev
               int w, int oc, int kh, int kw, int sh, int sw, int ph, int pw, int qh, int qw, hipStream_t s);
 void weight_dims(int oc, int ic, int kh, int kw, int* ocp, int* kp);
 size_t packed_weight_bytes(int oc, int ic, int kh, int kw);
+// Two filters over the same input packed as one: the first one's 32-row tiles, then the second one's.
+size_t packed_weight_pair_bytes(int oc_a, int oc_b, int ic, int kh, int kw);
+int pack_weights_pair(const int32_t* w_a, int oc_a, const int32_t* w_b, int oc_b, int8_t* wp, int ic, int kh, int kw, hipStream_t s);
 
 size_t packed_depthwise_diag_bytes(int c, int kh, int kw);
 int pack_depthwise_diag(const int32_t* w, int8_t* wp, int c, int kh, int kw, hipStream_t s);

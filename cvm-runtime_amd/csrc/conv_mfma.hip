@@ -239,11 +239,17 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       if (p >= P || p < Plo) continue;
       const int n = (int)fastdiv((unsigned)p, g.div_ohw);
       const int rem = p - n * OHW;
-      const int oc = oc0 + ch[m];
-      int32_t* y32 = reinterpret_cast<int32_t*>(out) + (int64_t)n * ep.o32_img + (int64_t)oc * ep.o32_ch + (int64_t)rem * ep.o32_px;
+      int oc = oc0 + ch[m];
+      // two destinations (Epilogue::split, a multiple of 32, so the four channels of a group share one)
+      const bool second = ep.split > 0 && oc >= ep.split;
+      oc = second ? oc - ep.split : oc;
+      const int limit = second ? ep.oc_b : (ep.split > 0 ? ep.oc_a : g.OC);
+      const int o_ch = second ? ep.o32_ch_b : ep.o32_ch;
+      int32_t* y32 = second ? ep.out_b + (int64_t)n * ep.o32_img_b + (int64_t)oc * ep.o32_ch_b + (int64_t)rem * ep.o32_px_b
+                            : reinterpret_cast<int32_t*>(out) + (int64_t)n * ep.o32_img + (int64_t)oc * ep.o32_ch + (int64_t)rem * ep.o32_px;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (oc + e < g.OC) y32[(int64_t)e * ep.o32_ch] = val[m * 4 + e];
+        if (oc + e < limit) y32[(int64_t)e * o_ch] = val[m * 4 + e];
     }
     return;
   }
@@ -1712,6 +1718,23 @@ size_t packed_weight_bytes(int oc, int ic, int kh, int kw) {
   return (size_t)(ocp / 32) * (kp / 32 + 1) * 1024 + 8192;
 }
 
+size_t packed_weight_pair_bytes(int oc_a, int oc_b, int ic, int kh, int kw) {
+  int ocp, kp;
+  weight_dims(oc_b, ic, kh, kw, &ocp, &kp);
+  // the first filter's tiles, the second one's as pack_weights writes them (rounded up to four), four more that
+  // the large-tile kernel's requests may touch, and the slack of packed_weight_bytes
+  return (size_t)((oc_a + 31) / 32 + ocp / 32 + 4) * (kp / 32 + 1) * 1024 + 8192;
+}
+
+int pack_weights_pair(const int32_t* w_a, int oc_a, const int32_t* w_b, int oc_b, int8_t* wp, int ic, int kh, int kw, hipStream_t s) {
+  int ocp, kp;
+  weight_dims(oc_a, ic, kh, kw, &ocp, &kp);
+  // the first filter is written with its tiles rounded up to four; the second one then overwrites the padding tiles
+  const int rc = pack_weights(w_a, wp, oc_a, ic, kh, kw, s);
+  if (rc) return rc;
+  return pack_weights(w_b, wp + (size_t)((oc_a + 31) / 32) * (kp / 32 + 1) * 1024, oc_b, ic, kh, kw, s);
+}
+
 int pack_activations(const int32_t* x, int8_t* xp, int n, int c, int hw, hipStream_t s) {
   const int cp = pad_channels(c);
   const int64_t npix = (int64_t)n * hw;
@@ -2023,6 +2046,12 @@ static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom&
   } else if (ep.o32_ch < 1 || ep.o32_px < 1 || ep.o32_img < 0) {
     return arg_error("conv int32 output strides");
   }
+  if (ep.split) {
+    if (ep.out_mode != OUT_I32_NCHW || ep.residual || ep.pool || ep.split < 32 || (ep.split % 32) != 0 || ep.oc_a < 1 ||
+        ep.oc_a > ep.split || ep.oc_b < 1 || g.OC != ep.split + ep.oc_b || !ep.out_b || ((uintptr_t)ep.out_b & 3) ||
+        ep.o32_ch_b < 1 || ep.o32_px_b < 1 || ep.o32_img_b < 0 || g.dw || g.row_bytes)
+      return arg_error("conv with two int32 destinations: bad split");
+  }
   if (ep.pool) {   // pixels are numbered window by window (conv_out_pixel)
     if (!conv_pool_eligible(g) || ep.out_mode != OUT_I8_ACT || ep.residual)
       return arg_error("conv with fused 2x2 max-pool: not eligible (int8 pixel-blocked tensors, even output extent, no residual)");
@@ -2076,7 +2105,7 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (wave_ok && force_wave && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced >= 0 && wave_forced < kNumWaveCfgs) cfg = wave_forced;
   if (ep.pool && cfg < 0) cfg = g.OC > 32 ? 3 : 6;   // the tiled kernel has no pooled form
-  const int kslices = ws && !ep.pool ? conv_slices(g, ep) : 1;
+  const int kslices = ws && !ep.pool && !ep.split ? conv_slices(g, ep) : 1;
   if (kslices > 1 && wave_ok) {
     const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
     if (ws_bytes < need || ((uintptr_t)ws & 15)) return arg_error("conv K-slice workspace");

@@ -379,6 +379,47 @@ int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, c
                        pad_h, pad_w, dil_h, dil_w, stream);
 }
 
+size_t cvmhip_packed_weight_pair_bytes(int oc_a, int oc_b, int ic, int kh, int kw) {
+  if (oc_a < 1 || oc_b < 1 || ic < 1 || kh < 1 || kw < 1) return 0;
+  return packed_weight_pair_bytes(oc_a, oc_b, ic, kh, kw);
+}
+
+int cvmhip_pack_weights_pair(const int32_t* w_a, int oc_a, const int32_t* w_b, int oc_b, void* wp, int ic, int kh, int kw, void* stream) {
+  if (!w_a || !w_b || !wp || ((uintptr_t)wp & 15) || oc_a < 1 || oc_b < 1 || ic < 1 || kh < 1 || kw < 1) return arg_error("pack_weights_pair");
+  return pack_weights_pair(w_a, oc_a, w_b, oc_b, reinterpret_cast<int8_t*>(wp), ic, kh, kw, as_stream(stream));
+}
+
+int cvmhip_conv2d_i8_nhwc_pair(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                               int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b, int64_t image_stride_b, int oc_b,
+                               int n, int ic, int h, int wd, int kh, int kw,
+                               int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
+  if (!xp || !wp || !out_a || !out_b) return arg_error("conv2d_i8_nhwc_pair null tensor");
+  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc_a < 1 || oc_b < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+    return arg_error("conv2d_i8_nhwc_pair attributes");
+  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("conv2d_i8_nhwc_pair kernel exceeds input");
+  const int split = (oc_a + 31) / 32 * 32;
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
+  g.OC = split + oc_b;
+  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  if (image_stride_a < (int64_t)g.OH * g.OW * oc_a || image_stride_b < (int64_t)g.OH * g.OW * oc_b)
+    return arg_error("conv2d_i8_nhwc_pair image stride");
+  Epilogue ep = {};
+  ep.bias = bias;
+  if (!make_chain(chain, &ep.chain) || !make_chain(nullptr, &ep.chain2)) return arg_error("conv2d_i8_nhwc_pair chain");
+  ep.out_mode = OUT_I32_NCHW;
+  ep.out_cp = pad_channels(g.OC);
+  ep.o32_img = image_stride_a; ep.o32_ch = 1; ep.o32_px = oc_a;
+  ep.split = split; ep.oc_a = oc_a; ep.oc_b = oc_b;
+  ep.o32_img_b = image_stride_b; ep.o32_ch_b = 1; ep.o32_px_b = oc_b;
+  ep.out_b = out_b;
+  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out_a, g, ep, as_stream(stream));
+}
+
 // ---- row-window convolution over at most 4 input channels (the RGB stem of a network)
 int cvmhip_stem_eligible(int c, int kh, int kw, int dil_h, int dil_w) { return stem_eligible(c, kh, kw, dil_h, dil_w) ? 1 : 0; }
 

@@ -20,6 +20,7 @@
 //     straight into its slice of the concatenated tensor.
 // Every value a later node or the caller can observe is computed by the same
 // integer arithmetic as in node-by-node execution.
+#include <cstring>
 #include <algorithm>
 #include <climits>
 #include <cstdlib>
@@ -327,6 +328,8 @@ void HipGraphRuntime::BuildPlan() {
       PlanStep st;
       st.label = op;
       st.bias = has_bias ? entry_ptr_[entry_id(n.inputs[2])] : nullptr;
+      st.wsrc = we;
+      st.bsrc = has_bias ? entry_id(n.inputs[2]) : kNone;
       bool ok = params_const;
       uint32_t src = xe;
       if (ok && op == "conv2d") {
@@ -411,9 +414,43 @@ void HipGraphRuntime::BuildPlan() {
         st.src2 = kNone;
         Bound b;
         const uint32_t out = follow_chain(out0, &st.chain, &b);
-        if (st.kind == PlanStep::CONV && fuse_head(out, &st)) head_safe[st.dst].push_back(FitsI8(b));
-        else finish_output(&st, out, b);
-        plan.push_back(st);
+        bool paired = false;
+        if (st.kind == PlanStep::CONV && fuse_head(out, &st)) {
+          head_safe[st.dst].push_back(FitsI8(b));
+          // The other head of the same feature map (same input, filter size, strides, padding, dilation and chain):
+          // the two become one convolution whose filter is the first head's rows, padded to a multiple of 32,
+          // followed by the second head's, and whose workgroups write to the slice their channels belong to.
+          for (size_t k = plan.size(); hooks_.head_pair && k-- > 0 && !paired;) {
+            PlanStep& o = plan[k];
+            if (o.kind != PlanStep::CONV || !o.nhwc || o.pair || o.src != st.src || o.n != st.n || o.c != st.c || o.h != st.h ||
+                o.w != st.w || o.kh != st.kh || o.kw != st.kw || o.sh != st.sh || o.sw != st.sw || o.ph != st.ph ||
+                o.pw != st.pw || o.dh != st.dh || o.dw != st.dw || std::memcmp(&o.chain, &st.chain, sizeof(st.chain)) != 0)
+              continue;
+            const int split = (o.oc + 31) / 32 * 32;
+            auto both = std::make_shared<DeviceBuffer>();
+            Check(cvmhip_alloc(&both->ptr, cvmhip_packed_weight_pair_bytes(o.oc, st.oc, st.c, st.kh, st.kw)), "filter buffer");
+            Check(cvmhip_pack_weights_pair(entry_ptr_[o.wsrc], o.oc, entry_ptr_[st.wsrc], st.oc, both->ptr, st.c, st.kh, st.kw, stream_),
+                  "filter pack");
+            auto bias = std::make_shared<DeviceBuffer>();
+            Check(cvmhip_alloc(&bias->ptr, static_cast<size_t>(split + st.oc) * 4), "bias buffer");
+            Check(cvmhip_memset32(bias->ptr, 0, static_cast<size_t>(split + st.oc), stream_), "bias buffer");
+            if (o.bias) Check(cvmhip_copy_d2d(bias->ptr, o.bias, static_cast<size_t>(o.oc) * 4, stream_), "bias copy");
+            if (st.bias)
+              Check(cvmhip_copy_d2d(static_cast<int32_t*>(bias->ptr) + split, st.bias, static_cast<size_t>(st.oc) * 4, stream_), "bias copy");
+            o.weights = both;
+            o.pair_bias = bias;
+            o.pair = true;
+            o.dst2 = st.dst;
+            o.dst_off2 = st.dst_off;
+            o.img_stride2 = st.img_stride;
+            o.oc2 = st.oc;
+            o.label += "+head";
+            paired = true;
+          }
+        } else {
+          finish_output(&st, out, b);
+        }
+        if (!paired) plan.push_back(st);
         done = true;
       }
     } else if (op == "elemwise_add") {
@@ -722,6 +759,14 @@ void HipGraphRuntime::RunStep(PlanStep& st) {
         Check(cvmhip_conv2d_stem_i8(static_cast<DeviceBuffer*>(st.aux.get())->ptr, static_cast<DeviceBuffer*>(st.weights.get())->ptr,
                                     st.bias, &st.chain, out, st.out_i8 ? 1 : 0, st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw,
                                     st.sh, st.sw, st.ph, st.pw, stream_), "conv2d_stem_i8");
+        break;
+      }
+      if (st.nhwc && st.pair) {
+        Check(cvmhip_conv2d_i8_nhwc_pair(i8_ptr_[st.src], static_cast<DeviceBuffer*>(st.weights.get())->ptr,
+                                         static_cast<const int32_t*>(static_cast<DeviceBuffer*>(st.pair_bias.get())->ptr), &st.chain,
+                                         entry_ptr_[st.dst] + st.dst_off, st.img_stride, st.oc, entry_ptr_[st.dst2] + st.dst_off2,
+                                         st.img_stride2, st.oc2, st.n, st.c, st.h, st.w, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw,
+                                         st.dh, st.dw, stream_), "conv2d_i8_nhwc_pair");
         break;
       }
       if (st.nhwc) {

@@ -451,6 +451,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   hooks_.pool_fuse = env("CVM_HIP_POOLFUSE") != "0";
+  hooks_.head_pair = env("CVM_HIP_HEADPAIR") != "0";
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
   hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : kind.rfind("b", 0) == 0 ? 3 : 0;
   if (!cfg.empty() && cfg[0] >= '0' && cfg[0] <= '9') hooks_.wave_cfg = std::atoi(cfg.c_str());

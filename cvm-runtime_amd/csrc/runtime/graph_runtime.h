@@ -108,6 +108,14 @@ struct PlanStep {
                                   // dst is the pooled tensor, oh x ow its extent
   bool nhwc = false;              // CONV writes int32 pixel-major rows into a slice of entry dst (a fused detection head)
   int64_t dst_off = 0, img_stride = 0;  // that slice: first element, and elements from one image to the next
+  // CONV, nhwc: a second head over the same input folded into this launch (cvmhip_conv2d_i8_nhwc_pair): its slice, its
+  // channel count, and the merged bias (the first head's, zeros up to a multiple of 32, the second head's)
+  bool pair = false;
+  uint32_t dst2 = 0;
+  int64_t dst_off2 = 0, img_stride2 = 0;
+  int oc2 = 0;
+  std::shared_ptr<void> pair_bias;
+  uint32_t wsrc = UINT32_MAX, bsrc = UINT32_MAX;   // CONV: entries of the filter and the bias (UINT32_MAX: none)
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;
 };
 
@@ -211,7 +219,7 @@ class HipGraphRuntime {
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;

@@ -473,6 +473,27 @@ def conv2d_stem_pool3_i8(x, w, bias, chain1, strides, padding, pool_oh, pool_ow)
     return out
 
 
+def pack_weights_pair(w_a, w_b):
+    """Two OIHW filters over the same input packed as one (the first one's rows padded to a multiple of 32)."""
+    L = lib()
+    oc_a, ic, kh, kw = w_a.shape
+    oc_b = w_b.shape[0]
+    L.cvmhip_packed_weight_pair_bytes.restype = ctypes.c_size_t
+    wp = _workspace(L.cvmhip_packed_weight_pair_bytes(oc_a, oc_b, ic, kh, kw), w_a.device)
+    check(L.cvmhip_pack_weights_pair(_ptr(w_a), oc_a, _ptr(w_b), oc_b, _vp(wp), ic, kh, kw, _stream()))
+    return wp
+
+
+def conv2d_i8_nhwc_pair(xp, n, ic, h, w, wp, kh, kw, out_a, offset_a, stride_a, oc_a, out_b, offset_b, stride_b, oc_b,
+                        bias=None, chain1=None, strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    """Two detection heads over the same tensor in one launch; see conv2d_i8_nhwc for the meaning of offset / stride."""
+    check(lib().cvmhip_conv2d_i8_nhwc_pair(_vp(xp), _vp(wp), _ptr(bias), ctypes.byref(chain1) if chain1 else None,
+                                           ctypes.c_void_p(out_a.data_ptr() + 4 * offset_a), ctypes.c_int64(stride_a), oc_a,
+                                           ctypes.c_void_p(out_b.data_ptr() + 4 * offset_b), ctypes.c_int64(stride_b), oc_b,
+                                           n, ic, h, w, kh, kw, strides[0], strides[1], padding[0], padding[1],
+                                           dilation[0], dilation[1], _stream()))
+
+
 def pack_depthwise_weights(w):
     c, one, kh, kw = w.shape
     wp = _workspace(lib().cvmhip_packed_depthwise_bytes(c, kh, kw), w.device)

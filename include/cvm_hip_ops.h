@@ -321,6 +321,17 @@ int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, doubl
 int cvmhip_conv2d_i8_nhwc(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                           int32_t* out, int64_t image_stride, int n, int ic, int h, int wd, int oc, int kh, int kw,
                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* Two such convolutions over the SAME input with the same filter size, strides, padding, dilation and chain (the
+ * class and the box head of one feature map of a detector) in ONE launch: the filters are packed behind one another by
+ * cvmhip_pack_weights_pair (the first one's rows padded to a multiple of 32), `bias` has
+ * ceil32(oc_a) + oc_b entries (the first head's, zeros up to the multiple of 32, the second head's) or is NULL, and
+ * every workgroup writes the rows of the head its channels belong to.  Same values as two cvmhip_conv2d_i8_nhwc calls. */
+size_t cvmhip_packed_weight_pair_bytes(int oc_a, int oc_b, int ic, int kh, int kw);
+int cvmhip_pack_weights_pair(const int32_t* w_a, int oc_a, const int32_t* w_b, int oc_b, void* wp, int ic, int kh, int kw, void* stream);
+int cvmhip_conv2d_i8_nhwc_pair(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                               int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b, int64_t image_stride_b, int oc_b,
+                               int n, int ic, int h, int wd, int kh, int kw,
+                               int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
 /* conv2d over at most 4 input channels with kw <= 8, dilation 1 (the RGB stem of a network), in
  * row-window form: the input is packed once per inference into int8 [n][hp][wp][4], zero padded, so
  * that the kw taps x 4 channel bytes of a filter row are one contiguous window and no tap lies

@@ -249,6 +249,59 @@ def test_conv2d_i8_writes_a_detection_head_in_place(case, conv_kernel, dev):
     eq(out.cpu().numpy(), want, "conv2d_i8_nhwc")
 
 
+HEAD_PAIR_CASES = [
+    # n, ic, h, w, oc_a, oc_b, k, pad
+    (1, 64, 8, 8, 84, 16, 3, 1),        # SSD: 4 anchors x (21 classes, 4 coordinates)
+    (2, 128, 5, 7, 126, 24, 3, 1),      # 6 anchors, two images
+    (3, 32, 4, 4, 32, 5, 1, 0),         # the first head ends exactly on a tile boundary
+    (1, 512, 3, 3, 16, 126, 3, 1),      # the small head first, deep K
+    (1, 96, 16, 16, 200, 70, 3, 1),     # both heads span several tiles
+]
+HEAD_PAIR_KERNELS = [("auto", None, None), ("lds", None, None)] + [("wave", str(c), None) for c in range(8)] + [("big", None, t) for t in (1, 2, 3)]
+
+
+@pytest.mark.parametrize("kern", HEAD_PAIR_KERNELS, ids=lambda k: "%s%s%s" % (k[0], "-cfg" + k[1] if k[1] else "", "-tile%d" % k[2] if k[2] else ""))
+@pytest.mark.parametrize("case", HEAD_PAIR_CASES, ids=lambda c: "n%dc%dh%dw%d_a%db%dk%d" % c[:7])
+def test_two_detection_heads_in_one_launch(case, kern, dev):
+    """Two convolutions over the same tensor, each written pixel-major into its own slice of its own concatenated
+    tensor, computed as one convolution: equal to the oracle's two, nothing outside the slices touched."""
+    n, ic, h, w, oc_a, oc_b, k, pd = case
+    cid = "headpair-%s" % (case,)
+    x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+    wa, wb = synth.tensor(cid, "wa", (oc_a, ic, k, k), -127, 127), synth.tensor(cid, "wb", (oc_b, ic, k, k), -127, 127)
+    ba, bb = synth.tensor(cid, "ba", (oc_a,), -32768, 32768), synth.tensor(cid, "bb", (oc_b,), -32768, 32768)
+    ch = [("cvm_right_shift", 8, 9), ("cvm_clip", 8)]
+    wants, outs = [], []
+    for wt, b, before, after in ((wa, ba, 3, 11), (wb, bb, 0, 5)):
+        ref = run_chain(oracle.conv2d(x, wt, b, (1, 1), (pd, pd), (1, 1), 1), ch)
+        part = np.ascontiguousarray(ref.transpose(0, 2, 3, 1)).reshape(n, -1)
+        stride = before + part.shape[1] + after
+        want = np.full((n, stride), 77, np.int32)
+        want[:, before:before + part.shape[1]] = part
+        wants.append((want, before, stride))
+        outs.append(T(np.full((n, stride), 77, np.int32), dev))
+    split = (oc_a + 31) // 32 * 32
+    bias = np.zeros(split + oc_b, np.int32)
+    bias[:oc_a], bias[split:] = ba, bb
+    if kern[0] != "auto":
+        os.environ["CVM_HIP_CONV"] = kern[0]
+    if kern[1]:
+        os.environ["CVM_HIP_WAVECFG"] = kern[1]
+    if kern[2]:
+        os.environ["CVM_HIP_TILE"] = "%d,0" % kern[2]
+    try:
+        hipops.conv2d_i8_nhwc_pair(hipops.pack_act_i8(T(x, dev)), n, ic, h, w, hipops.pack_weights_pair(T(wa, dev), T(wb, dev)), k, k,
+                                   outs[0], wants[0][1], wants[0][2], oc_a, outs[1], wants[1][1], wants[1][2], oc_b,
+                                   T(bias, dev), hipops.chain(*ch), padding=(pd, pd))
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CVM_HIP_CONV", None)
+        os.environ.pop("CVM_HIP_WAVECFG", None)
+        os.environ.pop("CVM_HIP_TILE", None)
+    eq(outs[0].cpu().numpy(), wants[0][0], "first head, %s" % (kern,))
+    eq(outs[1].cpu().numpy(), wants[1][0], "second head, %s" % (kern,))
+
+
 STEM_CASES = [
     # n, c, h, w, oc, kh, kw, stride, pad
     (2, 3, 32, 32, 64, 7, 7, 2, 3),      # ResNet stem shape, shrunk
@@ -672,6 +725,29 @@ def test_planner_folds_2x2_max_pools_into_their_convolutions(dev):
     assert launches["1"] == launches["0"] - 5, launches   # all five pools of a VGG-16 follow an eligible convolution here
     ref = og.run_graph(js, graphgen.load_params(pb), x)
     got = np.frombuffer(outs["1"], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
+def test_planner_pairs_the_two_heads_of_a_feature_map(dev):
+    """The class head and the box head of each SSD feature map run as one launch; CVM_HIP_HEADPAIR=0 keeps two."""
+    g, heads = graphgen.ssd_mobilenet(size=128, alpha=0.5, config_id="headpair-ssd", neg_ids=True)
+    js, pb = g.build(heads)
+    x = synth.tensor("headpair-ssd", "data", g.shape((0, 0)), -127, 127)
+    outs, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_HEADPAIR"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = [m.inference(x.astype(np.int8).tobytes()) for _ in range(2)]
+            launches[mode] = m.launch_counts()[0]
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_HEADPAIR", None)
+    assert outs["1"][0] == outs["0"][0] and outs["1"][1] == outs["1"][0]
+    assert launches["1"] == launches["0"] - 7, launches   # seven feature maps
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"][0], np.int32 if tsize == 4 else np.int8).astype(np.int32)
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
 
 
