@@ -304,7 +304,7 @@ def main():
     n_timed = sum(v["launches"] for v in kt.values())
     pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall * 1e6) / max(n_timed, 1))
     pair_us = {"empty_us": pair_cost_us}
-    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big")}
+    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big", "k_conv_group", "k_conv_stem_pool")}
     dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
     conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
     launches = max(conv["launches"], 1)

@@ -1452,6 +1452,40 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   }
 }
 
+// ---------------------------------------------------------------- independent convolutions in one launch
+// Convolutions with int32 output that do not depend on one another (the detection heads of a network: seven launches
+// of 4 to 128 workgroups each, every one a chain of latencies on a mostly idle chip) as ONE grid.  The table gives
+// layer k the workgroup indices [first_k, first_k + blocks_k); a workgroup looks its layer up, copies the entry to
+// LDS and runs that layer's tile with the 8-wavefront configuration (64 or 32 output channels, K split 8 ways)
+// the table names.  Entries are SeqLayer records; px_per_share holds first_k and ptiles holds blocks_k.
+template <int MODE>
+__device__ __forceinline__ void group_layer_cfg(int cfg, const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g,
+                                                const Epilogue& ep, int pid, int tid, int* sPart, int* sBias) {
+  if (cfg == 0) conv_wave_tile<2, 2, 8, 8, 2, OUT_I32_NCHW, MODE, false, false>(xp, wf, out, g, ep, pid, tid, sPart, sBias);
+  else conv_wave_tile<1, 2, 8, 8, 4, OUT_I32_NCHW, MODE, false, false>(xp, wf, out, g, ep, pid, tid, sPart, sBias);
+}
+
+__global__ void __launch_bounds__(512, 1)
+k_conv_group(const SeqLayer* __restrict__ layers, int nlayers) {
+  __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: the partial sums of a 64 x 64 tile split 8 ways
+  __shared__ __attribute__((aligned(16))) int sBias[64];
+  constexpr int LWORDS = (int)(sizeof(SeqLayer) / 4);
+  __shared__ __attribute__((aligned(16))) uint32_t sLayer[LWORDS];
+  const int tid = threadIdx.x;
+  const int bid = blockIdx.x;
+  int l = 0;
+  for (int k = 1; k < nlayers; ++k)
+    if (bid >= layers[k].px_per_share) l = k;   // first workgroup index of layer k; ascending
+  if (tid < LWORDS) sLayer[tid] = reinterpret_cast<const uint32_t*>(layers + l)[tid];
+  __syncthreads();
+  const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer);
+  const int pid = bid - L.px_per_share;
+  const int cfg = L.kernel / 3, mode = L.kernel - cfg * 3;
+  if (mode == 0) group_layer_cfg<WAVE_IDENT>(cfg, L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+  else if (mode == 1) group_layer_cfg<WAVE_NOPAD>(cfg, L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+  else group_layer_cfg<WAVE_PAD>(cfg, L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+}
+
 // Second step of a K-sliced convolution: out = chain(sum over slices + bias), stored like the epilogue would
 // (int8 activations or int32 NCHW).  One thread per 4 consecutive channels of a pixel.
 template <int OUT>
@@ -2225,6 +2259,50 @@ int stem_pool(const int8_t* xs, const int8_t* wp, const int32_t* bias, const Dev
                     4.0 * n * sg.hp * sg.wp + (double)oc * c * kh * kw + (double)n * qh * qw * oc, desc);
   k_stem_pool<<<dim3((unsigned)a.tiles_x, (unsigned)a.tiles_y, (unsigned)n), 256, 0, s>>>(xs, wp, out, a);
   return check_launch("conv2d_stem_pool3_i8");
+}
+
+// ---- independent convolutions in one launch: host side
+// Fills entry `index` of a host copy of the table for a convolution with int32 output; its workgroups are
+// first_block .. first_block + *blocks - 1 of the launch.  CVMHIP_ERR_ARG "not eligible" when the layer cannot be one.
+int conv_group_layer(void* table, int index, int first_block, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g,
+                     const Epilogue& ep_in, int* blocks) {
+  Epilogue ep;
+  const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
+  if (prc) return prc;
+  const bool nopad = g.PH == 0 && g.PW == 0;
+  if ((g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I32_NCHW || ep.residual || ep.pool ||
+      !(nopad || (g.KH <= 32 && g.KW <= 32)) || first_block < 0)
+    return arg_error("conv_group_layer: not eligible (few-channel input, depthwise, or not an int32 output)");
+  // the 8-wavefront configuration with the tile the usual choice would take
+  const int usual = choose_wave_cfg(g);
+  const int cfg = (usual >= 4 && usual <= 6) || g.OC <= 32 ? 4 : 0;
+  const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
+                       ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
+  const WaveCfg& c = kWaveCfgs[cfg];
+  const int64_t nb = wave_cfg_blocks(c, g);
+  if (nb > 65536) return arg_error("conv_group_layer: not eligible (a layer that fills the chip by itself)");
+  g.octiles = (g.OC + 32 * c.tm - 1) / (32 * c.tm);
+  g.div_octiles = make_fastdiv((uint32_t)g.octiles);
+  SeqLayer& L = reinterpret_cast<SeqLayer*>(table)[index];
+  memset(&L, 0, sizeof(L));
+  L.px_per_share = first_block;
+  L.ptiles = (int)nb;
+  L.kernel = cfg * 3 + (mode == WAVE_IDENT ? 0 : mode == WAVE_NOPAD ? 1 : 2);
+  L.xp = xp;
+  L.wf = wp;
+  L.out = out;
+  L.g = g;
+  L.ep = ep;
+  if (blocks) *blocks = (int)nb;
+  return CVMHIP_OK;
+}
+int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, hipStream_t s) {
+  if (!dev_table || nlayers < 1 || total_blocks < 1 || ((uintptr_t)dev_table & 15)) return arg_error("conv_group_launch");
+  char desc[64];
+  snprintf(desc, sizeof(desc), "%d independent convolutions in one launch, grid %d", nlayers, total_blocks);
+  KernelTimer timer("k_conv_group", ops, s, bytes, desc);
+  k_conv_group<<<(unsigned)total_blocks, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers);
+  return check_launch("conv_group");
 }
 
 // ---- layer-sequence launch: host side

@@ -389,35 +389,67 @@ int cvmhip_pack_weights_pair(const int32_t* w_a, int oc_a, const int32_t* w_b, i
   return pack_weights_pair(w_a, oc_a, w_b, oc_b, reinterpret_cast<int8_t*>(wp), ic, kh, kw, as_stream(stream));
 }
 
+// One or two detection heads over one tensor: launched, or recorded as entry `group_index` of a table of independent
+// convolutions (group_table != NULL; its workgroups begin at first_block, *blocks receives their number).
+static int heads_any(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
+                     int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b, int64_t image_stride_b, int oc_b,
+                     int n, int ic, int h, int wd, int kh, int kw,
+                     int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream,
+                     void* group_table, int group_index, int first_block, int* blocks) {
+  if (!xp || !wp || !out_a) return arg_error("detection heads: null tensor");
+  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc_a < 1 || (out_b && oc_b < 1) || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
+      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
+    return arg_error("detection heads: attributes");
+  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
+    return arg_error("detection heads: kernel exceeds input");
+  const int split = out_b ? (oc_a + 31) / 32 * 32 : 0;
+  ConvGeom g = {};
+  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
+  g.OC = out_b ? split + oc_b : oc_a;
+  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
+  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
+  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
+  if (image_stride_a < (int64_t)g.OH * g.OW * oc_a || (out_b && image_stride_b < (int64_t)g.OH * g.OW * oc_b))
+    return arg_error("detection heads: image stride");
+  Epilogue ep = {};
+  ep.bias = bias;
+  if (!make_chain(chain, &ep.chain) || !make_chain(nullptr, &ep.chain2)) return arg_error("detection heads: chain");
+  ep.out_mode = OUT_I32_NCHW;
+  ep.out_cp = pad_channels(g.OC);
+  ep.o32_img = image_stride_a; ep.o32_ch = 1; ep.o32_px = oc_a;
+  if (out_b) {
+    ep.split = split; ep.oc_a = oc_a; ep.oc_b = oc_b;
+    ep.o32_img_b = image_stride_b; ep.o32_ch_b = 1; ep.o32_px_b = oc_b;
+    ep.out_b = out_b;
+  }
+  if (group_table)
+    return conv_group_layer(group_table, group_index, first_block, reinterpret_cast<const int8_t*>(xp),
+                            reinterpret_cast<const int8_t*>(wp), out_a, g, ep, blocks);
+  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out_a, g, ep, as_stream(stream));
+}
+
 int cvmhip_conv2d_i8_nhwc_pair(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                                int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b, int64_t image_stride_b, int oc_b,
                                int n, int ic, int h, int wd, int kh, int kw,
                                int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream) {
-  if (!xp || !wp || !out_a || !out_b) return arg_error("conv2d_i8_nhwc_pair null tensor");
-  if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc_a < 1 || oc_b < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
-      pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
-    return arg_error("conv2d_i8_nhwc_pair attributes");
-  if (h + 2 * pad_h < dil_h * (kh - 1) + 1 || wd + 2 * pad_w < dil_w * (kw - 1) + 1)
-    return arg_error("conv2d_i8_nhwc_pair kernel exceeds input");
-  const int split = (oc_a + 31) / 32 * 32;
-  ConvGeom g = {};
-  g.N = n; g.H = h; g.W = wd; g.Cp = pad_channels(ic); g.C = ic;
-  g.OC = split + oc_b;
-  g.OH = (h + 2 * pad_h - (dil_h * (kh - 1) + 1)) / stride_h + 1;
-  g.OW = (wd + 2 * pad_w - (dil_w * (kw - 1) + 1)) / stride_w + 1;
-  g.KH = kh; g.KW = kw; g.SH = stride_h; g.SW = stride_w; g.PH = pad_h; g.PW = pad_w; g.DH = dil_h; g.DW = dil_w;
-  if (image_stride_a < (int64_t)g.OH * g.OW * oc_a || image_stride_b < (int64_t)g.OH * g.OW * oc_b)
-    return arg_error("conv2d_i8_nhwc_pair image stride");
-  Epilogue ep = {};
-  ep.bias = bias;
-  if (!make_chain(chain, &ep.chain) || !make_chain(nullptr, &ep.chain2)) return arg_error("conv2d_i8_nhwc_pair chain");
-  ep.out_mode = OUT_I32_NCHW;
-  ep.out_cp = pad_channels(g.OC);
-  ep.o32_img = image_stride_a; ep.o32_ch = 1; ep.o32_px = oc_a;
-  ep.split = split; ep.oc_a = oc_a; ep.oc_b = oc_b;
-  ep.o32_img_b = image_stride_b; ep.o32_ch_b = 1; ep.o32_px_b = oc_b;
-  ep.out_b = out_b;
-  return conv_igemm(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out_a, g, ep, as_stream(stream));
+  if (!out_b) return arg_error("conv2d_i8_nhwc_pair null tensor");
+  return heads_any(xp, wp, bias, chain, out_a, image_stride_a, oc_a, out_b, image_stride_b, oc_b, n, ic, h, wd, kh, kw, stride_h,
+                   stride_w, pad_h, pad_w, dil_h, dil_w, stream, nullptr, 0, 0, nullptr);
+}
+
+size_t cvmhip_conv_group_layer_bytes(void) { return conv_seq_layer_bytes(); }
+
+int cvmhip_conv_group_heads(void* table, int index, int first_block, int* blocks, const void* xp, const void* wp, const int32_t* bias,
+                            const cvmhip_chain* chain, int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b,
+                            int64_t image_stride_b, int oc_b, int n, int ic, int h, int wd, int kh, int kw,
+                            int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w) {
+  if (!table || index < 0 || !blocks) return arg_error("conv_group_heads table");
+  return heads_any(xp, wp, bias, chain, out_a, image_stride_a, oc_a, out_b, image_stride_b, oc_b, n, ic, h, wd, kh, kw, stride_h,
+                   stride_w, pad_h, pad_w, dil_h, dil_w, nullptr, table, index, first_block, blocks);
+}
+
+int cvmhip_conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream) {
+  return conv_group_launch(dev_table, nlayers, total_blocks, ops, bytes, as_stream(stream));
 }
 
 // ---- row-window convolution over at most 4 input channels (the RGB stem of a network)

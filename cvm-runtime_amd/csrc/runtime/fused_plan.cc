@@ -670,6 +670,7 @@ void HipGraphRuntime::BuildPlan() {
   plan_ = std::move(plan);
   fused_ = true;
   if (hooks_.seq) BuildSequences();
+  if (hooks_.head_group) BuildGroups();
 }
 
 // Runs of at least three consecutive convolution steps that a layer-sequence launch can take (batch a multiple
@@ -728,6 +729,58 @@ void HipGraphRuntime::BuildSequences() {
   seq_error_host_ = static_cast<uint32_t*>(host);
   use_seq_ = true;
   CountSequenceModel(+1);
+}
+
+// Consecutive detection-head steps read feature maps and write slices of concatenated tensors, never one another's
+// results, and each is a few workgroups: two or more of them become one launch of independent convolutions.
+void HipGraphRuntime::BuildGroups() {
+  group_at_.assign(plan_.size(), -1);
+  const size_t entry = cvmhip_conv_group_layer_bytes();
+  std::vector<char> table;
+  size_t i = 0;
+  while (i < plan_.size()) {
+    table.clear();
+    int blocks = 0;
+    double ops = 0, bytes = 0;
+    size_t j = i;
+    for (; j < plan_.size(); ++j) {
+      const PlanStep& st = plan_[j];
+      if (st.kind != PlanStep::CONV || !st.nhwc || st.stem) break;
+      table.resize((j - i + 1) * entry);
+      int nb = 0;
+      const int32_t* bias = st.pair ? static_cast<const int32_t*>(static_cast<DeviceBuffer*>(st.pair_bias.get())->ptr) : st.bias;
+      const int rc = cvmhip_conv_group_heads(table.data(), static_cast<int>(j - i), blocks, &nb, i8_ptr_[st.src],
+                                             static_cast<DeviceBuffer*>(st.weights.get())->ptr, bias, &st.chain,
+                                             entry_ptr_[st.dst] + st.dst_off, st.img_stride, st.oc,
+                                             st.pair ? entry_ptr_[st.dst2] + st.dst_off2 : nullptr, st.img_stride2, st.oc2, st.n, st.c,
+                                             st.h, st.w, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw, st.dh, st.dw);
+      if (rc != CVMHIP_OK) break;
+      blocks += nb;
+      const int oh = (st.h + 2 * st.ph - (st.dh * (st.kh - 1) + 1)) / st.sh + 1, ow = (st.w + 2 * st.pw - (st.dw * (st.kw - 1) + 1)) / st.sw + 1;
+      const double px = static_cast<double>(st.n) * oh * ow, oc = st.oc + (st.pair ? st.oc2 : 0);
+      ops += 2.0 * px * oc * st.c * st.kh * st.kw;
+      bytes += static_cast<double>(st.n) * st.h * st.w * st.c + oc * st.c * st.kh * st.kw + 4.0 * px * oc;
+    }
+    const size_t count = j - i;
+    if (count >= 2) {
+      auto buf = std::make_shared<DeviceBuffer>();
+      Check(cvmhip_alloc(&buf->ptr, count * entry), "grouped-heads table");
+      Check(cvmhip_copy_h2d(buf->ptr, table.data(), count * entry, stream_), "grouped-heads table");
+      Check(cvmhip_stream_sync(stream_), "grouped-heads table");   // the host copy goes away
+      GroupRun r;
+      r.first = i;
+      r.last = j - 1;
+      r.owner = buf;
+      r.table = buf->ptr;
+      r.nlayers = static_cast<int>(count);
+      r.blocks = blocks;
+      r.ops = ops;
+      r.bytes = bytes;
+      group_at_[i] = static_cast<int>(groups_.size());
+      groups_.push_back(r);
+    }
+    i = j > i ? j : i + 1;
+  }
 }
 
 void HipGraphRuntime::RunStep(PlanStep& st) {

@@ -452,6 +452,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   hooks_.pool_fuse = env("CVM_HIP_POOLFUSE") != "0";
   hooks_.head_pair = env("CVM_HIP_HEADPAIR") != "0";
+  hooks_.head_group = env("CVM_HIP_HEADGROUP") != "0";
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
   hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : kind.rfind("b", 0) == 0 ? 3 : 0;
   if (!cfg.empty() && cfg[0] >= '0' && cfg[0] <= '9') hooks_.wave_cfg = std::atoi(cfg.c_str());
@@ -466,6 +467,7 @@ void HipGraphRuntime::Release() {
   plan_.clear();
   if (!seqs_.empty()) CountSequenceModel(-1);
   seqs_.clear();
+  groups_.clear();
   if (seq_sync_) { cvmhip_free(seq_sync_); seq_sync_ = nullptr; }
   if (seq_error_host_) { cvmhip_host_free(seq_error_host_); seq_error_host_ = nullptr; }
   execs_.clear();  // releases per-node device state before the stream goes away
@@ -716,7 +718,11 @@ void HipGraphRuntime::Launch() {
   if (fused_) {
     const bool seq = use_seq_;
     for (size_t i = 0; i < plan_.size();) {
-      if (seq && seq_at_[i] >= 0) {
+      if (!group_at_.empty() && group_at_[i] >= 0) {
+        const GroupRun& r = groups_[group_at_[i]];
+        HipCheck(cvmhip_conv_group_launch(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped detection heads");
+        i = r.last + 1;
+      } else if (seq && seq_at_[i] >= 0) {
         const SeqRun& r = seqs_[seq_at_[i]];
         HipCheck(cvmhip_conv_seq_launch(r.table, r.nlayers, seq_sync_, r.ops, r.bytes, stream_), "layer-sequence launch");
         seq_ran_ = true;

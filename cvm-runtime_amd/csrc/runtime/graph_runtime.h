@@ -163,7 +163,9 @@ class HipGraphRuntime {
     int seq = 0, lay = 0;
     if (use_seq_)
       for (const SeqRun& r : seqs_) { ++seq; lay += r.nlayers; }
-    if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq;
+    int grouped = 0;
+    for (const GroupRun& r : groups_) grouped += r.nlayers - 1;
+    if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq - (fused_ ? grouped : 0);
     if (sequences) *sequences = seq;
     if (layers) *layers = lay;
   }
@@ -219,7 +221,7 @@ class HipGraphRuntime {
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;
@@ -245,6 +247,17 @@ class HipGraphRuntime {
     double ops = 0, bytes = 0;          // algorithmic operations and HBM bytes of its layers (for the measurement harness)
   };
   void BuildSequences();
+  // Runs of consecutive detection-head steps (int32 pixel-major output, independent of one another) that share one launch
+  struct GroupRun {
+    size_t first = 0, last = 0;         // plan_ indices, inclusive
+    std::shared_ptr<void> owner;        // device copy of the layer table
+    void* table = nullptr;
+    int nlayers = 0, blocks = 0;
+    double ops = 0, bytes = 0;
+  };
+  void BuildGroups();
+  std::vector<GroupRun> groups_;
+  std::vector<int> group_at_;           // per plan_ index: the group that starts there, or -1
   void CalibrateSequences();            // measures a run with and without sequence launches, keeps the faster
   static void CountSequenceModel(int delta);   // models with sequence launches alive in this process
   void CheckSequences();                // after a synchronisation: did a sequence launch give up?

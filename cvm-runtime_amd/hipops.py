@@ -494,6 +494,45 @@ def conv2d_i8_nhwc_pair(xp, n, ic, h, w, wp, kh, kw, out_a, offset_a, stride_a, 
                                            dilation[0], dilation[1], _stream()))
 
 
+class HeadGroup:
+    """Independent detection-head convolutions that share one launch (cvmhip_conv_group_heads / cvmhip_conv_group_launch)."""
+
+    def __init__(self, device):
+        L = lib()
+        L.cvmhip_conv_group_layer_bytes.restype = ctypes.c_size_t
+        self.entry = L.cvmhip_conv_group_layer_bytes()
+        self.table = bytearray()
+        self.count = 0
+        self.blocks = 0
+        self.device = device
+        self.keep = []
+
+    def add(self, xp, n, ic, h, w, wp, kh, kw, out_a, offset_a, stride_a, oc_a, out_b=None, offset_b=0, stride_b=0, oc_b=0,
+            bias=None, chain1=None, strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+        self.table.extend(bytes(self.entry))
+        buf = (ctypes.c_char * len(self.table)).from_buffer(self.table)
+        nb = ctypes.c_int()
+        _apply_conv_tuning()
+        rc = lib().cvmhip_conv_group_heads(buf, self.count, self.blocks, ctypes.byref(nb), _vp(xp), _vp(wp), _ptr(bias),
+                                           ctypes.byref(chain1) if chain1 else None,
+                                           ctypes.c_void_p(out_a.data_ptr() + 4 * offset_a), ctypes.c_int64(stride_a), oc_a,
+                                           ctypes.c_void_p(out_b.data_ptr() + 4 * offset_b) if out_b is not None else None,
+                                           ctypes.c_int64(stride_b), oc_b, n, ic, h, w, kh, kw, strides[0], strides[1],
+                                           padding[0], padding[1], dilation[0], dilation[1])
+        del buf
+        if rc != 0:
+            del self.table[-self.entry:]
+        check(rc)
+        self.count += 1
+        self.blocks += nb.value
+        self.keep += [xp, wp, bias, out_a, out_b]
+
+    def launch(self):
+        dev = torch.frombuffer(bytearray(self.table), dtype=torch.uint8).to(self.device)
+        check(lib().cvmhip_conv_group_launch(_vp(dev), self.count, self.blocks, ctypes.c_double(0), ctypes.c_double(0), _stream()))
+        torch.cuda.synchronize()
+
+
 def pack_depthwise_weights(w):
     c, one, kh, kw = w.shape
     wp = _workspace(lib().cvmhip_packed_depthwise_bytes(c, kh, kw), w.device)

@@ -332,6 +332,20 @@ int cvmhip_conv2d_i8_nhwc_pair(const void* xp, const void* wp, const int32_t* bi
                                int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b, int64_t image_stride_b, int oc_b,
                                int n, int ic, int h, int wd, int kh, int kw,
                                int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* Detection heads of different feature maps do not depend on one another and are a handful of workgroups each: they can
+ * share ONE launch.  No counterpart in the reference.  Use: fill a host table of n * cvmhip_conv_group_layer_bytes()
+ * bytes with cvmhip_conv_group_heads (entry i describes what cvmhip_conv2d_i8_nhwc -- out_b NULL -- or
+ * cvmhip_conv2d_i8_nhwc_pair with the same arguments would compute; first_block is the sum of the *blocks of the entries
+ * before it; status 10 when the layer cannot be an entry: input channels not padded to 32), copy the table to the device
+ * and call cvmhip_conv_group_launch with the number of entries and the sum of all *blocks.  The entries must not read what
+ * another entry of the same launch writes. */
+size_t cvmhip_conv_group_layer_bytes(void);
+int cvmhip_conv_group_heads(void* table, int index, int first_block, int* blocks, const void* xp, const void* wp, const int32_t* bias,
+                            const cvmhip_chain* chain, int32_t* out_a, int64_t image_stride_a, int oc_a, int32_t* out_b,
+                            int64_t image_stride_b, int oc_b, int n, int ic, int h, int wd, int kh, int kw,
+                            int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+/* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
+int cvmhip_conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream);
 /* conv2d over at most 4 input channels with kw <= 8, dilation 1 (the RGB stem of a network), in
  * row-window form: the input is packed once per inference into int8 [n][hp][wp][4], zero padded, so
  * that the kw taps x 4 channel bytes of a filter row are one contiguous window and no tap lies

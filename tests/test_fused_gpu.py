@@ -302,6 +302,68 @@ def test_two_detection_heads_in_one_launch(case, kern, dev):
     eq(outs[1].cpu().numpy(), wants[1][0], "second head, %s" % (kern,))
 
 
+def test_independent_detection_heads_share_one_launch(dev):
+    """Seven head layers of different feature maps (pairs and single heads, 64- and 32-channel tiles, padded and 1x1) recorded
+    into one table and launched once: every slice equals the oracle, nothing else is touched."""
+    specs = [
+        # n, ic, h, w, oc_a, oc_b (0: single head), k, pad
+        (1, 256, 16, 16, 84, 16, 3, 1),
+        (1, 512, 8, 8, 126, 24, 3, 1),
+        (1, 1024, 4, 4, 126, 24, 3, 1),
+        (1, 64, 6, 5, 20, 0, 3, 1),
+        (1, 128, 2, 2, 84, 16, 3, 1),
+        (1, 96, 1, 1, 40, 0, 1, 0),
+        (1, 32, 9, 9, 16, 100, 1, 0),
+    ]
+    grp = hipops.HeadGroup(dev)
+    checks = []
+    ch = [("cvm_right_shift", 8, 9), ("cvm_clip", 8)]
+    for i, (n, ic, h, w, oc_a, oc_b, k, pd) in enumerate(specs):
+        cid = "headgroup-%d" % i
+        x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+        outs = []
+        ws, bs = [], []
+        for name, oc, before, after in (("a", oc_a, 3 + i, 2), ("b", oc_b, i, 7)):
+            if oc == 0:
+                continue
+            wt = synth.tensor(cid, "w" + name, (oc, ic, k, k), -127, 127)
+            b = synth.tensor(cid, "b" + name, (oc,), -32768, 32768)
+            ref = run_chain(oracle.conv2d(x, wt, b, (1, 1), (pd, pd), (1, 1), 1), ch)
+            part = np.ascontiguousarray(ref.transpose(0, 2, 3, 1)).reshape(n, -1)
+            stride = before + part.shape[1] + after
+            want = np.full((n, stride), 77, np.int32)
+            want[:, before:before + part.shape[1]] = part
+            out = T(np.full((n, stride), 77, np.int32), dev)
+            outs.append((out, before, stride))
+            checks.append((out, want, "%d%s" % (i, name)))
+            ws.append(wt)
+            bs.append(b)
+        xp = hipops.pack_act_i8(T(x, dev))
+        if oc_b:
+            split = (oc_a + 31) // 32 * 32
+            bias = np.zeros(split + oc_b, np.int32)
+            bias[:oc_a], bias[split:] = bs[0], bs[1]
+            grp.add(xp, n, ic, h, w, hipops.pack_weights_pair(T(ws[0], dev), T(ws[1], dev)), k, k, outs[0][0], outs[0][1], outs[0][2], oc_a,
+                    outs[1][0], outs[1][1], outs[1][2], oc_b, T(bias, dev), hipops.chain(*ch), padding=(pd, pd))
+        else:
+            grp.add(xp, n, ic, h, w, hipops.pack_weights(T(ws[0], dev)), k, k, outs[0][0], outs[0][1], outs[0][2], oc_a,
+                    bias=T(bs[0], dev), chain1=hipops.chain(*ch), padding=(pd, pd))
+    assert grp.count == len(specs)
+    grp.launch()
+    for out, want, what in checks:
+        eq(out.cpu().numpy(), want, "grouped head " + what)
+
+
+def test_head_group_refuses_few_channel_inputs(dev):
+    grp = hipops.HeadGroup(dev)
+    x = hipops.pack_act_i8(T(synth.tensor("hg-bad", "x", (1, 16, 4, 4), -127, 127), dev))
+    w = hipops.pack_weights(T(synth.tensor("hg-bad", "w", (8, 16, 1, 1), -127, 127), dev))
+    out = T(np.zeros((1, 128), np.int32), dev)
+    with pytest.raises(CvmHipError):
+        grp.add(x, 1, 16, 4, 4, w, 1, 1, out, 0, 128, 8)
+    assert grp.count == 0
+
+
 STEM_CASES = [
     # n, c, h, w, oc, kh, kw, stride, pad
     (2, 3, 32, 32, 64, 7, 7, 2, 3),      # ResNet stem shape, shrunk
@@ -728,12 +790,37 @@ def test_planner_folds_2x2_max_pools_into_their_convolutions(dev):
     assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
 
 
+def test_planner_groups_the_heads_of_all_feature_maps(dev):
+    """All detection heads of an SSD (consecutive, independent steps) share one launch; CVM_HIP_HEADGROUP=0 keeps one per
+    feature map."""
+    g, heads = graphgen.ssd_mobilenet(size=128, alpha=0.5, config_id="headgroup-ssd", neg_ids=True)
+    js, pb = g.build(heads)
+    x = synth.tensor("headgroup-ssd", "data", g.shape((0, 0)), -127, 127)
+    outs, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_HEADGROUP"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = [m.inference(x.astype(np.int8).tobytes()) for _ in range(3)]
+            launches[mode] = m.launch_counts()[0]
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_HEADGROUP", None)
+    assert outs["1"][0] == outs["0"][0] and outs["1"][1] == outs["1"][0] and outs["1"][2] == outs["1"][0]
+    assert launches["1"] == launches["0"] - 6, launches   # seven paired heads in one launch
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"][0], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
 def test_planner_pairs_the_two_heads_of_a_feature_map(dev):
     """The class head and the box head of each SSD feature map run as one launch; CVM_HIP_HEADPAIR=0 keeps two."""
     g, heads = graphgen.ssd_mobilenet(size=128, alpha=0.5, config_id="headpair-ssd", neg_ids=True)
     js, pb = g.build(heads)
     x = synth.tensor("headpair-ssd", "data", g.shape((0, 0)), -127, 127)
     outs, launches = {}, {}
+    os.environ["CVM_HIP_HEADGROUP"] = "0"   # count the launches of the heads themselves
     for mode in ("1", "0"):
         os.environ["CVM_HIP_HEADPAIR"] = mode
         try:
@@ -744,6 +831,7 @@ def test_planner_pairs_the_two_heads_of_a_feature_map(dev):
             m.close()
         finally:
             os.environ.pop("CVM_HIP_HEADPAIR", None)
+    os.environ.pop("CVM_HIP_HEADGROUP", None)
     assert outs["1"][0] == outs["0"][0] and outs["1"][1] == outs["1"][0]
     assert launches["1"] == launches["0"] - 7, launches   # seven feature maps
     ref = og.run_graph(js, graphgen.load_params(pb), x)
