@@ -220,10 +220,11 @@ size_t conv_slices_workspace_bytes(const ConvGeom& g, const Epilogue& ep);
 // Epilogue::pool: int8 pixel-blocked input and output (channels padded to 32 on both sides), an even output extent,
 // a filter side of at most 32.
 bool conv_pool_eligible(const ConvGeom& g);
-// Independent convolutions with int32 output in one launch (k_conv_group): table entries of conv_seq_layer_bytes() bytes.
+// Independent convolutions in one launch (k_conv_group / k_conv_group8): table entries of conv_seq_layer_bytes() bytes; the
+// entries of one table all have int32 output or all int8 output.
 int conv_group_layer(void* table, int index, int first_block, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g,
                      const Epilogue& ep, int* blocks);
-int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, hipStream_t s);
+int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, int out_is_i8, double ops, double bytes, hipStream_t s);
 int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, void* ws, size_t ws_bytes,
                   hipStream_t s);
 

@@ -1486,6 +1486,34 @@ k_conv_group(const SeqLayer* __restrict__ layers, int nlayers) {
   else group_layer_cfg<WAVE_PAD>(cfg, L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
 }
 
+// The same for convolutions with int8 output (independent layers of a network at a small batch, e.g. the first 1x1 layer
+// and the shortcut projection of a ResNet block, each far fewer workgroups than the chip has CUs): 32-channel tiles, K
+// split 8 ways, 64 KiB of partial sums, so two workgroups share a CU.
+template <int MODE>
+__device__ __forceinline__ void group8_layer(const SeqLayer& L, int pid, int tid, int* sPart, int* sBias) {
+  conv_wave_tile<1, 2, 8, 8, 4, OUT_I8_ACT, MODE, false, false>(L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+}
+__global__ void __launch_bounds__(512, 2)
+k_conv_group8(const SeqLayer* __restrict__ layers, int nlayers) {
+  __shared__ __attribute__((aligned(16))) int sPart[16384];
+  __shared__ __attribute__((aligned(16))) int sBias[32];
+  constexpr int LWORDS = (int)(sizeof(SeqLayer) / 4);
+  __shared__ __attribute__((aligned(16))) uint32_t sLayer[LWORDS];
+  const int tid = threadIdx.x;
+  const int bid = blockIdx.x;
+  int l = 0;
+  for (int k = 1; k < nlayers; ++k)
+    if (bid >= layers[k].px_per_share) l = k;
+  if (tid < LWORDS) sLayer[tid] = reinterpret_cast<const uint32_t*>(layers + l)[tid];
+  __syncthreads();
+  const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer);
+  const int pid = bid - L.px_per_share;
+  const int mode = L.kernel % 3;
+  if (mode == 0) group8_layer<WAVE_IDENT>(L, pid, tid, sPart, sBias);
+  else if (mode == 1) group8_layer<WAVE_NOPAD>(L, pid, tid, sPart, sBias);
+  else group8_layer<WAVE_PAD>(L, pid, tid, sPart, sBias);
+}
+
 // Second step of a K-sliced convolution: out = chain(sum over slices + bias), stored like the epilogue would
 // (int8 activations or int32 NCHW).  One thread per 4 consecutive channels of a pixel.
 template <int OUT>
@@ -2270,12 +2298,13 @@ int conv_group_layer(void* table, int index, int first_block, const int8_t* xp, 
   const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
   if (prc) return prc;
   const bool nopad = g.PH == 0 && g.PW == 0;
-  if ((g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I32_NCHW || ep.residual || ep.pool ||
+  const bool i8 = ep.out_mode == OUT_I8_ACT;
+  if ((g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || (!i8 && ep.residual) || ep.pool ||
       !(nopad || (g.KH <= 32 && g.KW <= 32)) || first_block < 0)
-    return arg_error("conv_group_layer: not eligible (few-channel input, depthwise, or not an int32 output)");
-  // the 8-wavefront configuration with the tile the usual choice would take
+    return arg_error("conv_group_layer: not eligible (few-channel input, depthwise, fused pool)");
+  // the 8-wavefront configuration with the tile the usual choice would take (int8 output: always 32 channels)
   const int usual = choose_wave_cfg(g);
-  const int cfg = (usual >= 4 && usual <= 6) || g.OC <= 32 ? 4 : 0;
+  const int cfg = i8 || (usual >= 4 && usual <= 6) || g.OC <= 32 ? 4 : 0;
   const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
                        ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
   const WaveCfg& c = kWaveCfgs[cfg];
@@ -2296,12 +2325,13 @@ int conv_group_layer(void* table, int index, int first_block, const int8_t* xp, 
   if (blocks) *blocks = (int)nb;
   return CVMHIP_OK;
 }
-int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, hipStream_t s) {
+int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, int out_is_i8, double ops, double bytes, hipStream_t s) {
   if (!dev_table || nlayers < 1 || total_blocks < 1 || ((uintptr_t)dev_table & 15)) return arg_error("conv_group_launch");
   char desc[64];
-  snprintf(desc, sizeof(desc), "%d independent convolutions in one launch, grid %d", nlayers, total_blocks);
+  snprintf(desc, sizeof(desc), "%d independent convolutions in one launch, grid %d%s", nlayers, total_blocks, out_is_i8 ? " i8" : " i32");
   KernelTimer timer("k_conv_group", ops, s, bytes, desc);
-  k_conv_group<<<(unsigned)total_blocks, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers);
+  if (out_is_i8) k_conv_group8<<<(unsigned)total_blocks, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers);
+  else k_conv_group<<<(unsigned)total_blocks, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers);
   return check_launch("conv_group");
 }
 

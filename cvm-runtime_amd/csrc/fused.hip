@@ -271,7 +271,8 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
                          int n, int ic, int h, int wd, int oc, int kh, int kw,
                          int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream,
                          void* ws = nullptr, size_t ws_bytes = 0, size_t* ws_query = nullptr, void* seq_table = nullptr,
-                         int seq_index = 0, int pool = 0, int* pool_query = nullptr) {
+                         int seq_index = 0, int pool = 0, int* pool_query = nullptr, void* group_table = nullptr,
+                         int group_index = 0, int group_first = 0, int* group_blocks = nullptr) {
   if (!xp || !wp || !out) return arg_error("conv2d_i8 null tensor");
   if (n < 1 || ic < 1 || h < 1 || wd < 1 || oc < 1 || kh < 1 || kw < 1 || stride_h < 1 || stride_w < 1 ||
       pad_h < 0 || pad_w < 0 || dil_h < 1 || dil_w < 1)
@@ -305,6 +306,9 @@ static int conv2d_i8_any(const void* xp, const void* wp, const int32_t* bias, co
     *ws_query = nhwc_image_stride >= 0 ? 0 : conv_slices_workspace_bytes(g, ep);
     return CVMHIP_OK;
   }
+  if (group_table)   // describe the launch as one entry of a launch of independent convolutions
+    return conv_group_layer(group_table, group_index, group_first, reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp),
+                            out, g, ep, group_blocks);
   if (seq_table)   // describe the launch as one layer of a layer-sequence launch instead of issuing it
     return conv_seq_layer(seq_table, seq_index, reinterpret_cast<const int8_t*>(xp), reinterpret_cast<const int8_t*>(wp), out, g, ep);
   if (nhwc_image_stride >= 0) ws = nullptr;
@@ -449,7 +453,20 @@ int cvmhip_conv_group_heads(void* table, int index, int first_block, int* blocks
 }
 
 int cvmhip_conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream) {
-  return conv_group_launch(dev_table, nlayers, total_blocks, ops, bytes, as_stream(stream));
+  return conv_group_launch(dev_table, nlayers, total_blocks, 0, ops, bytes, as_stream(stream));
+}
+
+int cvmhip_conv_group_conv_i8(void* table, int index, int first_block, int* blocks, const void* xp, const void* wp, const int32_t* bias,
+                              const cvmhip_chain* chain, const void* residual, const cvmhip_chain* chain2, void* out,
+                              int n, int ic, int h, int wd, int oc, int kh, int kw,
+                              int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w) {
+  if (!table || index < 0 || !blocks) return arg_error("conv_group_conv_i8 table");
+  return conv2d_i8_any(xp, wp, bias, chain, residual, chain2, out, 1, -1, n, ic, h, wd, oc, kh, kw, stride_h, stride_w, pad_h, pad_w,
+                       dil_h, dil_w, nullptr, nullptr, 0, nullptr, nullptr, 0, 0, nullptr, table, index, first_block, blocks);
+}
+
+int cvmhip_conv_group_launch_i8(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream) {
+  return conv_group_launch(dev_table, nlayers, total_blocks, 1, ops, bytes, as_stream(stream));
 }
 
 // ---- row-window convolution over at most 4 input channels (the RGB stem of a network)

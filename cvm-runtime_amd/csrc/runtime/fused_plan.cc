@@ -461,6 +461,35 @@ void HipGraphRuntime::BuildPlan() {
         b.lo = -256;
         b.hi = 254;
         const uint32_t out = follow_chain(out0, &chain, &b);
+        // At batch sizes no layer sequence takes (not a multiple of the sequence kernel's shares), a block whose two
+        // addends are convolutions -- the main path's last layer and the shortcut projection, which reads the block's
+        // input like the main path's first layer does -- is reordered: the projection moves next to that first layer
+        // (the two are then independent neighbours and share a launch, see BuildGroups) and the earlier convolution
+        // takes the add.
+        if (hooks_.conv_group && shape_[ae][0] % cvmhip_conv_seq_shares() != 0) {
+          const int pa = producer_step[ae], pb = producer_step[be];
+          const int late = pa > pb ? pa : pb, early = pa > pb ? pb : pa;
+          const uint32_t le = pa > pb ? ae : be, ee = pa > pb ? be : ae;
+          auto plain = [&](int s, uint32_t e) {
+            return s >= 0 && plan[s].kind == PlanStep::CONV && !plan[s].stem && !plan[s].nhwc && plan[s].out_i8 && plan[s].src2 == kNone &&
+                   !plan[s].pool2 && plan[s].dst == e && uses[e].size() == 1 && !is_head[e];
+          };
+          if (early >= 0 && plain(late, le) && plain(early, ee)) {
+            int first = -1;   // the first convolution of the main path: reads what the late one reads
+            for (int s = 0; s < early && first < 0; ++s)
+              if (plan[s].kind == PlanStep::CONV && !plan[s].stem && plan[s].out_i8 && plan[s].src == plan[late].src) first = s;
+            if (first >= 0) {
+              const int to = first + 1;
+              const PlanStep moved = plan[late];
+              plan.erase(plan.begin() + late);
+              plan.insert(plan.begin() + to, moved);
+              for (int& v : producer_step) {
+                if (v == late) v = to;
+                else if (v >= to && v < late) ++v;
+              }
+            }
+          }
+        }
         // fold into the convolution that produced one addend, when the other addend exists by then
         bool folded = false;
         for (int swap = 0; swap < 2 && !folded; ++swap) {
@@ -670,7 +699,7 @@ void HipGraphRuntime::BuildPlan() {
   plan_ = std::move(plan);
   fused_ = true;
   if (hooks_.seq) BuildSequences();
-  if (hooks_.head_group) BuildGroups();
+  BuildGroups();
 }
 
 // Runs of at least three consecutive convolution steps that a layer-sequence launch can take (batch a multiple
@@ -780,6 +809,64 @@ void HipGraphRuntime::BuildGroups() {
       groups_.push_back(r);
     }
     i = j > i ? j : i + 1;
+  }
+  if (!hooks_.head_group) { groups_.clear(); group_at_.assign(plan_.size(), -1); }
+  // The same for consecutive convolutions with int8 output that do not read one another's results (at a small batch the
+  // first 1x1 layer and the shortcut projection of a ResNet block, which the planner has put side by side), as long as
+  // all of them together are one round of workgroups (two per CU); only when no layer-sequence launch exists, which
+  // covers such layers at its batch sizes.
+  if (!hooks_.conv_group || !seqs_.empty()) return;
+  i = 0;
+  while (i < plan_.size()) {
+    table.clear();
+    int blocks = 0;
+    double ops = 0, bytes = 0;
+    std::vector<uint32_t> written;
+    size_t j = i;
+    for (; j < plan_.size(); ++j) {
+      const PlanStep& st = plan_[j];
+      if (st.kind != PlanStep::CONV || st.stem || st.nhwc || st.ws || !st.out_i8 || st.pool2 || group_at_[j] >= 0) break;
+      bool reads_member = false;
+      for (uint32_t w : written) reads_member = reads_member || st.src == w || st.src2 == w;
+      if (reads_member) break;
+      table.resize((j - i + 1) * entry);
+      int nb = 0;
+      const void* res = st.src2 == kNone ? nullptr : i8_ptr_[st.src2];
+      const int rc = cvmhip_conv_group_conv_i8(table.data(), static_cast<int>(j - i), blocks, &nb, i8_ptr_[st.src],
+                                               static_cast<DeviceBuffer*>(st.weights.get())->ptr, st.bias, &st.chain, res, &st.chain2,
+                                               i8_ptr_[st.dst], st.n, st.c, st.h, st.w, st.oc, st.kh, st.kw, st.sh, st.sw, st.ph, st.pw,
+                                               st.dh, st.dw);
+      if (rc != CVMHIP_OK || blocks + nb > 512) break;
+      blocks += nb;
+      written.push_back(st.dst);
+      const int oh = (st.h + 2 * st.ph - (st.dh * (st.kh - 1) + 1)) / st.sh + 1, ow = (st.w + 2 * st.pw - (st.dw * (st.kw - 1) + 1)) / st.sw + 1;
+      const double px = static_cast<double>(st.n) * oh * ow;
+      ops += 2.0 * px * st.oc * st.c * st.kh * st.kw;
+      bytes += static_cast<double>(st.n) * st.h * st.w * st.c + static_cast<double>(st.oc) * st.c * st.kh * st.kw +
+               px * st.oc * (st.src2 != kNone ? 2.0 : 1.0);
+    }
+    const size_t count = j - i;
+    if (count >= 2) {
+      auto buf = std::make_shared<DeviceBuffer>();
+      Check(cvmhip_alloc(&buf->ptr, count * entry), "grouped-convolutions table");
+      Check(cvmhip_copy_h2d(buf->ptr, table.data(), count * entry, stream_), "grouped-convolutions table");
+      Check(cvmhip_stream_sync(stream_), "grouped-convolutions table");
+      GroupRun r;
+      r.first = i;
+      r.last = j - 1;
+      r.owner = buf;
+      r.table = buf->ptr;
+      r.nlayers = static_cast<int>(count);
+      r.blocks = blocks;
+      r.i8 = true;
+      r.ops = ops;
+      r.bytes = bytes;
+      group_at_[i] = static_cast<int>(groups_.size());
+      groups_.push_back(r);
+      i = j;
+    } else {
+      i = i + 1;
+    }
   }
 }
 

@@ -453,6 +453,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.pool_fuse = env("CVM_HIP_POOLFUSE") != "0";
   hooks_.head_pair = env("CVM_HIP_HEADPAIR") != "0";
   hooks_.head_group = env("CVM_HIP_HEADGROUP") != "0";
+  hooks_.conv_group = env("CVM_HIP_CONVGROUP") != "0";
   const std::string kind = env("CVM_HIP_CONV"), cfg = env("CVM_HIP_WAVECFG"), tile = env("CVM_HIP_TILE");
   hooks_.conv_kernel = kind.rfind("l", 0) == 0 ? 1 : kind.rfind("w", 0) == 0 ? 2 : kind.rfind("b", 0) == 0 ? 3 : 0;
   if (!cfg.empty() && cfg[0] >= '0' && cfg[0] <= '9') hooks_.wave_cfg = std::atoi(cfg.c_str());
@@ -720,7 +721,8 @@ void HipGraphRuntime::Launch() {
     for (size_t i = 0; i < plan_.size();) {
       if (!group_at_.empty() && group_at_[i] >= 0) {
         const GroupRun& r = groups_[group_at_[i]];
-        HipCheck(cvmhip_conv_group_launch(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped detection heads");
+        if (r.i8) HipCheck(cvmhip_conv_group_launch_i8(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped convolutions");
+        else HipCheck(cvmhip_conv_group_launch(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped detection heads");
         i = r.last + 1;
       } else if (seq && seq_at_[i] >= 0) {
         const SeqRun& r = seqs_[seq_at_[i]];

@@ -221,7 +221,7 @@ class HipGraphRuntime {
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true;
+    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true, conv_group = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
   };
   Hooks hooks_;
@@ -253,6 +253,7 @@ class HipGraphRuntime {
     std::shared_ptr<void> owner;        // device copy of the layer table
     void* table = nullptr;
     int nlayers = 0, blocks = 0;
+    bool i8 = false;                    // int8 outputs (k_conv_group8) instead of detection heads
     double ops = 0, bytes = 0;
   };
   void BuildGroups();

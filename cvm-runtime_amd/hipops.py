@@ -527,8 +527,35 @@ class HeadGroup:
         self.blocks += nb.value
         self.keep += [xp, wp, bias, out_a, out_b]
 
-    def launch(self):
+    def add_conv_i8(self, xp, n, ic, h, w, wp, oc, kh, kw, bias=None, chain1=None, residual=None, chain2=None,
+                    strides=(1, 1), padding=(0, 0), dilation=(1, 1)):
+        """An entry with int8 output (what conv2d_i8 would compute); returns the output buffer.  A table holds either such
+        entries or head entries; launch with launch(i8=True)."""
+        oh, ow = conv_out_hw(h, w, kh, kw, strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+        out = _act_buffer(n * oh * ow, oc, xp.device)
+        self.table.extend(bytes(self.entry))
+        buf = (ctypes.c_char * len(self.table)).from_buffer(self.table)
+        nb = ctypes.c_int()
+        _apply_conv_tuning()
+        rc = lib().cvmhip_conv_group_conv_i8(buf, self.count, self.blocks, ctypes.byref(nb), _vp(xp), _vp(wp), _ptr(bias),
+                                             ctypes.byref(chain1) if chain1 else None, _vp(residual),
+                                             ctypes.byref(chain2) if chain2 else None, _vp(out), n, ic, h, w, oc, kh, kw,
+                                             strides[0], strides[1], padding[0], padding[1], dilation[0], dilation[1])
+        del buf
+        if rc != 0:
+            del self.table[-self.entry:]
+        check(rc)
+        self.count += 1
+        self.blocks += nb.value
+        self.keep += [xp, wp, bias, residual, out]
+        return out
+
+    def launch(self, i8=False):
         dev = torch.frombuffer(bytearray(self.table), dtype=torch.uint8).to(self.device)
+        if i8:
+            check(lib().cvmhip_conv_group_launch_i8(_vp(dev), self.count, self.blocks, ctypes.c_double(0), ctypes.c_double(0), _stream()))
+            torch.cuda.synchronize()
+            return
         check(lib().cvmhip_conv_group_launch(_vp(dev), self.count, self.blocks, ctypes.c_double(0), ctypes.c_double(0), _stream()))
         torch.cuda.synchronize()
 

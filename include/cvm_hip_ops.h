@@ -346,6 +346,15 @@ int cvmhip_conv_group_heads(void* table, int index, int first_block, int* blocks
                             int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
 /* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
 int cvmhip_conv_group_launch(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream);
+/* The same for convolutions with int8 output that do not depend on one another (at a small batch the first 1x1 layer and
+ * the shortcut projection of a ResNet block are 50-400 workgroups each): entry i describes what cvmhip_conv2d_i8 with the
+ * same arguments and an int8 output would compute; a table holds either int32 entries or int8 entries, launched by
+ * cvmhip_conv_group_launch or cvmhip_conv_group_launch_i8. */
+int cvmhip_conv_group_conv_i8(void* table, int index, int first_block, int* blocks, const void* xp, const void* wp, const int32_t* bias,
+                              const cvmhip_chain* chain, const void* residual, const cvmhip_chain* chain2, void* out,
+                              int n, int ic, int h, int wd, int oc, int kh, int kw,
+                              int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+int cvmhip_conv_group_launch_i8(const void* dev_table, int nlayers, int total_blocks, double ops, double bytes, void* stream);
 /* conv2d over at most 4 input channels with kw <= 8, dilation 1 (the RGB stem of a network), in
  * row-window form: the input is packed once per inference into int8 [n][hp][wp][4], zero padded, so
  * that the kw taps x 4 channel bytes of a filter row are one contiguous window and no tap lies

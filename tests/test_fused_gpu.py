@@ -354,6 +354,63 @@ def test_independent_detection_heads_share_one_launch(dev):
         eq(out.cpu().numpy(), want, "grouped head " + what)
 
 
+def test_independent_int8_convolutions_share_one_launch(dev):
+    """Convolutions with int8 output that do not depend on one another (a 1x1 layer, a strided projection, a 3x3 layer with a
+    residual, a dilated one) recorded into one table and launched once: each equals the oracle's conv2d + chains."""
+    specs = [
+        # n, ic, h, w, oc, k, stride, pad, dilation, residual
+        (1, 64, 14, 14, 64, 1, 1, 0, 1, False),
+        (1, 64, 14, 14, 256, 1, 2, 0, 1, False),
+        (2, 128, 9, 7, 100, 3, 1, 1, 1, True),
+        (1, 32, 12, 12, 40, 3, 1, 2, 2, False),
+        (3, 256, 4, 4, 512, 1, 1, 0, 1, True),
+    ]
+    grp = hipops.HeadGroup(dev)
+    checks = []
+    ch1, ch2 = [("cvm_right_shift", 8, 11)], [("relu",), ("cvm_right_shift", 8, 1)]
+    for i, (n, ic, h, w, oc, k, st, pd, dl, res) in enumerate(specs):
+        cid = "convgroup-%d" % i
+        x = synth.tensor(cid, "x", (n, ic, h, w), -127, 127)
+        wt = synth.tensor(cid, "w", (oc, ic, k, k), -127, 127)
+        b = synth.tensor(cid, "b", (oc,), -32768, 32768)
+        ref = run_chain(oracle.conv2d(x, wt, b, (st, st), (pd, pd), (dl, dl), 1), ch1)
+        rp = None
+        if res:
+            r = synth.tensor(cid, "r", ref.shape, -127, 127)
+            ref = run_chain(oracle.elemwise("elemwise_add", ref, r), ch2)
+            rp = hipops.pack_act_i8(T(r, dev))
+        out = grp.add_conv_i8(hipops.pack_act_i8(T(x, dev)), n, ic, h, w, hipops.pack_weights(T(wt, dev)), oc, k, k, T(b, dev),
+                              hipops.chain(*ch1), rp, hipops.chain(*ch2) if res else None, (st, st), (pd, pd), (dl, dl))
+        checks.append((out, ref, n, oc))
+    grp.launch(i8=True)
+    for i, (out, ref, n, oc) in enumerate(checks):
+        eq(act_to_nchw(out, n, oc, ref.shape[2], ref.shape[3]), ref, "grouped int8 convolution %d" % i)
+
+
+def test_planner_groups_the_projection_with_the_first_layer_of_its_block(dev):
+    """At a batch no layer sequence takes, the shortcut projection of a ResNet block moves next to the block's first 1x1
+    layer and the two share a launch (one per stage); CVM_HIP_CONVGROUP=0 keeps the graph's order."""
+    g, heads = graphgen.resnet50(3, width=32, blocks=(1, 2, 1, 1), size=64, classes=20, config_id="convgroup-r50")
+    js, pb = g.build(heads)
+    x = synth.tensor("convgroup-r50", "data", g.shape((0, 0)), -127, 127)
+    outs, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["CVM_HIP_CONVGROUP"] = mode
+        try:
+            m = runtime.HipModel(js, pb)
+            outs[mode] = [m.inference(x.astype(np.int8).tobytes()) for _ in range(3)]
+            launches[mode] = m.launch_counts()[0]
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_CONVGROUP", None)
+    assert outs["1"][0] == outs["0"][0] and outs["1"][1] == outs["1"][0] and outs["1"][2] == outs["1"][0]
+    assert launches["1"] == launches["0"] - 4, launches
+    ref = og.run_graph(js, graphgen.load_params(pb), x)
+    got = np.frombuffer(outs["1"][0], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+    assert np.array_equal(got, np.concatenate([r.ravel() for r in ref]))
+
+
 def test_head_group_refuses_few_channel_inputs(dev):
     grp = hipops.HeadGroup(dev)
     x = hipops.pack_act_i8(T(synth.tensor("hg-bad", "x", (1, 16, 4, 4), -127, 127), dev))
