@@ -123,7 +123,7 @@ def layer_table(args, pkg, L, model, title):
             else:
                 seq.append((name, us))
         want = [e["kernel"] for e in step]
-        alias = {"k_max_pool_i8": ("k_max_pool_i8", "k_max_pool_i8x16")}
+        alias = {"k_max_pool_i8": ("k_max_pool_i8", "k_max_pool_i8x16"), "k_conv_group": ("k_conv_group", "k_conv_group8")}
         same = lambda got, w: got == w or got in alias.get(w, ())
         hits, i = [], 0
         while i + per_step <= len(seq):
@@ -149,7 +149,7 @@ def layer_table(args, pkg, L, model, title):
     tot_ops = tot_bytes = 0.0
     excess = []
     for i, (e, u) in enumerate(zip(step, dur)):
-        is_conv = e["kernel"].startswith("k_conv")
+        is_conv = e["kernel"].startswith("k_conv") or e["kernel"] == "k_stem_pool"
         ops = e["work"] if is_conv else 0.0
         byts = e["bytes"] if is_conv else e["work"]
         tot_ops += ops
@@ -304,7 +304,7 @@ def main():
     n_timed = sum(v["launches"] for v in kt.values())
     pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall * 1e6) / max(n_timed, 1))
     pair_us = {"empty_us": pair_cost_us}
-    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big", "k_conv_group", "k_conv_stem_pool")}
+    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big", "k_conv_group", "k_stem_pool")}
     dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
     conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
     launches = max(conv["launches"], 1)

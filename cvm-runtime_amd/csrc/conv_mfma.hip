@@ -2283,7 +2283,7 @@ int stem_pool(const int8_t* xs, const int8_t* wp, const int32_t* bias, const Dev
   char desc[128] = "";
   if (kernel_timing_enabled())
     snprintf(desc, sizeof(desc), "%dx%d/%d %d->%d in %dx%dx%d out %dx%d + 3x3/2 max-pool -> %dx%d", kh, kw, sh, c, oc, n, h, w, oh, ow, qh, qw);
-  KernelTimer timer("k_conv_stem_pool", 2.0 * n * (double)oh * ow * oc * c * kh * kw, s,
+  KernelTimer timer("k_stem_pool", 2.0 * n * (double)oh * ow * oc * c * kh * kw, s,
                     4.0 * n * sg.hp * sg.wp + (double)oc * c * kh * kw + (double)n * qh * qw * oc, desc);
   k_stem_pool<<<dim3((unsigned)a.tiles_x, (unsigned)a.tiles_y, (unsigned)n), 256, 0, s>>>(xs, wp, out, a);
   return check_launch("conv2d_stem_pool3_i8");
