@@ -454,22 +454,43 @@ k_nms_select(const int32_t* __restrict__ valid_count, int32_t* __restrict__ y,
     __syncthreads();
     if (tid < 64) {
       const int l16 = tid & (NMS_BM_WORDS - 1);
-      uint32_t remw = 0, cur[4], nxt[4];
+      // The walk goes block by block (32 rows = one word of the set).  Inside a block only the bits of that word
+      // matter, and they are a chain of scalar steps over the block's rows, using the diagonal block (lane j of
+      // diagv: row 32 B + j, word B).  The rows that acted then OR their whole matrix rows into the set for the
+      // blocks to come -- independent LDS reads spread over the four groups of 16 lanes, off the chain.
+      // (One step per row through the vector registers -- read the set's word, test, OR the row -- took 88 clocks a
+      // row, 16 of the kernel's 21 us for 400 candidates.)
+      uint32_t remw = 0;
+      const int keep_u = __builtin_amdgcn_readfirstlane(keep);   // the chain below is scalar: say so
+      const int nblocks = (keep_u + 31) >> 5;
+      for (int B = 0; B < nblocks; ++B) {
+        const int rowj = B * 32 + (tid & 31);
+        const uint32_t diagv = rowj < keep ? s_mask[rowj * NMS_BM_WORDS + B] : 0u;
+        uint32_t cur = (uint32_t)__builtin_amdgcn_readlane((int)remw, B);
+        const int here = keep_u - B * 32 < 32 ? keep_u - B * 32 : 32;
+        const uint32_t valid = here >= 32 ? 0xffffffffu : (1u << here) - 1u;
+        // 32 steps of three scalar instructions each (test the row's bit, select its diagonal bits or nothing, OR), the
+        // diagonal rows fetched from the lanes beforehand with constant lane numbers.  Only bits behind a row count
+        // (a row never removes an earlier one), so a row's bit is final when the walk passes it and the rows that
+        // acted are the ones whose bit is still clear at the end.
+        uint32_t d[32];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) cur[u] = s_mask[u * NMS_BM_WORDS + l16];
-      for (int i = 0; i < keep; i += 4) {
+        for (int jj = 0; jj < 32; ++jj) d[jj] = (uint32_t)__builtin_amdgcn_readlane((int)diagv, jj) & ~((2u << jj) - 1u);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {  // the next four matrix rows are on their way while these four are decided
-          const int r = i + 4 + u < NMS_BM_ROWS ? i + 4 + u : NMS_BM_ROWS - 1;
-          nxt[u] = s_mask[r * NMS_BM_WORDS + l16];
+        for (int jj = 0; jj < 32; ++jj) cur |= ((cur >> jj) & 1u) ? 0u : d[jj];
+        const uint32_t acted = ~cur & valid;
+        // lane (q, l16), q = lane / 16: word l16 of the rows q, q + 4, ... of the block, eight reads in flight
+        uint32_t acc = 0;
+        const int q = tid >> 4;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int jj = q + 4 * u;
+          const uint32_t w = s_mask[(B * 32 + jj) * NMS_BM_WORDS + l16];   // rows past `keep` lie inside the matrix and never act
+          acc |= ((acted >> jj) & 1u) ? w : 0u;
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int r = i + u;
-          const uint32_t word = (uint32_t)__builtin_amdgcn_readlane((int)remw, r >> 5);
-          if (r < keep && !((word >> (r & 31)) & 1u)) remw |= cur[u];
-          cur[u] = nxt[u];
-        }
+        acc |= (uint32_t)__shfl_xor((int)acc, 16, 64);
+        acc |= (uint32_t)__shfl_xor((int)acc, 32, 64);
+        remw |= acc;
       }
       const int live = keep - l16 * 32;
       const uint32_t e = ~remw & s_pos[l16] & (live >= 32 ? 0xffffffffu : live <= 0 ? 0u : (1u << live) - 1u);
