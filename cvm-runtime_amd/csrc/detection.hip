@@ -37,18 +37,30 @@ __global__ void __launch_bounds__(GVC_CHUNK)
 k_gvc_scatter(const int32_t* __restrict__ x, const int32_t* __restrict__ counts, int32_t* __restrict__ valid_count,
               int32_t* __restrict__ y, int n, int k, int32_t thr, int nchunks) {
   __shared__ int wsum[GVC_CHUNK / 64];
+  __shared__ int s_bef[GVC_CHUNK / 64], s_tot[GVC_CHUNK / 64];
   __shared__ int s_before, s_total;
   const int b = blockIdx.y, chunk = blockIdx.x;
-  if (threadIdx.x == 0) {
+  {
+    // the counts are summed by all threads (one thread walking a hundred of them is a chain of a hundred loads)
     int before = 0, total = 0;
-    for (int c = 0; c < nchunks; ++c) {
+    for (int c = threadIdx.x; c < nchunks; c += GVC_CHUNK) {
       const int v = counts[b * nchunks + c];
-      if (c < chunk) before += v;
+      before += c < chunk ? v : 0;
       total += v;
     }
-    s_before = before;
-    s_total = total;
-    if (chunk == 0) valid_count[b] = total;
+    for (int d = 32; d >= 1; d >>= 1) {
+      before += __shfl_xor(before, d, 64);
+      total += __shfl_xor(total, d, 64);
+    }
+    if ((threadIdx.x & 63) == 0) { s_bef[threadIdx.x >> 6] = before; s_tot[threadIdx.x >> 6] = total; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      before = total = 0;
+      for (int w = 0; w < GVC_CHUNK / 64; ++w) { before += s_bef[w]; total += s_tot[w]; }
+      s_before = before;
+      s_total = total;
+      if (chunk == 0) valid_count[b] = total;
+    }
   }
   const int row = chunk * GVC_CHUNK + threadIdx.x;
   const int32_t* src = x + ((int64_t)b * n + row) * k;
