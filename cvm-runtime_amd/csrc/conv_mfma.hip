@@ -1489,14 +1489,17 @@ k_conv_group(const SeqLayer* __restrict__ layers, int nlayers) {
 // The same for convolutions with int8 output (independent layers of a network at a small batch, e.g. the first 1x1 layer
 // and the shortcut projection of a ResNet block, each far fewer workgroups than the chip has CUs): 32-channel tiles, K
 // split 8 ways, 64 KiB of partial sums, so two workgroups share a CU.
+// (a layer with fewer than two chunks of K per wavefront after an 8-way split runs unsplit instead: its eight
+// wavefronts then take eight pixel tiles side by side)
 template <int MODE>
 __device__ __forceinline__ void group8_layer(const SeqLayer& L, int pid, int tid, int* sPart, int* sBias) {
-  conv_wave_tile<1, 2, 8, 8, 4, OUT_I8_ACT, MODE, false, false>(L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+  if (L.kernel / 3 == 4) conv_wave_tile<1, 2, 8, 8, 4, OUT_I8_ACT, MODE, false, false>(L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
+  else conv_wave_tile<1, 2, 1, 8, 4, OUT_I8_ACT, MODE, false, false>(L.xp, L.wf, L.out, L.g, L.ep, pid, tid, sPart, sBias);
 }
 __global__ void __launch_bounds__(512, 2)
 k_conv_group8(const SeqLayer* __restrict__ layers, int nlayers) {
   __shared__ __attribute__((aligned(16))) int sPart[16384];
-  __shared__ __attribute__((aligned(16))) int sBias[32];
+  __shared__ __attribute__((aligned(16))) int sBias[256];   // unsplit: a copy per wavefront
   constexpr int LWORDS = (int)(sizeof(SeqLayer) / 4);
   __shared__ __attribute__((aligned(16))) uint32_t sLayer[LWORDS];
   const int tid = threadIdx.x;
@@ -2304,10 +2307,14 @@ int conv_group_layer(void* table, int index, int first_block, const int8_t* xp, 
     return arg_error("conv_group_layer: not eligible (few-channel input, depthwise, fused pool)");
   // the 8-wavefront configuration with the tile the usual choice would take (int8 output: always 32 channels)
   const int usual = choose_wave_cfg(g);
-  const int cfg = i8 || (usual >= 4 && usual <= 6) || g.OC <= 32 ? 4 : 0;
+  int cfg = i8 || (usual >= 4 && usual <= 6) || g.OC <= 32 ? 4 : 0;
   const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
                        ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
-  const WaveCfg& c = kWaveCfgs[cfg];
+  // int8 entries with fewer than two chunks per wavefront after the split: eight wavefronts side by side, unsplit
+  static const WaveCfg kUnsplit8 = {1, 2, 1, 8, 2};
+  const bool unsplit = i8 && g.K / 32 < 16;
+  const WaveCfg& c = unsplit ? kUnsplit8 : kWaveCfgs[cfg];
+  if (unsplit) cfg = 8;   // any code but 4: see group8_layer
   const int64_t nb = wave_cfg_blocks(c, g);
   if (nb > 65536) return arg_error("conv_group_layer: not eligible (a layer that fills the chip by itself)");
   g.octiles = (g.OC + 32 * c.tm - 1) / (32 * c.tm);
