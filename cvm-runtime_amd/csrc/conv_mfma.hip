@@ -213,6 +213,42 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   const bool whole = blocked && (NG % 4 == 0);   // whole tiles: 16 bytes per lane
   const bool halves = blocked && NG == 2;         // half a tile (q pair): 8 bytes per lane
 
+  // Fused 2x2 max-pool between registers (Epilogue::pool == 2; the host sets it only for tiles of four pixel blocks, a
+  // pixel-blocked int8 output, no residual and a chain that never decreases when its input grows): the window's
+  // four values are the same register of the tile's four blocks, so the maximum costs three quarters of an
+  // instruction a value, and chain, packing and store then work on a quarter of the values.  Adding the bias first
+  // keeps the reference's wrap-around sum; taking the maximum before a non-decreasing chain changes no result.
+  if constexpr (!RANGE && OUT == OUT_I8_ACT && TN == 4 && NG % 16 == 0) {
+    if (ep.pool == 2) {
+      int8_t* y8p = reinterpret_cast<int8_t*>(out);
+#pragma unroll
+      for (int i = 0; i < NG / 16; ++i) {
+        int32_t red[16];
+#pragma unroll
+        for (int qe = 0; qe < 16; ++qe) {
+          const int32_t a = val[(i * 4 + 0) * 16 + qe], b = val[(i * 4 + 1) * 16 + qe], c = val[(i * 4 + 2) * 16 + qe],
+                        d = val[(i * 4 + 3) * 16 + qe];
+          const int32_t ab = a > b ? a : b, cd = c > d ? c : d;
+          red[qe] = ab > cd ? ab : cd;
+        }
+        run_chain(ep.chain, red);
+        uint32_t a = pack_bytes(red[0], red[1], red[2], red[3]), b = pack_bytes(red[4], red[5], red[6], red[7]),
+                 c = pack_bytes(red[8], red[9], red[10], red[11]), d = pack_bytes(red[12], red[13], red[14], red[15]);
+        half_swap(a, c);
+        half_swap(b, d);
+        uint32_t w[4] = {a, c, b, d};
+        const int tile_first = oc0 + ch_wave + ((u0 >> 4) + i) * 32;
+        const int first = tile_first + lgrp * 16;
+        if (tile_first + 32 > g.OC) mask_channels(w, first, g.OC);
+        const int window = (px_wave >> 2) + lrow;   // px_wave is a multiple of 128: 32 windows per wavefront tile
+        if (px_wave < P && first < ocp) {
+          const v4i pk4 = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+          __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8p + act_offset(window, first, ocp)));
+        }
+      }
+      return;
+    }
+  }
   // one copy of each step, the residual part an update in place under a uniform condition (two
   // alternative paths that meet again cost a register-to-register copy of every value)
   run_chain(ep.chain, val);
@@ -526,7 +562,10 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
 // Image and output coordinates of output pixel index p.  Ordinary order: p = (n * OH + oh) * OW + ow.  With a fused 2x2
 // max-pool (Epilogue::pool) the pixels are numbered window by window, p = 4 * window + 2 * (oh % 2) + ow % 2 with
 // window = (n * OH/2 + oh/2) * OW/2 + ow/2, and the host has set div_ohw and div_ow to divide by OH*OW/4 and OW/2.
-__device__ __forceinline__ void conv_out_pixel(const ConvGeom& g, const bool pool, const unsigned p, int& n, int& oh, int& ow) {
+// pool == 2 (wavefront tiles of four pixel blocks, pixel count a multiple of 128): the four pixels of a window lie in
+// the four blocks of a wavefront's tile at the same lane, p = 128 * (window / 32) + 32 * sub + window % 32, so the
+// maximum is taken between registers.
+__device__ __forceinline__ void conv_out_pixel(const ConvGeom& g, const int pool, const unsigned p, int& n, int& oh, int& ow) {
   const int OHW = g.OH * g.OW;
   if (!pool) {
     n = (int)fastdiv(p, g.div_ohw);
@@ -534,13 +573,14 @@ __device__ __forceinline__ void conv_out_pixel(const ConvGeom& g, const bool poo
     oh = (int)fastdiv((unsigned)rem, g.div_ow);
     ow = rem - oh * g.OW;
   } else {
-    const unsigned q = p >> 2;
+    const unsigned q = pool == 2 ? ((p >> 7) << 5) | (p & 31u) : p >> 2;
+    const unsigned sub = pool == 2 ? (p >> 5) & 3u : p & 3u;
     n = (int)fastdiv(q, g.div_ohw);
     const int rem = (int)q - n * (OHW >> 2);
     const int qh = (int)fastdiv((unsigned)rem, g.div_ow);
     const int qw = rem - qh * (g.OW >> 1);
-    oh = 2 * qh + (int)((p >> 1) & 1u);
-    ow = 2 * qw + (int)(p & 1u);
+    oh = 2 * qh + (int)(sub >> 1);
+    ow = 2 * qw + (int)(sub & 1u);
   }
 }
 
@@ -675,7 +715,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       const bool ok = COH ? (p >= p_begin && p < p_end) : p < P;
       const unsigned pp = ok ? (unsigned)p : 0u;
       int n, oh, ow;
-      conv_out_pixel(g, !COH && MODE != WAVE_ROWS && ep.pool != 0, pp, n, oh, ow);
+      conv_out_pixel(g, (!COH && MODE != WAVE_ROWS) ? ep.pool : 0, pp, n, oh, ow);
       const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
       rowbase[j] = (n * g.H + ih0) * g.W + iw0;
       if (MODE == WAVE_ROWS) rowbase[j] *= 4;   // byte offset of the window of filter row 0 (g.H, g.W: stored size, no padding left)
@@ -1030,7 +1070,7 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
     const bool ok = p < P;
     const unsigned pp = ok ? (unsigned)p : 0u;
     int n, oh, ow;
-    conv_out_pixel(g, ep.pool != 0, pp, n, oh, ow);
+    conv_out_pixel(g, ep.pool, pp, n, oh, ow);
     const int ih0 = oh * g.SH - g.PH, iw0 = ow * g.SW - g.PW;
     rowbase[q] = (n * g.H + ih0) * g.W + iw0;
     unsigned rm, cm;
@@ -2170,6 +2210,11 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
   if (wave_ok && force_wave && cfg < 0) cfg = g.OC > 32 ? 3 : 6;
   if (wave_ok && cfg >= 0 && wave_forced >= 0 && wave_forced < kNumWaveCfgs) cfg = wave_forced;
   if (ep.pool && cfg < 0) cfg = g.OC > 32 ? 3 : 6;   // the tiled kernel has no pooled form
+  // The pool's maximum can be taken between registers (Epilogue::pool = 2, set below for kernels whose wavefront tile
+  // is four pixel blocks wide) when whole wavefront tiles cover the pixels and the chain never decreases as its input
+  // grows, which holds for every stage without a multiplication.
+  bool pool_in_registers = ep.pool != 0 && (g.P % 128) == 0;
+  for (int t = 0; t < ep.chain.count; ++t) pool_in_registers = pool_in_registers && ep.chain.st[t].mul == 1;
   const int kslices = ws && !ep.pool && !ep.split ? conv_slices(g, ep) : 1;
   if (kslices > 1 && wave_ok) {
     const size_t need = (size_t)kslices * g.N * g.OC * g.OH * g.OW * 4;
@@ -2214,6 +2259,7 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
     if (tune.kernel == CONV_KERNEL_BIG && tune.tile_wm >= 1 && tune.tile_wm <= 3 && bcfg >= 0) bcfg = tune.tile_wm - 1;
     if (bcfg >= 0 && kslices <= 1) {
       const BigCfg& c = kBigCfgs[bcfg];
+      if (pool_in_registers && c.tn == 4) ep.pool = 2;
       const int64_t nbig = big_cfg_blocks(c, g);
       if (nbig > 0x7fffffff) return arg_error("conv grid too large");
       g.octiles = (g.OC + c.wgm * c.tm * 32 - 1) / (c.wgm * c.tm * 32);
@@ -2233,6 +2279,7 @@ int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, con
                                 ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
     const int64_t wnb = wave_cfg_blocks(kWaveCfgs[cfg], g);
     if (wnb > 0x7fffffff) return arg_error("conv grid too large");
+    if (pool_in_registers && kWaveCfgs[cfg].tn == 4 && kWaveCfgs[cfg].ksplit == 1) ep.pool = 2;
     g.octiles = (g.OC + 32 * kWaveCfgs[cfg].tm - 1) / (32 * kWaveCfgs[cfg].tm);
     g.div_octiles = make_fastdiv((uint32_t)g.octiles);
     const ConvDesc desc(g, ep, "wave", cfg, mode, (long)wnb);

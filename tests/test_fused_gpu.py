@@ -627,6 +627,9 @@ POOL_FUSED_CASES = [
     (1, 64, 34, 30, 40, 3, 1, 0, 1, True),      # no padding, few channels
     (4, 160, 14, 14, 256, 3, 1, 1, 1, True),    # five channel blocks per tap
     (1, 32, 4, 4, 32, 3, 1, 1, 1, True),        # a single pixel tile, mostly empty
+    (2, 64, 16, 16, 160, 3, 1, 1, 1, True),     # 512 pixels: whole 128-pixel wavefront tiles, the maximum between registers
+    (1, 128, 32, 32, 96, 3, 1, 1, 1, False),    # 1024 pixels, 96 channels (ragged last 128-channel tile of the large-tile kernel)
+    (3, 32, 16, 8, 64, 1, 1, 0, 1, True),       # 384 pixels, 1x1
 ]
 # kernel, wavefront configuration, large tile
 POOL_FUSED_KERNELS = [("auto", None, None)] + [("wave", str(c), None) for c in range(8)] + [("big", None, t) for t in (1, 2, 3)]
