@@ -183,7 +183,7 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
 
 // RANGE: only the pixels [p_begin, p_end) are stored (one share of a layer inside the layer-sequence
 // kernel); the stores are then ordinary ones, because the next layer reads the tensor from this L2.
-template <int TN, int NG, int OUT, bool RANGE = false>
+template <int TN, int NG, int OUT, bool RANGE = false, bool POOLR = false>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
                                               int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
                                               uint32_t (&rp)[NG], int p_begin = 0, int p_end = 0) {
@@ -218,8 +218,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   // four values are the same register of the tile's four blocks, so the maximum costs three quarters of an
   // instruction a value, and chain, packing and store then work on a quarter of the values.  Adding the bias first
   // keeps the reference's wrap-around sum; taking the maximum before a non-decreasing chain changes no result.
-  if constexpr (!RANGE && OUT == OUT_I8_ACT && TN == 4 && NG % 16 == 0) {
-    if (ep.pool == 2) {
+  // (POOLR is a template argument: the same code behind a run-time test made the ordinary epilogue of every
+  // four-block tile slower -- ResNet-50's input layer went from 10 to 30 us)
+  if constexpr (POOLR && !RANGE && OUT == OUT_I8_ACT && TN == 4 && NG % 16 == 0) {
+    {
       int8_t* y8p = reinterpret_cast<int8_t*>(out);
 #pragma unroll
       for (int i = 0; i < NG / 16; ++i) {
@@ -654,7 +656,7 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate) {
   }
 }
 
-template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH>
+template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH, bool POOLR = false>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
@@ -970,10 +972,10 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   }
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT, COH>(val, kw_ * NU, bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
+  finish_groups<TN, NU, OUT, COH, POOLR>(val, kw_ * NU, bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
 }
 
-template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false>
+template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false, bool POOLR = false>
 __global__ void __launch_bounds__(NW * 64, MINW)
 k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
             const ConvGeom g, const Epilogue ep) {
@@ -983,7 +985,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   int pid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
-  conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
+  conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false, POOLR>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
 }
 
 // ---------------------------------------------------------------- large-tile kernel
@@ -1013,7 +1015,7 @@ __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int I, int TM, int TN, int OUT>
+template <int I, int TM, int TN, int OUT, bool POOLR>
 __device__ __forceinline__ void big_epilogue_rows(v16i (&acc)[TM][TN], const int* sBias, int ch_wave, int oc0, int px_wave, int lane,
                                                   void* out, const ConvGeom& g, const Epilogue& ep) {
   if constexpr (I < TM) {
@@ -1024,12 +1026,12 @@ __device__ __forceinline__ void big_epilogue_rows(v16i (&acc)[TM][TN], const int
       for (int e = 0; e < 16; ++e) val[j * 16 + e] = acc[I][j][e];
     uint32_t rp[TN * 4];
     if (ep.residual) load_residual<TN, TN * 4>(rp, I * TN * 4, ch_wave, oc0, px_wave, lane, g, ep);
-    finish_groups<TN, TN * 4, OUT>(val, I * TN * 4, sBias, ch_wave, oc0, px_wave, lane, out, g, ep, rp);
-    big_epilogue_rows<I + 1, TM, TN, OUT>(acc, sBias, ch_wave, oc0, px_wave, lane, out, g, ep);
+    finish_groups<TN, TN * 4, OUT, false, POOLR>(val, I * TN * 4, sBias, ch_wave, oc0, px_wave, lane, out, g, ep, rp);
+    big_epilogue_rows<I + 1, TM, TN, OUT, POOLR>(acc, sBias, ch_wave, oc0, px_wave, lane, out, g, ep);
   }
 }
 
-template <int WGM, int WGN, int TM, int TN, int OUT>
+template <int WGM, int WGN, int TM, int TN, int OUT, bool POOLR = false>
 __global__ void __launch_bounds__(256, (TM * TN <= 8 ? 2 : 1))
 k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out, const ConvGeom g, const Epilogue ep) {
   static_assert(WGM * WGN == 4, "four wavefronts");
@@ -1234,7 +1236,7 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
 
   // ---- epilogue, one row of TN tiles at a time (the row index is a template argument: an accumulator indexed by a
   // loop variable that the compiler does not unroll would be moved to scratch memory as a whole)
-  big_epilogue_rows<0, TM, TN, OUT>(acc, sBias, wm * TM * 32, oc0, px0 + wn * TN * 32, lane, out, g, ep);
+  big_epilogue_rows<0, TM, TN, OUT, POOLR>(acc, sBias, wm * TM * 32, oc0, px0 + wn * TN * 32, lane, out, g, ep);
 }
 
 // ---------------------------------------------------------------- row-window convolution + 3x3 stride-2 max-pool
@@ -2052,6 +2054,14 @@ static int choose_big_cfg(const ConvGeom& g) {
 template <int OUT>
 static void launch_big_out(int cfg, unsigned grid, hipStream_t s, const int8_t* xp, const int8_t* wp, void* out, const ConvGeom& g,
                            const Epilogue& ep) {
+  if constexpr (OUT == OUT_I8_ACT) {
+    if (ep.pool == 2) {   // the maximum of a fused 2x2 pool between registers: instantiations of their own
+      if (cfg == 0) k_conv_big<2, 2, 4, 4, OUT, true><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+      else if (cfg == 1) k_conv_big<2, 2, 2, 4, OUT, true><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+      else k_conv_big<1, 4, 2, 4, OUT, true><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+      return;
+    }
+  }
   if (cfg == 0) k_conv_big<2, 2, 4, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
   else if (cfg == 1) k_conv_big<2, 2, 2, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
   else k_conv_big<1, 4, 2, 4, OUT><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
@@ -2067,7 +2077,14 @@ static void launch_wave(int cfg, int mode, unsigned grid, hipStream_t s, const i
     case 4: launch_wave_cfg<1, 2, 8, 8, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
     case 5: launch_wave_cfg<1, 2, 4, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
     case 6: launch_wave_cfg<1, 2, 1, 4, 4, 2>(mode, grid, s, xp, wp, out, g, ep); break;
-    default: launch_wave_cfg<2, 4, 1, 4, 1, 2>(mode, grid, s, xp, wp, out, g, ep); break;
+    default:
+      if (ep.pool == 2 && ep.out_mode == OUT_I8_ACT) {   // the maximum of a fused 2x2 pool between registers (never the row-window or 1x1-identity mode)
+        if (mode == WAVE_NOPAD) k_conv_wave<2, 4, 1, 4, 1, 2, OUT_I8_ACT, WAVE_NOPAD, false, true><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+        else k_conv_wave<2, 4, 1, 4, 1, 2, OUT_I8_ACT, WAVE_PAD, false, true><<<grid, 256, 0, s>>>(xp, wp, out, g, ep);
+        break;
+      }
+      launch_wave_cfg<2, 4, 1, 4, 1, 2>(mode, grid, s, xp, wp, out, g, ep);
+      break;
   }
 }
 
