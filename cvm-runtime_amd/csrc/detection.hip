@@ -184,6 +184,15 @@ k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_coun
 constexpr int TOPK_THREADS = 1024, TOPK_ROWS = 32, TOPK_WAVES = TOPK_THREADS / 64;  // rows per thread
 constexpr int TOPK_MAX_N = TOPK_THREADS * TOPK_ROWS, TOPK_MAX_K = 2048;
 
+// rows of this wavefront whose key is at least `cand`, over the first RB rows of every lane
+template <int RB>
+__device__ __forceinline__ int topk_count_ge(const uint32_t (&key)[TOPK_ROWS], uint32_t cand) {
+  int c = 0;
+#pragma unroll
+  for (int r = 0; r < RB; ++r) c += __popcll(__ballot(key[r] >= cand));
+  return c;
+}
+
 __global__ void __launch_bounds__(TOPK_THREADS)
 k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, int32_t* __restrict__ rank,
                 int n, int k, int score_index, int topk) {
@@ -205,11 +214,17 @@ k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid
   // scores as unsigned keys that compare like the signed values; rows past the end hold key 0 and are
   // told apart by their index wherever a real key could be 0 too
   uint32_t key[TOPK_ROWS];
+  // All loads are issued before the first result is used (rows past the end re-read the last valid row):
+  // a load under a condition, or with its select right behind it, waits for the one before it, and a
+  // dozen round trips to memory in a row were a third of this kernel.
 #pragma unroll
   for (int r = 0; r < TOPK_ROWS; ++r) {
-    const int i = r * TOPK_THREADS + tid;
-    key[r] = (r < R && i < vc) ? (uint32_t)xb[(int64_t)i * k + score_index] ^ 0x80000000u : 0u;
+    const int i = r * TOPK_THREADS + tid, ic = i < vc ? i : vc - 1;
+    key[r] = (uint32_t)xb[(int64_t)ic * k + score_index];
   }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < TOPK_ROWS; ++r) key[r] = r * TOPK_THREADS + tid < vc ? key[r] ^ 0x80000000u : 0u;
   // Bits above the highest bit in which two live keys differ are common to all keys: the bisection
   // only walks the bits below (8 steps for scores that span 8 bits, whatever their offset).
   uint32_t kand = 0xffffffffu, kor = 0;
@@ -232,11 +247,19 @@ k_nms_topk_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid
   uint32_t T = top_bit >= 0 ? (kor & ~((2u << top_bit) - 1u)) : kor;
   for (int bit = all ? -1 : top_bit; bit >= 0; --bit) {
     const uint32_t cand = T | (1u << bit);
-    int c = 0;
-#pragma unroll
-    for (int r = 0; r < TOPK_ROWS; ++r) {
-      if (r >= R) break;
-      c += __popcll(__ballot(key[r] >= cand));
+    // rows past R hold key 0 < cand; counting in blocks of four rows keeps row tests out of the loop (the
+    // scalar unit, shared by the 16 wavefronts, is what this loop waits for)
+    int c;
+    switch ((R + 3) >> 2) {
+      case 0: c = 0; break;
+      case 1: c = topk_count_ge<4>(key, cand); break;
+      case 2: c = topk_count_ge<8>(key, cand); break;
+      case 3: c = topk_count_ge<12>(key, cand); break;
+      case 4: c = topk_count_ge<16>(key, cand); break;
+      case 5: c = topk_count_ge<20>(key, cand); break;
+      case 6: c = topk_count_ge<24>(key, cand); break;
+      case 7: c = topk_count_ge<28>(key, cand); break;
+      default: c = topk_count_ge<32>(key, cand); break;
     }
     int* part = s_part[bit & 1];
     if (lane == 0) part[wave] = c;
