@@ -1611,13 +1611,18 @@ __global__ void __launch_bounds__(256) k_pack_act(const int32_t* __restrict__ x,
     if (p >= npix) continue;
     const int64_t n = p / hw;
     const int pix = (int)(p - n * hw);
-    uint32_t pack = 0;
+    // four loads in flight (channels past the last re-read it and are masked afterwards): a load under a
+    // condition waits for the one before it
+    int32_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int ch = c0 + j;
-      const int32_t v = ch < c ? x[(n * c + ch) * hw + pix] : 0;
-      pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
+      const int ch = c0 + j < c ? c0 + j : c - 1;
+      v[j] = x[(n * c + ch) * hw + pix];
     }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t pack = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pack |= (c0 + j < c ? (uint32_t)(uint8_t)(int8_t)v[j] : 0u) << (8 * j);
     xp[i] = pack;
   }
 }
@@ -1670,15 +1675,19 @@ __global__ void __launch_bounds__(256) k_pack_stem(const int32_t* __restrict__ x
     const int64_t n = fastdiv(t, div_hp);
     const int p = (int)(t - (unsigned)n * (unsigned)hp);
     const int ih = p - ph, iw = q - pw;
-    uint32_t pack = 0;
-    if (n < nimg && ih >= 0 && ih < h && iw >= 0 && iw < w) {   // the slack behind the last image is cleared
+    // the slack behind the last image and the padding ring are cleared; every thread loads (from the
+    // nearest pixel inside, the last channel again past c) so that its loads are all in flight at once
+    const bool inside = n < nimg && ih >= 0 && ih < h && iw >= 0 && iw < w;
+    const int64_t nc = n < nimg ? n : nimg - 1;
+    const int ihc = ih < 0 ? 0 : (ih < h ? ih : h - 1), iwc = iw < 0 ? 0 : (iw < w ? iw : w - 1);
+    int32_t v[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int32_t v = j < c ? x[((n * c + j) * h + ih) * w + iw] : 0;
-        pack |= (uint32_t)(uint8_t)(int8_t)v << (8 * j);
-      }
-    }
-    xs[i] = pack;
+    for (int j = 0; j < 4; ++j) v[j] = x[((nc * c + (j < c ? j : c - 1)) * h + ihc) * w + iwc];
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t pack = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pack |= (j < c ? (uint32_t)(uint8_t)(int8_t)v[j] : 0u) << (8 * j);
+    xs[i] = inside ? pack : 0u;
   }
 }
 
