@@ -1573,14 +1573,29 @@ __global__ void __launch_bounds__(256) k_slices_finish(const int32_t* __restrict
     const int oc = (int)(i - p * oc4) * 4;
     const int64_t n = p / OHW;
     const int rem = (int)(p - n * OHW);
+    // Every load is issued whatever the channel or slice (clamped, masked afterwards), two slices at a time: a
+    // load under a condition waits for the one before it, and this kernel is a few round trips to memory.
     int32_t v[4];
+    int64_t at[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      int32_t acc = (ep.bias && oc + e < g.OC) ? ep.bias[oc + e] : 0;
-      if (oc + e < g.OC)
-        for (int k = 0; k < kslices; ++k) acc = wadd(acc, part[(int64_t)k * slice_stride + (n * g.OC + oc + e) * OHW + rem]);
-      v[e] = acc;
+      const int ce = oc + e < g.OC ? oc + e : g.OC - 1;
+      at[e] = (n * g.OC + ce) * OHW + rem;
+      v[e] = ep.bias ? ep.bias[ce] : 0;
     }
+    for (int k0 = 0; k0 < kslices; k0 += 2) {
+      const bool two = k0 + 1 < kslices;
+      const int32_t* p0 = part + (int64_t)k0 * slice_stride;
+      const int32_t* p1 = part + (int64_t)(two ? k0 + 1 : k0) * slice_stride;
+      int32_t t0[4], t1[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { t0[e] = p0[at[e]]; t1[e] = p1[at[e]]; }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = wadd(wadd(v[e], t0[e]), two ? t1[e] : 0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = oc + e < g.OC ? v[e] : 0;
     run_chain(ep.chain, v);
     if (OUT == OUT_I32_NCHW) {
       int32_t* y32 = reinterpret_cast<int32_t*>(out) + n * ep.o32_img + (int64_t)oc * ep.o32_ch + (int64_t)rem * ep.o32_px;
@@ -1756,11 +1771,19 @@ k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const 
     int32_t acc[DENSE_MB];
 #pragma unroll
     for (int r = 0; r < DENSE_MB; ++r) acc[r] = 0;
+    // rows past the last one repeat it (their sums are not stored): no load sits under a condition, so the
+    // nine loads of a step are in flight together
+    const int32_t* xr[DENSE_MB];
+#pragma unroll
+    for (int r = 0; r < DENSE_MB; ++r) xr[r] = x + (int64_t)(m0 + (r < rows ? r : rows - 1)) * k;
     for (int t = lane; t < k; t += 64) {
       const int32_t wv = wr[t];
+      int32_t xv[DENSE_MB];
 #pragma unroll
-      for (int r = 0; r < DENSE_MB; ++r)
-        if (r < rows) acc[r] = wadd(acc[r], wmul(x[(int64_t)(m0 + r) * k + t], wv));
+      for (int r = 0; r < DENSE_MB; ++r) xv[r] = xr[r][t];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < DENSE_MB; ++r) acc[r] = wadd(acc[r], wmul(xv[r], wv));
     }
 #pragma unroll
     for (int r = 0; r < DENSE_MB; ++r) {
