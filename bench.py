@@ -24,8 +24,8 @@ PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 # passes summarised in the named file under profiles/ (a counter pass cannot run inside this program, so the
 # figures are carried here; each is reported only for the workload and kernel it was measured on)
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("resnet50", "k_conv_seq", 16): (548.4e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt"),
-    ("vgg16", "k_conv_big", 16): (33.7e6, "profiles/k_conv_big_vgg16_b16_traffic.txt"),
+    ("resnet50", "k_conv_seq", 16): (548.6e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt"),
+    ("vgg16", "k_conv_big", 16): (33.8e6, "profiles/k_conv_big_vgg16_b16_traffic.txt"),
 }
 
 
