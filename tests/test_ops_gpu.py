@@ -319,7 +319,11 @@ def test_non_max_suppression(case, dev):
                                           ((-2 ** 31, -2 ** 31 + 2), 2049, 3000),    # one more: all-pairs ranking
                                           ((0, 1000), 1, 700),
                                           ((-50, 50), 400, 300),                  # top_k above the row count: every row ranked in the list
-                                          ((-2 ** 31, 2 ** 31 - 1), 2048, 2048)]) # ... with the list full
+                                          ((-2 ** 31, 2 ** 31 - 1), 2048, 2048),  # ... with the list full
+                                          ((-2 ** 31, 2 ** 31 - 1), 400, 32768),  # the most rows the selection path takes: 32 per thread
+                                          ((-2 ** 31, -2 ** 31 + 3), 1000, 20000),  # the lowest scores there are, in long runs; 20 rows per thread
+                                          ((-100, 100), 2048, 28700),             # 29 rows per thread, the last block of four partly filled
+                                          ((0, 2 ** 20), 600, 14000)])            # 14 rows per thread
 def test_nms_top_k_selection(score, topk, n, dev):
     """Rows past top_k only need to be known as such; the first top_k must come out in the stable-sort order."""
     x = _boxes("nms-topk-%s-%d" % (score, topk), 2, n, -1, 3, score=score, extent=256)
