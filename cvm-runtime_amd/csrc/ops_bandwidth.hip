@@ -221,12 +221,24 @@ __global__ void __launch_bounds__(256) k_max_pool_3x3s2(const int32_t* __restric
     int32_t m0 = INT32_MIN, m1 = INT32_MIN;
     const int extra = pw ? -1 : 4;                 // the fifth column, relative to 4j
     const bool extra_ok = pw ? j > 0 : 4 * j + 4 < w;
+    // All six loads are issued before the first is used (rows outside the image read the nearest row inside and
+    // are masked afterwards): a load under a condition waits for the one before it.
+    int4 vv[3];
+    int32_t ee[3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int ih = 2 * p + r - ph;
+      const int64_t at = (int64_t)(ih < 0 ? 0 : (ih < h ? ih : h - 1)) * w;
+      vv[r] = *reinterpret_cast<const int4*>(xp + at);
+      ee[r] = xp[at + (extra_ok ? extra : 0)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
       const int ih = 2 * p + r - ph;
       if (ih < 0 || ih >= h) continue;
-      const int4 v = *reinterpret_cast<const int4*>(xp + (int64_t)ih * w);
-      const int32_t e = extra_ok ? xp[(int64_t)ih * w + extra] : INT32_MIN;
+      const int4 v = vv[r];
+      const int32_t e = extra_ok ? ee[r] : INT32_MIN;
       if (pw) {   // windows 4j-1..4j+1 and 4j+1..4j+3
         m0 = max(m0, max(e, max(v.x, v.y)));
         m1 = max(m1, max(v.y, max(v.z, v.w)));
@@ -238,6 +250,28 @@ __global__ void __launch_bounds__(256) k_max_pool_3x3s2(const int32_t* __restric
     int32_t* yp = y + (int64_t)row * ow + 2 * j;
     yp[0] = m0;
     if (2 * j + 1 < ow) yp[1] = m1;
+  }
+}
+
+// 2x2 windows with stride 2 and no padding, every window inside the image, rows a multiple of 4 long and an even
+// number of outputs per row: one thread per pair of adjacent outputs, two aligned 16-byte loads in flight and one
+// 8-byte store, so a wavefront reads and writes whole contiguous KiBs.
+__global__ void __launch_bounds__(256) k_max_pool_2x2s2(const int32_t* __restrict__ x, int32_t* __restrict__ y,
+                                                        uint32_t total_pairs, int h, int w, int oh, int ow) {
+  const uint32_t pairs = (uint32_t)ow >> 1;
+  const uint32_t stride = gridDim.x * blockDim.x;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total_pairs; i += stride) {
+    const uint32_t row = i / pairs;
+    const int j = (int)(i - row * pairs);
+    const uint32_t nc = row / (uint32_t)oh;
+    const int p = (int)(row - nc * (uint32_t)oh);
+    const int32_t* xp = x + (int64_t)nc * h * w + (int64_t)(2 * p) * w + 4 * j;
+    const int4 a = *reinterpret_cast<const int4*>(xp);
+    const int4 b = *reinterpret_cast<const int4*>(xp + w);
+    int2 o;
+    o.x = max(max(a.x, a.y), max(b.x, b.y));
+    o.y = max(max(a.z, a.w), max(b.z, b.w));
+    *reinterpret_cast<int2*>(y + (int64_t)row * ow + 2 * j) = o;
   }
 }
 
@@ -557,6 +591,13 @@ int cvmhip_max_pool2d(const int32_t* x, int32_t* y, int n, int c, int h, int w,
       (((uintptr_t)x) & 15) == 0 && total < INT32_MAX && (int64_t)n * c * h * w < ((int64_t)1 << 40)) {
     const int64_t pairs = (int64_t)n * c * oh * ((ow + 1) / 2);
     k_max_pool_3x3s2<<<grid_for(pairs, 256, 256 * 64), 256, 0, as_stream(stream)>>>(x, y, (uint32_t)pairs, h, w, oh, ow, pad_h, pad_w);
+    return check_launch("max_pool2d");
+  }
+  if (kh == 2 && kw == 2 && stride_h == 2 && stride_w == 2 && pad_h == 0 && pad_w == 0 && (w & 3) == 0 && (ow & 1) == 0 &&
+      2 * ow <= w && 2 * oh <= h && (((uintptr_t)x) & 15) == 0 && (((uintptr_t)y) & 7) == 0 && total < INT32_MAX &&
+      (int64_t)n * c * h * w < ((int64_t)1 << 40)) {
+    const int64_t pairs = total / 2;
+    k_max_pool_2x2s2<<<grid_for(pairs, 256, 256 * 64), 256, 0, as_stream(stream)>>>(x, y, (uint32_t)pairs, h, w, oh, ow);
     return check_launch("max_pool2d");
   }
   const unsigned grid = grid_for(total, 256, 256 * 64);

@@ -189,7 +189,15 @@ def test_broadcast(op, dev):
                                   ((1, 3, 16, 20), (3, 3), (2, 2), (0, 1), False),
                                   ((1, 3, 16, 20), (3, 3), (2, 2), (1, 0), False),
                                   ((2, 3, 12, 12), (3, 3), (2, 2), (1, 1), True),
-                                  ((1, 2, 11, 16), (3, 3), (2, 2), (0, 0), True)])
+                                  ((1, 2, 11, 16), (3, 3), (2, 2), (0, 0), True),
+                                  # 2x2 stride 2 without padding on rows of a multiple of 4 (the paired kernel): an odd
+                                  # height, one pair per row, ceil_mode with a last window past the image (general kernel)
+                                  ((2, 3, 16, 16), (2, 2), (2, 2), (0, 0), False),
+                                  ((1, 5, 9, 12), (2, 2), (2, 2), (0, 0), False),
+                                  ((3, 2, 8, 4), (2, 2), (2, 2), (0, 0), False),
+                                  ((1, 2, 8, 20), (2, 2), (2, 2), (0, 0), True),
+                                  ((1, 2, 7, 12), (2, 2), (2, 2), (0, 0), True),
+                                  ((2, 64, 56, 56), (2, 2), (2, 2), (0, 0), False)])
 def test_max_pool2d(case, dev):
     shape, k, s, p, ceil = case
     x = synth.tensor("pool", str(case), shape, -2 ** 31, 2 ** 31 - 1)
