@@ -171,7 +171,14 @@ __device__ __forceinline__ int4 max_pool_reduce(const int4 (&v)[NT]) {
 // Forced kernel choice of the calling thread (thread-local; automatic by default): which implicit-GEMM kernel,
 // which configuration of the wavefront kernel (-1 = automatic), which tile of the tiled kernel (0 = automatic).
 enum { CONV_KERNEL_AUTO = 0, CONV_KERNEL_LDS = 1, CONV_KERNEL_WAVE = 2, CONV_KERNEL_BIG = 3 };
-struct ConvTuning { int kernel, wave_cfg, tile_wm, tile_wn; };
+struct ConvTuning {
+  int kernel, wave_cfg, tile_wm, tile_wn;
+  // layer-sequence launches: polls after which a wait at a layer boundary gives up
+  int seq_spin_limit;
+  unsigned long long* seq_stamps;   // device memory for time stamps inside sequence launches (nullptr: none), see CVM_SEQ_STAMP
+  int seq_stamp_layers;             // layers it has room for: 256 workgroups x layers x 8 words
+  signed char seq_layer_cfg[64];    // configuration forced for entry i of the next sequence tables (-1: automatic)
+};
 void set_conv_tuning(const ConvTuning& t);
 
 int pad_channels(int c);
@@ -238,6 +245,7 @@ size_t conv_seq_layer_bytes();
 size_t conv_seq_sync_bytes();
 int conv_seq_shares();
 int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep);
+int conv_seq_layer_config(const void* table, int index);   // configuration of the tile kernel chosen for an entry
 int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s);
 
 }  // namespace cvmhip

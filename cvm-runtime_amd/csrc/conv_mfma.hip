@@ -643,6 +643,10 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate) {
   if (!gate.counter) return;
   unsigned v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
   int spins = 0;
+  if (v < gate.target && gate.spin_limit <= 0) {   // no patience at all (the host's test of its fall-back): give up at once
+    __hip_atomic_store(gate.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
   while (v < gate.target) {
     __builtin_amdgcn_s_sleep(1);
     v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
@@ -656,11 +660,26 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate) {
   }
 }
 
+// Optional time stamps of a layer inside a layer-sequence launch (cvmhip_set_seq_stamps): eight 64-bit words per
+// workgroup and layer -- 0 tile entered, 1 boundary passed, 2 first operand batch multiplied, 3 K loop done, 4 K-split
+// exchange done, 5 epilogue issued, 6 counted out, 7 layer begun -- written by the workgroup's first thread for the
+// first tile of the layer.  A null pointer (the normal case) costs a scalar branch per stamp.
+#define CVM_SEQ_STAMP(i, dep)                                              \
+  do {                                                                     \
+    if constexpr (COH) {                                                   \
+      if (tr) {                                                            \
+        asm volatile("" ::"v"(dep));                                       \
+        if (tid == 0) tr[i] = __builtin_amdgcn_s_memtime();                \
+      }                                                                    \
+    }                                                                      \
+  } while (0)
 template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH, bool POOLR = false>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
-                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0}) {
+                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0},
+                                               unsigned long long* tr = nullptr) {
+  CVM_SEQ_STAMP(0, tid);
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
   constexpr int BM = 32 * TM;             // output channels per workgroup
   constexpr int WPIX = 32 * TN;           // pixels per wavefront
@@ -784,6 +803,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   auto pass_gate = [&]() __attribute__((always_inline)) {
     if constexpr (COH) {
       gate_wait(gate);
+      CVM_SEQ_STAMP(1, tid);
     }
   };
   auto fetch = [&](const bool gated) __attribute__((always_inline)) -> regs_t {
@@ -921,10 +941,12 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     // bound by exactly that.
     residual_coh();
     consume(R0, true);
+    CVM_SEQ_STAMP(2, acc[0][0][0]);
   } else {
     regs_t R1 = fetch(false);
     residual_coh();
     consume(R0, true);
+    CVM_SEQ_STAMP(2, acc[0][0][0]);
     for (int it = 1; it < niter; it += 2) {
       R0 = fetch(false);
       consume(R1, false);
@@ -933,6 +955,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       consume(R0, false);
     }
   }
+  CVM_SEQ_STAMP(3, acc[0][0][0]);
   if (bias_lane < BM) bias_lds[bias_lane] = bias_mine;
 
   // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
@@ -970,9 +993,11 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
 #pragma unroll
         for (int e = 0; e < 16; ++e) val[((i * TN + j) * 16 + e) % (NU * 4)] = acc[i][j][e];
   }
+  CVM_SEQ_STAMP(4, val[0]);
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
   finish_groups<TN, NU, OUT, COH, POOLR>(val, kw_ * NU, bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
+  CVM_SEQ_STAMP(5, tid);
 }
 
 template <int TM, int TN, int KSPLIT, int NW, int D, int MINW, int OUT, int MODE, bool SLICES = false, bool POOLR = false>
@@ -1389,7 +1414,7 @@ enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
 template <int TM, int TN, int KSPLIT, int NW, int D, int MODE>
 __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                                 int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
-                                                int p_end, const LayerGate gate) {
+                                                int p_end, const LayerGate gate, unsigned long long* tr) {
   constexpr int UNITS = 8 / NW;   // tiles a workgroup computes side by side
   const int half = UNITS == 2 ? (tid >> 8) : 0;
   const int htid = UNITS == 2 ? (tid & 255) : tid;
@@ -1397,7 +1422,7 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
     conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
                                                                          sPart + half * 16384, sBias + half * 256, p_begin, p_end,
-                                                                         base == 0 ? gate : LayerGate{nullptr, 0, nullptr, 0});
+                                                                         base == 0 ? gate : LayerGate{nullptr, 0, nullptr, 0}, base == 0 ? tr : nullptr);
     if (KSPLIT > 1) __syncthreads();   // the next tile reuses the LDS of the partial sums
   }
 }
@@ -1405,20 +1430,21 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
 template <int MODE>
 __device__ __forceinline__ void seq_layer_cfg(int cfg, const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                               int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
-                                              int p_end, const LayerGate gate) {
+                                              int p_end, const LayerGate gate, unsigned long long* tr) {
   switch (cfg) {
-    case 0: seq_layer_tiles<2, 2, 8, 8, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    case 1: seq_layer_tiles<2, 2, 4, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    case 2: seq_layer_tiles<2, 2, 2, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    case 3: seq_layer_tiles<2, 2, 1, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    case 4: seq_layer_tiles<1, 2, 8, 8, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    case 5: seq_layer_tiles<1, 2, 4, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
-    default: seq_layer_tiles<1, 2, 1, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate); break;
+    case 0: seq_layer_tiles<2, 2, 8, 8, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    case 1: seq_layer_tiles<2, 2, 4, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    case 2: seq_layer_tiles<2, 2, 2, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    case 3: seq_layer_tiles<2, 2, 1, 4, 2, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    case 4: seq_layer_tiles<1, 2, 8, 8, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    case 5: seq_layer_tiles<1, 2, 4, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
+    default: seq_layer_tiles<1, 2, 1, 4, 4, MODE>(xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr); break;
   }
 }
 
 __global__ void __launch_bounds__(512, 1)
-k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit) {
+k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit,
+           unsigned long long* __restrict__ stamps, int stamp_layers) {
   __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: one 8-wavefront tile set or two 4-wavefront ones
   __shared__ __attribute__((aligned(16))) int sBias[512];    // per half: one copy, or one per wavefront of an unsplit tile
   __shared__ int s_rank;
@@ -1469,10 +1495,19 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
     // layer l may read what layer l - 1 wrote once all 32 workgroups of the XCD have counted themselves out of it
     const LayerGate gate = {l > 0 ? my + SEQ_BAR : nullptr, (unsigned)l * SEQ_WG_PER_SHARE, error, spin_limit};
-    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
-    else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
-    else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate);
-    if (l + 1 == nlayers) break;
+    unsigned long long* tr = stamps && l < stamp_layers ? stamps + ((size_t)((int)xcc * SEQ_WG_PER_SHARE + rank) * stamp_layers + l) * 8 : nullptr;
+    if (tr && tid == 0) tr[7] = __builtin_amdgcn_s_memtime();
+    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
+    else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
+    else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
+    if (l + 1 == nlayers) {
+      if (tr) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
+      }
+      break;
+    }
     if (fetch_next) {
       sLayer[(l + 1) & 1][tid] = next0;
       if (tid + 64 < LWORDS) sLayer[(l + 1) & 1][tid + 64] = next1;
@@ -1480,6 +1515,7 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (tr && tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
     if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   // the last workgroup of a share to finish clears the share's counters for the next launch
@@ -1796,7 +1832,12 @@ k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const 
 
 // ---------------------------------------------------------------- host side
 // Kernel choice forced by the calling thread (tests and tuning runs); automatic unless set.
-static thread_local ConvTuning t_conv_tuning = {CONV_KERNEL_AUTO, -1, 0, 0};
+static ConvTuning default_tuning() {
+  ConvTuning t = {CONV_KERNEL_AUTO, -1, 0, 0, 2000000, nullptr, 0, {}};
+  memset(t.seq_layer_cfg, -1, sizeof(t.seq_layer_cfg));
+  return t;
+}
+static thread_local ConvTuning t_conv_tuning = default_tuning();
 void set_conv_tuning(const ConvTuning& t) { t_conv_tuning = t; }
 
 int pad_channels(int c) {
@@ -2453,9 +2494,10 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT || ep.pool ||
       !(nopad || (g.KH <= 32 && g.KW <= 32)))
     return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
+  const ConvTuning tune = t_conv_tuning;
   // a layer that fills the chip several times over is faster as a launch of the large-tile kernel than as a layer of a
   // sequence (whose tile is the wavefront kernel's); a run of layers ends there
-  if (t_conv_tuning.kernel == CONV_KERNEL_AUTO && t_conv_tuning.wave_cfg < 0 && choose_big_cfg(g) >= 0)
+  if (tune.kernel == CONV_KERNEL_AUTO && tune.wave_cfg < 0 && choose_big_cfg(g) >= 0)
     return arg_error("conv_seq_layer: not eligible (a layer for the large-tile kernel)");
   SeqLayer& L = reinterpret_cast<SeqLayer*>(table)[index];
   memset(&L, 0, sizeof(L));
@@ -2464,8 +2506,8 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   ConvGeom share = g;
   share.P = L.px_per_share;
   int cfg = choose_wave_cfg(share, SEQ_WG_PER_SHARE);
-  const ConvTuning tune = t_conv_tuning;
   if (tune.wave_cfg >= 0 && tune.wave_cfg <= 6) cfg = tune.wave_cfg;
+  if (index < 64 && tune.seq_layer_cfg[index] >= 0 && tune.seq_layer_cfg[index] <= 6) cfg = tune.seq_layer_cfg[index];
   if (cfg > 6) cfg = 3;
   const int mode = (g.KH == 1 && g.KW == 1 && g.SH == 1 && g.SW == 1 && nopad && g.OH == g.H && g.OW == g.W)
                        ? WAVE_IDENT : nopad ? WAVE_NOPAD : WAVE_PAD;
@@ -2491,13 +2533,19 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   return CVMHIP_OK;
 }
 
+int conv_seq_layer_config(const void* table, int index) {
+  return reinterpret_cast<const SeqLayer*>(table)[index].kernel / 3;
+}
+
 int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s) {
   if (!dev_table || nlayers < 1 || !sync || ((uintptr_t)dev_table & 15) || ((uintptr_t)sync & 255)) return arg_error("conv_seq_launch");
   char desc[64];
   snprintf(desc, sizeof(desc), "%d convolutions in one launch", nlayers);
   KernelTimer timer("k_conv_seq", ops, s, bytes, desc);
+  const ConvTuning tune = t_conv_tuning;
   k_conv_seq<<<SEQ_SHARES * SEQ_WG_PER_SHARE, 512, 0, s>>>(reinterpret_cast<const SeqLayer*>(dev_table), nlayers,
-                                                          reinterpret_cast<unsigned*>(sync), 2000000);
+                                                          reinterpret_cast<unsigned*>(sync), tune.seq_spin_limit, tune.seq_stamps,
+                                                          tune.seq_stamp_layers);
   return check_launch("conv_seq");
 }
 
@@ -2509,7 +2557,35 @@ extern "C" {
 
 int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn) {
   if (kernel < CONV_KERNEL_AUTO || kernel > CONV_KERNEL_BIG) return arg_error("set_conv_tuning kernel");
-  set_conv_tuning(ConvTuning{kernel, wave_cfg, tile_wm, tile_wn});
+  ConvTuning t = t_conv_tuning;
+  t.kernel = kernel; t.wave_cfg = wave_cfg; t.tile_wm = tile_wm; t.tile_wn = tile_wn;
+  set_conv_tuning(t);
+  return CVMHIP_OK;
+}
+
+int cvmhip_set_seq_layer_config(int index, int config) {
+  ConvTuning t = t_conv_tuning;
+  if (index < 0) memset(t.seq_layer_cfg, -1, sizeof(t.seq_layer_cfg));   // all automatic again
+  else if (index < 64 && config >= -1 && config < 127) t.seq_layer_cfg[index] = (signed char)config;
+  else return arg_error("set_seq_layer_config");
+  set_conv_tuning(t);
+  return CVMHIP_OK;
+}
+
+int cvmhip_set_seq_stamps(void* stamps, int layers) {
+  if (layers < 0 || (stamps && ((uintptr_t)stamps & 7))) return arg_error("set_seq_stamps");
+  ConvTuning t = t_conv_tuning;
+  t.seq_stamps = stamps && layers > 0 ? reinterpret_cast<unsigned long long*>(stamps) : nullptr;
+  t.seq_stamp_layers = t.seq_stamps ? layers : 0;
+  set_conv_tuning(t);
+  return CVMHIP_OK;
+}
+
+int cvmhip_set_seq_tuning(int spin_limit) {
+  if (spin_limit < 0) return arg_error("set_seq_tuning");
+  ConvTuning t = t_conv_tuning;
+  t.seq_spin_limit = spin_limit;
+  set_conv_tuning(t);
   return CVMHIP_OK;
 }
 

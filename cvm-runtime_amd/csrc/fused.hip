@@ -371,6 +371,11 @@ int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp
                        pad_h, pad_w, dil_h, dil_w, nullptr, nullptr, 0, nullptr, table, index);
 }
 
+int cvmhip_conv_seq_layer_config(const void* table, int index) {
+  if (!table || index < 0) return -1;
+  return conv_seq_layer_config(table, index);
+}
+
 int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream) {
   return conv_seq_launch(dev_table, nlayers, sync, ops, bytes, as_stream(stream));
 }

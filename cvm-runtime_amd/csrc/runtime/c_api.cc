@@ -150,6 +150,16 @@ int CVMHIPLaunchCounts(void* net, int* launches_per_run, int* sequence_launches,
   API_END();
 }
 
+int CVMHIPSequenceConfigs(void* net, int* configs, int capacity, int* count) {
+  API_BEGIN();
+  NOT_NULL(net);
+  NOT_NULL(count);
+  const std::vector<int> v = static_cast<HipModel*>(net)->runtime()->SequenceConfigs();
+  *count = static_cast<int>(v.size());
+  for (int i = 0; configs && i < capacity && i < *count; ++i) configs[i] = v[i];
+  API_END();
+}
+
 int CVMHIPProfileOps(void* net, char* json_out, int capacity) {
   API_BEGIN();
   NOT_NULL(net);

@@ -744,12 +744,16 @@ void HipGraphRuntime::BuildSequences() {
         r.bytes += static_cast<double>(st.n) * st.h * st.w * st.c + static_cast<double>(st.oc) * st.c * st.kh * st.kw +
                    px * st.oc * (st.src2 != kNone ? 2.0 : 1.0);
       }
+      for (size_t k = 0; k < count; ++k) r.cfgs.push_back(cvmhip_conv_seq_layer_config(table.data(), static_cast<int>(k)));
       seq_at_[i] = static_cast<int>(seqs_.size());
       seqs_.push_back(r);
     }
     i = j > i ? j : i + 1;
   }
   if (seqs_.empty()) return;
+  // a second model with sequence launches: what the first one has in flight is drained once
+  if (CountSequenceModel(+1) > 1) Check(cvmhip_device_sync(), "drain the device");
+  seq_counted_ = true;
   const size_t words = cvmhip_conv_seq_sync_bytes() / 4;
   Check(cvmhip_alloc(&seq_sync_, words * 4), "layer-sequence counters");
   Check(cvmhip_memset32(seq_sync_, 0, words, stream_), "layer-sequence counters");
@@ -757,7 +761,6 @@ void HipGraphRuntime::BuildSequences() {
   Check(cvmhip_host_alloc(&host, 64), "layer-sequence status");
   seq_error_host_ = static_cast<uint32_t*>(host);
   use_seq_ = true;
-  CountSequenceModel(+1);
 }
 
 // Consecutive detection-head steps read feature maps and write slices of concatenated tensors, never one another's

@@ -161,7 +161,7 @@ class HipGraphRuntime {
   bool fused() const { return fused_; }
   void LaunchCounts(int* launches, int* sequences, int* layers) const {
     int seq = 0, lay = 0;
-    if (use_seq_)
+    if (SeqNow())
       for (const SeqRun& r : seqs_) { ++seq; lay += r.nlayers; }
     int grouped = 0;
     for (const GroupRun& r : groups_) grouped += r.nlayers - 1;
@@ -223,7 +223,11 @@ class HipGraphRuntime {
   struct Hooks {
     bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true, conv_group = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
+    // layer-sequence launches: CVM_HIP_SEQ_SPIN=<polls> patience of a wait at a layer boundary (0: every wait gives up at once)
+    int seq_spin = 2000000;
+    std::vector<std::pair<int, int>> seq_layer_cfg;   // CVM_HIP_SEQCFG: (layer of a sequence, configuration)
   };
+  void ApplyTuning();   // hands the hooks to the kernels' per-thread tuning record
   Hooks hooks_;
   void ReadHooks();
 
@@ -245,8 +249,17 @@ class HipGraphRuntime {
     void* table = nullptr;
     int nlayers = 0;
     double ops = 0, bytes = 0;          // algorithmic operations and HBM bytes of its layers (for the measurement harness)
+    std::vector<int> cfgs;              // configuration of the tile kernel per layer
   };
   void BuildSequences();
+ public:
+  // configurations of the tile kernel chosen for the layers of all sequence launches, in order
+  std::vector<int> SequenceConfigs() const {
+    std::vector<int> v;
+    for (const SeqRun& r : seqs_) v.insert(v.end(), r.cfgs.begin(), r.cfgs.end());
+    return v;
+  }
+ private:
   // Runs of consecutive detection-head steps (int32 pixel-major output, independent of one another) that share one launch
   struct GroupRun {
     size_t first = 0, last = 0;         // plan_ indices, inclusive
@@ -260,13 +273,17 @@ class HipGraphRuntime {
   std::vector<GroupRun> groups_;
   std::vector<int> group_at_;           // per plan_ index: the group that starts there, or -1
   void CalibrateSequences();            // measures a run with and without sequence launches, keeps the faster
-  static void CountSequenceModel(int delta);   // models with sequence launches alive in this process
+  static int CountSequenceModel(int delta);    // models with sequence launches alive in this process, after the change
+  bool SeqNow() const;                  // does the next run use sequence launches?
+  bool seq_mode_ = false;               // what the launches being issued (and the captured graph) use
+  void DropSequences();                 // sequence launches are off for good for this model
   void CheckSequences();                // after a synchronisation: did a sequence launch give up?
   std::vector<SeqRun> seqs_;
   std::vector<int> seq_at_;             // per plan_ index: the run that starts there, or -1
   void* seq_sync_ = nullptr;            // counters and error word of the sequence launches (device)
   uint32_t* seq_error_host_ = nullptr;  // pinned copy of the error word
   bool use_seq_ = false;
+  bool seq_counted_ = false;            // this model is counted among the models with sequence launches
   bool seq_ran_ = false;                // a sequence launch was issued since the last check
 };
 

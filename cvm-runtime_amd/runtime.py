@@ -142,6 +142,14 @@ class HipModel:
         _ck(lib().CVMHIPLaunchCounts(self.net, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)), "CVMHIPLaunchCounts")
         return a.value, b.value, c.value
 
+    def sequence_configs(self):
+        """Tile-kernel configuration of every convolution inside the model's layer-sequence launches."""
+        n = ctypes.c_int()
+        _ck(lib().CVMHIPSequenceConfigs(self.net, None, ctypes.c_int(0), ctypes.byref(n)), "CVMHIPSequenceConfigs")
+        buf = (ctypes.c_int * max(n.value, 1))()
+        _ck(lib().CVMHIPSequenceConfigs(self.net, buf, ctypes.c_int(n.value), ctypes.byref(n)), "CVMHIPSequenceConfigs")
+        return list(buf[:n.value])
+
     def profile_ops(self):
         buf = ctypes.create_string_buffer(1 << 16)
         _ck(lib().CVMHIPProfileOps(self.net, buf, ctypes.c_int(len(buf))), "CVMHIPProfileOps")

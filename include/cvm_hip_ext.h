@@ -24,6 +24,9 @@ int CVMHIPTimeRun(void* net, int iterations, float* elapsed_ms);
 /* What a run of the model issues: kernel launches per run, how many of them are layer-sequence launches
  * (cvmhip_conv_seq_launch) and how many convolutions those contain.  Any pointer may be NULL. */
 int CVMHIPLaunchCounts(void* net, int* launches_per_run, int* sequence_launches, int* layers_in_sequences);
+/* The configuration of the tile kernel chosen for every convolution inside the model's layer-sequence launches, in
+ * order: *count receives how many there are, the first min(capacity, *count) are written to configs (may be NULL). */
+int CVMHIPSequenceConfigs(void* net, int* configs, int capacity, int* count);
 /* Per-operator device time of one run as a JSON object {"op": ms, ...}
  * (the table the reference prints under -DPROFILE, graph_runtime.cc:62-87). */
 int CVMHIPProfileOps(void* net, char* json_out, int capacity);

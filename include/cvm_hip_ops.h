@@ -258,6 +258,19 @@ int cvmhip_pad_channels(int channels);
  * wavefront kernel (-1 automatic) and a tile of the tiled kernel (wm, wn in 1..2; 0 automatic; with kernel 3, wm = 1..3
  * picks the 256x256, 128x256 or 64x512 tile).  The library never reads the environment on a launch. */
 int cvmhip_set_conv_tuning(int kernel, int wave_cfg, int tile_wm, int tile_wn);
+/* The same for layer-sequence launches (cvmhip_conv_seq_*) of the calling thread: `spin_limit` = polls after which a wait
+ * at a layer boundary gives up and raises the launch's error word (default 2 000 000; 0 makes every wait give up at
+ * once, which is how the fall-back of a caller is tested without hanging a kernel). */
+int cvmhip_set_seq_tuning(int spin_limit);
+/* Measurement hook: later layer-sequence launches of the calling thread write time stamps (shader clock) into `stamps`,
+ * device memory of 256 x layers x 8 64-bit words: per workgroup (XCD * 32 + rank among the XCD's workgroups)
+ * and layer, words 0..7 = tile entered, boundary passed, first operands multiplied, K loop done, K-split exchange
+ * done, epilogue issued, counted out, layer begun.  NULL switches them off (the default).  A launch captured into a
+ * graph keeps the pointer it was captured with. */
+int cvmhip_set_seq_stamps(void* stamps, int layers);
+/* Tuning hook: the configuration of the tile kernel for entry `index` (< 64) of the sequence tables that
+ * cvmhip_conv_seq_layer fills next on this thread; -1 = automatic; index < 0 resets every entry. */
+int cvmhip_set_seq_layer_config(int index, int config);
 /* int32 NCHW <-> int8 act layout (narrowing is static_cast<int8_t>) */
 int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream);
 int cvmhip_unpack_nhwc_i8(const void* xp, int32_t* x, int n, int c, int hw, void* stream);
@@ -312,6 +325,8 @@ int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp
                           const void* residual, const cvmhip_chain* chain2, void* out,
                           int n, int ic, int h, int wd, int oc, int kh, int kw,
                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
+/* configuration of the tile kernel that cvmhip_conv_seq_layer chose for entry `index` of a host table */
+int cvmhip_conv_seq_layer_config(const void* table, int index);
 /* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
 int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream);
 /* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values

@@ -87,16 +87,82 @@ def test_chain_of_convolutions_in_one_launch(name, dev):
     _check(g, heads, "seq-" + name)
 
 
+@pytest.mark.parametrize("batch", (8, 16))
 @pytest.mark.parametrize("cfg", range(7))
-def test_every_configuration_of_the_tile_kernel_inside_a_sequence(cfg, dev):
-    """CVM_HIP_WAVECFG forces one configuration for every layer of the sequence (all three addressing modes occur)."""
-    g, heads = _chain("seq-cfg%d" % cfg, 8, 3, 12, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (128, 3, 2, True, None),
-                                                     (128, 1, 2, True, None), (256, 3, 1, False, None), (256, 1, 1, True, None)])
+def test_every_configuration_of_the_tile_kernel_inside_a_sequence(cfg, batch, dev):
+    """CVM_HIP_WAVECFG forces one configuration for every layer of the sequence (all three addressing modes occur).
+    The model reports the configuration its table was built with: the forced one, for every layer."""
+    cid = "seq-cfg%d-b%d" % (cfg, batch)
+    g, heads = _chain(cid, batch, 3, 12, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (128, 3, 2, True, None),
+                                           (128, 1, 2, True, None), (256, 3, 1, False, 2), (256, 1, 1, True, None)])
     os.environ["CVM_HIP_WAVECFG"] = str(cfg)
     try:
-        _check(g, heads, "seq-cfg%d" % cfg)
+        _check(g, heads, cid)
+        js, pb = g.build(heads)
+        os.environ["CVM_HIP_SEQ"] = "1"
+        m = runtime.HipModel(js, pb)
+        try:
+            built = m.sequence_configs()
+        finally:
+            m.close()
+        assert built == [cfg] * 5, built
     finally:
         os.environ.pop("CVM_HIP_WAVECFG", None)
+        os.environ.pop("CVM_HIP_SEQ", None)
+
+
+def test_single_layers_of_a_sequence_take_the_configuration_named_for_them(dev):
+    """CVM_HIP_SEQCFG="index:config,...": the tuning hook for one layer at a time; the others keep the automatic choice."""
+    n, c, hw, layers = CHAINS["b16_ragged_shares_7x7"]
+    g, heads = _chain("seq-percfg", n, c, hw, layers)
+    js, pb = g.build(heads)
+    os.environ["CVM_HIP_SEQ"] = "1"
+    try:
+        m = runtime.HipModel(js, pb)
+        auto = m.sequence_configs()
+        m.close()
+        os.environ["CVM_HIP_SEQCFG"] = "1:6,3:5"
+        m = runtime.HipModel(js, pb)
+        forced = m.sequence_configs()
+        m.close()
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+        os.environ.pop("CVM_HIP_SEQCFG", None)
+    want = list(auto)
+    want[1], want[3] = 6, 5
+    assert forced == want, (auto, forced)
+    os.environ["CVM_HIP_SEQCFG"] = "1:6,3:5"
+    try:
+        _check(g, heads, "seq-percfg")
+    finally:
+        os.environ.pop("CVM_HIP_SEQCFG", None)
+
+
+def test_a_sequence_launch_that_gives_up_is_repeated_with_one_launch_per_layer(dev):
+    """CVM_HIP_SEQ_SPIN=0: every wait at a layer boundary gives up at once (all workgroups still run to the end and
+    exit normally), so the launch raises its error word; the runtime must notice after the run, switch sequence
+    launches off for the model and repeat the run with one launch per layer.  The bytes returned are the right ones
+    every time, and the model reports no sequence launches afterwards."""
+    g, heads = graphgen.resnet50(16, width=32, size=64, classes=100, config_id="seq-giveup")
+    js, pb = g.build(heads)
+    x = synth.tensor("seq-giveup", "data", g.shape((0, 0)), -127, 127).astype(np.int8)
+    want = _run(js, pb, x, "0")
+    os.environ["CVM_HIP_SEQ"] = "1"
+    os.environ["CVM_HIP_SEQ_SPIN"] = "0"
+    try:
+        m = runtime.HipModel(js, pb)
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+        os.environ.pop("CVM_HIP_SEQ_SPIN", None)
+    try:
+        assert m.launch_counts()[1] >= 1
+        outs = [np.frombuffer(m.inference(x.tobytes()), np.int32) for _ in range(4)]
+        after = m.launch_counts()
+    finally:
+        m.close()
+    for o in outs:
+        assert np.array_equal(o, want)
+    assert after[1] == 0 and after[2] == 0, after
 
 
 def test_resnet50_shrunk_batch16_and_resnet20_batch64(dev):
