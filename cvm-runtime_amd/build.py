@@ -18,6 +18,8 @@ LIB = os.path.join(HERE, "libcvm_runtime_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-fsigned-char", "-fvisibility=hidden", "-I" + os.path.join(HERE, "..", "include")]
+# extra preprocessor definitions for a measurement build, e.g. CVM_HIP_DEFINES="-DCVM_SEQ_STAMPS"
+COMMON += os.environ.get("CVM_HIP_DEFINES", "").split()
 # packed-fp32 code generation is switched off for all device code
 DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

@@ -69,9 +69,13 @@ __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
 #pragma unroll
         for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s1;
       }
-      if ((q.add | q.s2) != 0) {
+      if (q.add != 0) {
 #pragma unroll
-        for (int e = 0; e < N; ++e) v[e] = wadd(v[e], q.add) >> q.s2;
+        for (int e = 0; e < N; ++e) v[e] = wadd(v[e], q.add);
+      }
+      if (q.s2 != 0) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s2;
       }
     }
   }
@@ -126,6 +130,19 @@ template <bool COH>
 __device__ __forceinline__ int4 ld16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned uni = 0) {
   const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)uni, COH ? 16 : 0);
   return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
+}
+// Stores through a buffer descriptor: a 32-bit offset per lane instead of a 64-bit address, and the instruction is a
+// plain vector-memory store whatever the compiler knows about the pointer (a pointer read from a table in LDS is
+// "generic" to it and would be stored through with flat instructions, which also count as LDS traffic).
+__device__ __forceinline__ void st16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, const v4i v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v4u{(unsigned)v[0], (unsigned)v[1], (unsigned)v[2], (unsigned)v[3]}, rs, (int)off, 0, 0);
+}
+__device__ __forceinline__ void st8_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, uint32_t a, uint32_t b) {
+  typedef unsigned v2u_ __attribute__((ext_vector_type(2)));
+  __builtin_amdgcn_raw_buffer_store_b64(v2u_{a, b}, rs, (int)off, 0, 0);
+}
+__device__ __forceinline__ void st4_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, uint32_t a) {
+  __builtin_amdgcn_raw_buffer_store_b32(a, rs, (int)off, 0, 0);
 }
 __device__ __forceinline__ int4 ld16_l2(__amdgpu_buffer_rsrc_t rs, unsigned off) {
   const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 16 /* sc1: device scope */);
@@ -183,7 +200,8 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
 
 // RANGE: only the pixels [p_begin, p_end) are stored (one share of a layer inside the layer-sequence
 // kernel); the stores are then ordinary ones, because the next layer reads the tensor from this L2.
-template <int TN, int NG, int OUT, bool RANGE = false, bool POOLR = false>
+// BIASED: the accumulators already hold the bias (the wavefront kernel starts them from it), sBias is not read.
+template <int TN, int NG, int OUT, bool RANGE = false, bool POOLR = false, bool BIASED = false>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
                                               int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
                                               uint32_t (&rp)[NG], int p_begin = 0, int p_end = 0) {
@@ -200,9 +218,11 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     const int t = u >> 2;
     gj[m] = t % TN;
     ch[m] = ch_wave + (t / TN) * 32 + (u & 3) * 8 + lgrp * 4;
-    const int4 bv = *reinterpret_cast<const int4*>(sBias + ch[m]);
-    val[m * 4] = wadd(val[m * 4], bv.x); val[m * 4 + 1] = wadd(val[m * 4 + 1], bv.y);
-    val[m * 4 + 2] = wadd(val[m * 4 + 2], bv.z); val[m * 4 + 3] = wadd(val[m * 4 + 3], bv.w);
+    if constexpr (!BIASED) {
+      const int4 bv = *reinterpret_cast<const int4*>(sBias + ch[m]);
+      val[m * 4] = wadd(val[m * 4], bv.x); val[m * 4 + 1] = wadd(val[m * 4 + 1], bv.y);
+      val[m * 4 + 2] = wadd(val[m * 4 + 2], bv.z); val[m * 4 + 3] = wadd(val[m * 4 + 3], bv.w);
+    }
   }
   // byte offset of the KiB block (pixel block, 32 channels) that tile of group m belongs to
   auto block_off = [&](int m) {
@@ -326,7 +346,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       if (p < P && p >= Plo && first < ocp) {
         const v4i pk4 = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
         if constexpr (RANGE) {
-          *reinterpret_cast<v4i*>(y8 + block_off(t * 4) + lane * 16) = pk4;
+          st16_buf(act_rsrc(y8), (unsigned)block_off(t * 4) + (unsigned)lane * 16u, pk4);   // the tensor is smaller than 2^31 bytes (host)
         } else if (pool) {   // window p / 4 of the pooled tensor, the 16 channels this lane holds
           if ((lrow & 3) == 0) __builtin_nontemporal_store(pk4, reinterpret_cast<v4i*>(y8 + act_offset(p >> 2, first, ocp)));
         } else {
@@ -341,7 +361,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     const int first = oc0 + ch[0] - lgrp * 4 + lgrp * 8;
     mask_channels(w, first, g.OC);
     const int p = px_wave + gj[0] * 32 + lrow;
-    if (p < P && p >= Plo && first < ocp && store_lane) *reinterpret_cast<uint2*>(y8 + act_offset(p >> pshift, first, ocp)) = make_uint2(w[0], w[1]);
+    if (p < P && p >= Plo && first < ocp && store_lane) {
+      if constexpr (RANGE) st8_buf(act_rsrc(y8), (unsigned)act_offset(p >> pshift, first, ocp), w[0], w[1]);
+      else *reinterpret_cast<uint2*>(y8 + act_offset(p >> pshift, first, ocp)) = make_uint2(w[0], w[1]);
+    }
   } else {
 #pragma unroll
     for (int m = 0; m < NG; ++m) {
@@ -349,7 +372,10 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
       const int first = oc0 + ch[m];
       mask_channels(w, first, g.OC);
       const int p = px_wave + gj[m] * 32 + lrow;
-      if (p < P && p >= Plo && first < ocp && store_lane) *reinterpret_cast<uint32_t*>(y8 + act_offset(p >> pshift, first, ocp)) = w[0];
+      if (p < P && p >= Plo && first < ocp && store_lane) {
+        if constexpr (RANGE) st4_buf(act_rsrc(y8), (unsigned)act_offset(p >> pshift, first, ocp), w[0]);
+        else *reinterpret_cast<uint32_t*>(y8 + act_offset(p >> pshift, first, ocp)) = w[0];
+      }
     }
   }
 }
@@ -638,8 +664,9 @@ struct LayerGate {
   unsigned target;
   unsigned* error;
   int spin_limit;
+  unsigned* seen;      // LDS word of the workgroup (or of its half): the highest target its first wavefront has seen reached
 };
-__device__ __forceinline__ void gate_wait(const LayerGate& gate) {
+__device__ __forceinline__ void gate_poll(const LayerGate& gate) {
   if (!gate.counter) return;
   unsigned v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(gate.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
   int spins = 0;
@@ -659,11 +686,26 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate) {
     }
   }
 }
+// Only the first wavefront of a workgroup (of each half, when two tiles run side by side) polls the counter in the L2;
+// the others watch a word in LDS that it sets when it is through -- also when it gave up, so they never wait for longer
+// than it did.  Eight wavefronts of each of the XCD's 32 workgroups polling one address kept that L2 channel busy
+// with nothing but polls, in front of the very atomic adds they were waiting for.
+__device__ __forceinline__ void gate_wait(const LayerGate& gate, const int wave) {
+  if (!gate.counter) return;
+  if (wave != 0) {
+    while (__builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile unsigned*>(gate.seen)) < gate.target) __builtin_amdgcn_s_sleep(1);
+    return;
+  }
+  gate_poll(gate);
+  *reinterpret_cast<volatile unsigned*>(gate.seen) = gate.target;
+}
 
 // Optional time stamps of a layer inside a layer-sequence launch (cvmhip_set_seq_stamps): eight 64-bit words per
 // workgroup and layer -- 0 tile entered, 1 boundary passed, 2 first operand batch multiplied, 3 K loop done, 4 K-split
 // exchange done, 5 epilogue issued, 6 counted out, 7 layer begun -- written by the workgroup's first thread for the
-// first tile of the layer.  A null pointer (the normal case) costs a scalar branch per stamp.
+// first tile of the layer.  Only in a build with -DCVM_SEQ_STAMPS (cvm-runtime_amd/build.py: CVM_HIP_DEFINES): even
+// behind a null test the stamps cost the kernel a wait for all outstanding loads wherever two paths meet.
+#ifdef CVM_SEQ_STAMPS
 #define CVM_SEQ_STAMP(i, dep)                                              \
   do {                                                                     \
     if constexpr (COH) {                                                   \
@@ -673,11 +715,14 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate) {
       }                                                                    \
     }                                                                      \
   } while (0)
+#else
+#define CVM_SEQ_STAMP(i, dep) do { } while (0)
+#endif
 template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH, bool POOLR = false>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
-                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0},
+                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0, nullptr},
                                                unsigned long long* tr = nullptr) {
   CVM_SEQ_STAMP(0, tid);
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
@@ -791,7 +836,43 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
 #pragma unroll
   for (int j = 0; j < TN; ++j) tapoff[j] = kOutsideBuffer;
 
-  v16i acc[TM][TN];   // first written by the first MFMA of each tile, whose addend is the constant 0
+  // The accumulators start from the bias: the addend of a tile's first MFMA is the bias of its 32 output channels as the
+  // accumulator holds them (element e of a lane: channel (e / 4) * 8 + (lane / 32) * 4 + e % 4 of the tile), so the
+  // epilogue neither reads nor adds it.  After a K split one wavefront of each tile set brings it in (the one whose
+  // register groups are not permuted, kw_ == 0); the sums of the others start from zero.  The four 16-byte loads per
+  // 32 channels are the first requests of the tile and hit two addresses per wavefront each.
+  v16i binit[TM];
+  {
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < TM; ++i) binit[i] = zero16;
+    if (ep.bias && (KSPLIT == 1 || kw_ == 0)) {
+      const int OC = g.OC;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int first = oc0 + i * 32 + q * 8 + lgrp * 4;
+          int4 bv;
+          if (ep.bias_vec && (OC & 3) == 0) {   // whole groups of four channels, 16-byte aligned
+            const bool ok = first < OC;
+            bv = *reinterpret_cast<const int4*>(ep.bias + (ok ? first : 0));
+            bv = ok ? bv : zero4();
+          } else {
+            int b4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const bool ok = first + e < OC;
+              const int b = ep.bias[ok ? first + e : 0];
+              b4[e] = ok ? b : 0;
+            }
+            bv = make_int4(b4[0], b4[1], b4[2], b4[3]);
+          }
+          binit[i][q * 4] = bv.x; binit[i][q * 4 + 1] = bv.y; binit[i][q * 4 + 2] = bv.z; binit[i][q * 4 + 3] = bv.w;
+        }
+    }
+  }
+  v16i acc[TM][TN];   // first written by the first MFMA of each tile, whose addend is the bias
 
   // one batch = D chunks of both operands, one SSA value (see k_conv_igemm)
   typedef int regs_t __attribute__((ext_vector_type(4 * (TM + TN) * D)));
@@ -802,7 +883,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // COH: called once, between the filter requests and the activation requests of the first batch
   auto pass_gate = [&]() __attribute__((always_inline)) {
     if constexpr (COH) {
-      gate_wait(gate);
+      gate_wait(gate, wave);
       CVM_SEQ_STAMP(1, tid);
     }
   };
@@ -903,12 +984,11 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
         const int o = (d * (TM + TN) + TM + j) * 4;
         b[j] = v4i{R[o], R[o + 1], R[o + 2], R[o + 3]};
       }
-      const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], (first && d == 0) ? zero16 : acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], (first && d == 0) ? binit[i] : acc[i][j], 0, 0, 0);
     }
   };
 
@@ -919,14 +999,8 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // front of the first operand request).
   if (!COH && ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
   regs_t R0 = fetch(COH);
-  // Without a K split no wavefront needs anything from another one, so each stages its own copy of the bias in its
-  // own part of sBias and the tile needs no barrier at all: the wavefronts of a workgroup drift apart, and one's
-  // epilogue runs under another's operand requests (with a barrier per tile they all wait for memory together
-  // and then all do arithmetic together).
-  int bias_mine = 0;
-  const int bias_lane = KSPLIT == 1 ? lane : tid;
-  if (bias_lane < BM) bias_mine = (ep.bias && oc0 + bias_lane < g.OC) ? ep.bias[oc0 + bias_lane] : 0;
-  int* bias_lds = KSPLIT == 1 ? sBias + wave * BM : sBias;
+  // (Without a K split no wavefront needs anything from another one and the tile has no barrier at all: the
+  // wavefronts of a workgroup drift apart, and one's epilogue runs under another's operand requests.)
 
   // (COH) the residual is not needed before the epilogue: requested behind the operand batches that are in flight
   // at the start, it does not stand between the layer boundary and the first MFMA
@@ -956,7 +1030,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     }
   }
   CVM_SEQ_STAMP(3, acc[0][0][0]);
-  if (bias_lane < BM) bias_lds[bias_lane] = bias_mine;
 
   // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
   // wavefront kw_ then finalises the groups kw_*NU .. kw_*NU + NU-1 of the tile set
@@ -985,7 +1058,6 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
     }
   } else {
-    __builtin_amdgcn_wave_barrier();   // bias staged: written and read by this wavefront only, and LDS serves a wavefront in order
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -996,7 +1068,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   CVM_SEQ_STAMP(4, val[0]);
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT, COH, POOLR>(val, kw_ * NU, bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
+  finish_groups<TN, NU, OUT, COH, POOLR, true>(val, kw_ * NU, nullptr, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
   CVM_SEQ_STAMP(5, tid);
 }
 
@@ -1422,7 +1494,8 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
     conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
                                                                          sPart + half * 16384, sBias + half * 256, p_begin, p_end,
-                                                                         base == 0 ? gate : LayerGate{nullptr, 0, nullptr, 0}, base == 0 ? tr : nullptr);
+                                                                         base == 0 ? LayerGate{gate.counter, gate.target, gate.error, gate.spin_limit, gate.seen + half} : LayerGate{nullptr, 0, nullptr, 0, nullptr},
+                                                                         base == 0 ? tr : nullptr);
     if (KSPLIT > 1) __syncthreads();   // the next tile reuses the LDS of the partial sums
   }
 }
@@ -1448,6 +1521,7 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   __shared__ __attribute__((aligned(16))) int sPart[32768];   // 128 KiB: one 8-wavefront tile set or two 4-wavefront ones
   __shared__ __attribute__((aligned(16))) int sBias[512];    // per half: one copy, or one per wavefront of an unsplit tile
   __shared__ int s_rank;
+  __shared__ unsigned s_seen[2];   // per half of the workgroup: the highest layer boundary its first wavefront has seen reached
   // The current layer's table entry lives in LDS, where any field is a short read away wherever the code needs
   // it (a copy in registers would hold ~100 scalar registers for the whole layer, and reading it from memory
   // would begin every layer with a trip there).  The first wavefront requests the next entry when a layer
@@ -1467,8 +1541,11 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   unsigned* error = sync + SEQ_SHARES * SEQ_SYNC_WORDS;
   if (tid == 0) {
     const unsigned r = __hip_atomic_fetch_add(my + SEQ_ARRIVE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (xcc >= SEQ_SHARES || r >= SEQ_WG_PER_SHARE) __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // not the chip this kernel is laid out for
+    // not the chip this kernel is laid out for; or no patience at all, which is how a host tests its fall-back: the launch
+    // then reports failure whatever happens, and no wait inside it ever sleeps
+    if (xcc >= SEQ_SHARES || r >= SEQ_WG_PER_SHARE || spin_limit <= 0) __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_rank = (int)r;
+    s_seen[0] = s_seen[1] = 0u;
   }
   __syncthreads();
   const int rank = s_rank;
@@ -1494,18 +1571,24 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
     // layer l may read what layer l - 1 wrote once all 32 workgroups of the XCD have counted themselves out of it
-    const LayerGate gate = {l > 0 ? my + SEQ_BAR : nullptr, (unsigned)l * SEQ_WG_PER_SHARE, error, spin_limit};
+    const LayerGate gate = {l > 0 ? my + SEQ_BAR : nullptr, (unsigned)l * SEQ_WG_PER_SHARE, error, spin_limit, s_seen};
+#ifdef CVM_SEQ_STAMPS
     unsigned long long* tr = stamps && l < stamp_layers ? stamps + ((size_t)((int)xcc * SEQ_WG_PER_SHARE + rank) * stamp_layers + l) * 8 : nullptr;
     if (tr && tid == 0) tr[7] = __builtin_amdgcn_s_memtime();
+#else
+    unsigned long long* tr = nullptr;
+#endif
     if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
     else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
     else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
     if (l + 1 == nlayers) {
+#ifdef CVM_SEQ_STAMPS
       if (tr) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
       }
+#endif
       break;
     }
     if (fetch_next) {
@@ -1515,7 +1598,9 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+#ifdef CVM_SEQ_STAMPS
     if (tr && tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
+#endif
     if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   // the last workgroup of a share to finish clears the share's counters for the next launch
@@ -2494,6 +2579,8 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT || ep.pool ||
       !(nopad || (g.KH <= 32 && g.KW <= 32)))
     return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
+  // results are stored through a buffer descriptor with 32-bit offsets
+  if (act_bytes(g.P, ep.out_cp) > INT32_MAX) return arg_error("conv_seq_layer: not eligible (output tensor of 2 GiB or more)");
   const ConvTuning tune = t_conv_tuning;
   // a layer that fills the chip several times over is faster as a launch of the large-tile kernel than as a layer of a
   // sequence (whose tile is the wavefront kernel's); a run of layers ends there
@@ -2574,6 +2661,9 @@ int cvmhip_set_seq_layer_config(int index, int config) {
 
 int cvmhip_set_seq_stamps(void* stamps, int layers) {
   if (layers < 0 || (stamps && ((uintptr_t)stamps & 7))) return arg_error("set_seq_stamps");
+#ifndef CVM_SEQ_STAMPS
+  if (stamps) return arg_error("set_seq_stamps: this build has no time stamps (build with -DCVM_SEQ_STAMPS)");
+#endif
   ConvTuning t = t_conv_tuning;
   t.seq_stamps = stamps && layers > 0 ? reinterpret_cast<unsigned long long*>(stamps) : nullptr;
   t.seq_stamp_layers = t.seq_stamps ? layers : 0;

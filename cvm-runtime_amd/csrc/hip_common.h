@@ -151,6 +151,44 @@ __device__ __forceinline__ int32_t apply_chain(const DevChain& c, int32_t v) {
 
 inline bool stage_is_clamp(const DevStage& s) { return s.s1 == 0 && s.add == 0 && s.s2 == 0 && s.mul == 1; }
 
+// host: what a stage without a multiplication does to a value that already lies inside its clamp
+inline int64_t stage_shift_part(const DevStage& s, int64_t v) { return ((v >> s.s1) + s.add) >> s.s2; }
+
+// host: folds a pure clamp [clo, chi] that FOLLOWS stage p into p's own clamp, when that is exact for every input.
+// On p's clamped domain [lo, hi] the shift part f(v) = ((v >> s1) + add) >> s2 never wraps (checked) and is monotonic
+// with steps of at most one, so it takes every value between f(lo) and f(hi): clamping f's result to [clo, chi] then
+// equals clamping the input to [lo', hi'], lo' the smallest v with f(v) >= clo and hi' the largest with f(v) <= chi.
+inline bool merge_clamp_behind(DevStage* p, int32_t clo, int32_t chi) {
+  if (p->mul != 1 || clo > chi || p->lo > p->hi) return false;
+  if (p->s1 == 0 && p->s2 == 0) return false;   // not a shift: nothing says its steps are at most one
+  const int64_t lo = p->lo, hi = p->hi;
+  const int64_t a = (lo >> p->s1) + p->add, b = (hi >> p->s1) + p->add;
+  if (a < INT32_MIN || a > INT32_MAX || b < INT32_MIN || b > INT32_MAX) return false;   // the add could wrap
+  const int64_t flo = stage_shift_part(*p, lo), fhi = stage_shift_part(*p, hi);
+  if (fhi < clo || flo > chi) return false;     // the result would be a constant: leave the two stages as they are
+  int64_t nlo = lo, nhi = hi;
+  if (flo < clo) {   // smallest v in (lo, hi] with f(v) >= clo
+    int64_t l = lo, h = hi;   // f(l) < clo <= f(h)
+    while (h - l > 1) {
+      const int64_t m = l + (h - l) / 2;
+      if (stage_shift_part(*p, m) >= clo) h = m; else l = m;
+    }
+    nlo = h;
+  }
+  if (fhi > chi) {   // largest v in [lo, hi) with f(v) <= chi
+    int64_t l = lo, h = hi;   // f(l) <= chi < f(h)
+    while (h - l > 1) {
+      const int64_t m = l + (h - l) / 2;
+      if (stage_shift_part(*p, m) <= chi) l = m; else h = m;
+    }
+    nhi = l;
+  }
+  if (nlo > nhi) return false;
+  p->lo = (int32_t)nlo;
+  p->hi = (int32_t)nhi;
+  return true;
+}
+
 // host: validates and converts the C-ABI chain; returns false on a bad stage
 inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
   out->count = 0;
@@ -180,9 +218,16 @@ inline bool make_chain(const cvmhip_chain* in, DevChain* out) {
       }
     } else if (s.kind == CVMHIP_STAGE_MUL) {
       d.mul = s.lo;   // wrapping int32 product, as broadcast_mul computes it (broadcast.cc:75-86)
+    } else if (s.kind == CVMHIP_STAGE_CLAMP_SHIFT) {
+      if (s.shift_bit < 0 || s.shift_bit > 31 || s.lo > s.hi) return false;
+      d.lo = s.lo; d.hi = s.hi; d.s2 = s.shift_bit;
     } else {
       return false;
     }
+    // a pure clamp behind a shift stage becomes part of that stage's own clamp where that is exact
+    if (out->count > 0 && stage_is_clamp(d) && !stage_is_clamp(out->st[out->count - 1]) &&
+        merge_clamp_behind(&out->st[out->count - 1], d.lo, d.hi))
+      continue;
     // merge a pure clamp into a preceding pure clamp, or into the clamp of the stage that follows it
     if (out->count > 0 && stage_is_clamp(out->st[out->count - 1])) {
       DevStage& p = out->st[out->count - 1];

@@ -698,8 +698,38 @@ void HipGraphRuntime::BuildPlan() {
   }
   plan_ = std::move(plan);
   fused_ = true;
+  if (hooks_.fold_bias) FoldRequant();
   if (hooks_.seq) BuildSequences();
   BuildGroups();
+}
+
+// The rounding terms of a convolution's requantisation chains move into its bias (one add per channel at load instead
+// of one per value in every run), where the bias values and the number of int8 x int8 products prove that nothing
+// wraps; CVM_HIP_FOLDBIAS=0 keeps the chains as the graph gives them.
+void HipGraphRuntime::FoldRequant() {
+  for (PlanStep& st : plan_) {
+    const bool conv = st.kind == PlanStep::CONV && !st.pair, dw = st.kind == PlanStep::DWCONV;
+    if (!conv && !dw) continue;
+    std::vector<int32_t> bias(static_cast<size_t>(st.oc), 0), folded(static_cast<size_t>(st.oc));
+    if (st.bias) {
+      Check(cvmhip_copy_d2h(bias.data(), st.bias, bias.size() * 4, stream_), "read bias");
+      Check(cvmhip_stream_sync(stream_), "read bias");
+    }
+    const int64_t terms = dw ? static_cast<int64_t>(st.kh) * st.kw : static_cast<int64_t>(st.c) * st.kh * st.kw;
+    cvmhip_chain c1{}, c2{};
+    const bool residual = conv && st.src2 != kNone;
+    if (!cvmhip_fold_requant(st.bias ? bias.data() : nullptr, st.oc, terms * 128 * 128, &st.chain, &st.chain2, residual ? 1 : 0,
+                             folded.data(), &c1, &c2))
+      continue;
+    auto buf = std::make_shared<DeviceBuffer>();
+    Check(cvmhip_alloc(&buf->ptr, folded.size() * 4), "folded bias");
+    Check(cvmhip_copy_h2d(buf->ptr, folded.data(), folded.size() * 4, stream_), "folded bias");
+    Check(cvmhip_stream_sync(stream_), "folded bias");   // the host copy goes away
+    st.folded_bias = buf;
+    st.bias = static_cast<const int32_t*>(buf->ptr);
+    st.chain = c1;
+    if (residual) st.chain2 = c2;
+  }
 }
 
 // Runs of at least three consecutive convolution steps that a layer-sequence launch can take (batch a multiple

@@ -446,6 +446,7 @@ HipGraphRuntime::HipGraphRuntime(const std::string& graph_json, int device_id, b
 void HipGraphRuntime::ReadHooks() {
   auto env = [](const char* name) { const char* v = std::getenv(name); return std::string(v ? v : ""); };
   hooks_.fuse = env("CVM_HIP_FUSE") != "0";
+  hooks_.fold_bias = env("CVM_HIP_FOLDBIAS") != "0";
   hooks_.graph = env("CVM_HIP_GRAPH") != "0";
   hooks_.seq = env("CVM_HIP_SEQ") != "0";
   hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";

@@ -115,6 +115,7 @@ struct PlanStep {
   int64_t dst_off2 = 0, img_stride2 = 0;
   int oc2 = 0;
   std::shared_ptr<void> pair_bias;
+  std::shared_ptr<void> folded_bias;   // CONV, DWCONV: the bias with the chains' rounding terms added (device); `bias` then points here
   uint32_t wsrc = UINT32_MAX, bsrc = UINT32_MAX;   // CONV: entries of the filter and the bias (UINT32_MAX: none)
   int n = 0, c = 0, h = 0, w = 0, oc = 0, kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1, oh = 0, ow = 0;
 };
@@ -221,7 +222,7 @@ class HipGraphRuntime {
   // depthwise layers on the vector kernel, CVM_HIP_CONV=lds|wave, CVM_HIP_WAVECFG=<i> and
   // CVM_HIP_TILE="wm,wn" force an implicit-GEMM kernel, a configuration or a tile.
   struct Hooks {
-    bool fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true, conv_group = true;
+    bool fold_bias = true, fuse = true, graph = true, dw_on_mfma = true, seq = true, seq_forced = false, pool_fuse = true, head_pair = true, head_group = true, conv_group = true;
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
     // layer-sequence launches: CVM_HIP_SEQ_SPIN=<polls> patience of a wait at a layer boundary (0: every wait gives up at once)
     int seq_spin = 2000000;
@@ -251,6 +252,7 @@ class HipGraphRuntime {
     double ops = 0, bytes = 0;          // algorithmic operations and HBM bytes of its layers (for the measurement harness)
     std::vector<int> cfgs;              // configuration of the tile kernel per layer
   };
+  void FoldRequant();   // rounding terms of the convolutions' requantisation into their biases (cvmhip_fold_requant)
   void BuildSequences();
  public:
   // configurations of the tile kernel chosen for the layers of all sequence launches, in order

@@ -239,19 +239,34 @@ int cvmhip_conv2d_packed(const int32_t* x, const void* wp, const int32_t* bias, 
  * channels, each stored as the 1 KiB operand fragment of v_mfma_i32_32x32x32_i8:
  *   offset(p, c) = ((p/32)*(cp/32) + c/32)*1024 + ((c/16)%2)*512 + (p%32)*16 + c%16
  * A buffer for npix pixels has cvmhip_packed_act_bytes(npix, c) bytes, 16-byte aligned. */
-enum { CVMHIP_STAGE_RELU = 1, CVMHIP_STAGE_RSHIFT = 2, CVMHIP_STAGE_CLIP = 3, CVMHIP_STAGE_MUL = 4 };
+enum { CVMHIP_STAGE_RELU = 1, CVMHIP_STAGE_RSHIFT = 2, CVMHIP_STAGE_CLIP = 3, CVMHIP_STAGE_MUL = 4, CVMHIP_STAGE_CLAMP_SHIFT = 5 };
 typedef struct {
   int32_t kind;        /* CVMHIP_STAGE_* */
   int32_t precision;   /* RSHIFT */
   int32_t shift_bit;   /* RSHIFT */
   int32_t lo, hi;      /* CLIP: max(min(v, hi), lo).  MUL: v * lo, wrapping (broadcast_mul by a constant scalar,
-                          the requantisation scale in front of a cvm_right_shift; broadcast.cc:75-86) */
+                          the requantisation scale in front of a cvm_right_shift; broadcast.cc:75-86).
+                          CLAMP_SHIFT: min(max(v, lo), hi) >> shift_bit (arithmetic, 0..31, no rounding term): what is
+                          left of a cvm_right_shift whose rounding term the caller has added to the value beforehand,
+                          see cvmhip_fold_requant */
 } cvmhip_stage;
 typedef struct {
   int32_t count;       /* 0..4 stages, applied in order to the int32 value */
   cvmhip_stage stage[4];
 } cvmhip_chain;
 
+/* Host-side, no device needed.  cvmhip_chain_apply_host evaluates a chain on n int32 values exactly as the kernels do
+ * (the form the library prepares from the stages, with adjacent clamps merged).
+ * cvmhip_fold_requant rewrites the epilogue of a convolution  v = chain(acc + bias[oc]); if (residual) v = chain2(v + r)
+ * into an equivalent one with fewer instructions per value: the rounding terms of the cvm_right_shift stages are
+ * added to the bias (oc values, host memory; NULL = zeros) once per channel, and what remains of the stages are
+ * CVMHIP_STAGE_CLAMP_SHIFT stages.  max_abs_acc bounds |acc| (e.g. taps * channels * 128 * 128 for int8 operands);
+ * the rewrite is only made when acc + bias + rounding terms provably never wraps.  Returns 1 and fills bias_out
+ * (oc values), chain_out, chain2_out, or returns 0 and leaves them alone (chain shapes it does not handle, or no proof). */
+int cvmhip_chain_apply_host(const cvmhip_chain* chain, const int32_t* in, int64_t n, int32_t* out);
+int cvmhip_fold_requant(const int32_t* bias, int oc, int64_t max_abs_acc, const cvmhip_chain* chain,
+                        const cvmhip_chain* chain2, int has_residual, int32_t* bias_out, cvmhip_chain* chain_out,
+                        cvmhip_chain* chain2_out);
 int cvmhip_pad_channels(int channels);
 /* Test and tuning hook: forces, for the calling thread's later convolution launches, the implicit-GEMM kernel
  * (0 automatic, 1 LDS-tiled, 2 wavefront-private, 3 large-tile wherever the layout allows it), a configuration of the
@@ -266,7 +281,8 @@ int cvmhip_set_seq_tuning(int spin_limit);
  * device memory of 256 x layers x 8 64-bit words: per workgroup (XCD * 32 + rank among the XCD's workgroups)
  * and layer, words 0..7 = tile entered, boundary passed, first operands multiplied, K loop done, K-split exchange
  * done, epilogue issued, counted out, layer begun.  NULL switches them off (the default).  A launch captured into a
- * graph keeps the pointer it was captured with. */
+ * graph keeps the pointer it was captured with.  Only a library built with -DCVM_SEQ_STAMPS has them (the stamps cost
+ * the kernel waits even when unused); otherwise a non-NULL pointer is refused with CVMHIP_ERR_ARG. */
 int cvmhip_set_seq_stamps(void* stamps, int layers);
 /* Tuning hook: the configuration of the tile kernel for entry `index` (< 64) of the sequence tables that
  * cvmhip_conv_seq_layer fills next on this thread; -1 = automatic; index < 0 resets every entry. */
