@@ -23,10 +23,83 @@ PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 # HBM bytes per launch of the dominant kernel of a batch-16 workload, from the FETCH_SIZE and WRITE_SIZE counter
 # passes summarised in the named file under profiles/ (a counter pass cannot run inside this program, so the
 # figures are carried here; each is reported only for the workload and kernel it was measured on)
+# The third field is the first 16 hex digits of the SHA-256 of the kernels' source file as it was when the counters were
+# read: a figure is only reported while that file is unchanged, otherwise `traffic` is null (measured figures go stale).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("resnet50", "k_conv_seq", 16): (548.6e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt"),
-    ("vgg16", "k_conv_big", 16): (33.8e6, "profiles/k_conv_big_vgg16_b16_traffic.txt"),
+    ("resnet50", "k_conv_seq", 16): (548.6e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt", "unrecorded"),
+    ("vgg16", "k_conv_big", 16): (33.8e6, "profiles/k_conv_big_vgg16_b16_traffic.txt", "unrecorded"),
 }
+KERNEL_SOURCE = os.path.join(ROOT, "cvm-runtime_amd", "csrc", "conv_mfma.hip")
+
+
+def kernel_source_hash():
+    import hashlib
+    try:
+        return hashlib.sha256(open(KERNEL_SOURCE, "rb").read()).hexdigest()[:16]
+    except OSError:
+        return None
+
+
+def dominant_conv(kt, wall_s, steps):
+    """From the per-kernel event-pair totals of `steps` steps: the implicit-GEMM kernel that takes most of the step, its
+    average launch duration with the cost of an event pair taken off, and the figures derived from it."""
+    n_timed = sum(v["launches"] for v in kt.values())
+    pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall_s * 1e6) / max(n_timed, 1))
+    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big", "k_conv_group", "k_stem_pool")}
+    dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
+    conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
+    launches = max(conv["launches"], 1)
+    raw_avg_s = conv["ms"] / 1e3 / launches
+    avg_s = max(raw_avg_s - pair_cost_us * 1e-6, 1e-9)
+    return {"kernel": dom, "convs": convs, "conv": conv, "pair_cost_us": pair_cost_us, "raw_avg_s": raw_avg_s, "avg_s": avg_s,
+            "ops_per_launch": conv["work"] / launches}
+
+
+def side_workload(pkg, L, name, batch, steps, warmup, check):
+    """A second benchmark configuration measured in the same process, the same way as the headline one (input resident in
+    HBM, `steps` timed runs, then the same steps with an event pair around every launch): VGG-16 at batch 16 is where the
+    large-tile kernel runs, so its fraction of the matrix-core peak is in the driver's line too.  With `check` the first
+    image of the timed batch is compared with the CPU runtime's result for it."""
+    import numpy as np
+    import torch
+    from cvm_runtime_amd import graphgen, runtime, synth
+    g, heads = {"vgg16": graphgen.vgg16}[name](batch)
+    js, pb = g.build(heads)
+    x = synth.tensor("bench", "data", g.shape((0, 0)), -127, 127).astype(np.int8)
+    model = runtime.HipModel(js, pb)
+    counts = model.launch_counts()
+    model.set_input(x.tobytes())
+    model.time_run(max(warmup, 1))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.time_run(steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    L.cvmhip_kernel_timing_begin()
+    model.time_run(steps)
+    torch.cuda.synchronize()
+    buf = ctypes.create_string_buffer(1 << 16)
+    pkg.check(L.cvmhip_kernel_timing_end(buf, len(buf)))
+    kt = json.loads(buf.value.decode())
+    raw = model.get_output()
+    tsize = runtime.CVMAPIGetOutputTypeSize(model.net)
+    model.close()
+    d = dominant_conv(kt, wall, steps)
+    achieved = d["ops_per_launch"] / d["avg_s"] / 1e12
+    out = {"workload": "cfg4 VGG-16 quantised graph, batch %d, 3x224x224 int8, random int8 weights" % batch,
+           "ms_per_step": wall / steps * 1e3, "images_per_s": batch * steps / wall, "kernel_launches_per_step": counts[0],
+           "kernel": d["kernel"], "launches_per_step": d["conv"]["launches"] / steps, "avg_launch_us": d["avg_s"] * 1e6,
+           "algorithmic_gop_per_launch": d["ops_per_launch"] / 1e9, "achieved_tops": achieved, "frac": achieved / PEAK_I8_TOPS,
+           "all_conv_dense_tops": sum(v["work"] for v in d["convs"].values()) /
+                                  max(sum(v["ms"] / 1e3 - v["launches"] * d["pair_cost_us"] * 1e-6 for v in d["convs"].values()), 1e-9) / 1e12}
+    if check:
+        g1, h1 = {"vgg16": graphgen.vgg16}[name](1)
+        js1, pb1 = g1.build(h1)
+        _, want = cpu_baseline(js1, pb1, x[:1].astype(np.int32), 0.0)
+        per_image = len(raw) // batch
+        got = np.frombuffer(raw[:per_image], np.int32 if tsize == 4 else np.int8).astype(np.int32)
+        out["parity_checked"] = bool(got.shape == want.shape and np.array_equal(got, want))
+    return out
 
 
 def cpu_baseline(js1, pb1, x1, budget_s=20.0):
@@ -176,6 +249,8 @@ def main():
                     help="resnet50 (default) is the headline configuration; the others are the remaining benchmark "
                          "configurations, measured the same way (ssd512 always runs at batch 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vgg", action="store_true",
+                    help="skip the VGG-16 batch-16 figures that the headline configuration reports beside its own")
     ap.add_argument("--no-two-models", action="store_true",
                     help="skip the side measurement with two models in flight (keeps a profiler's kernel statistics to one model)")
     ap.add_argument("--suite", choices=("model", "ops"), default="model",
@@ -301,21 +376,25 @@ def main():
     # of a step is timed and the un-instrumented step is GPU-bound with its kernels back to back, so the
     # cost of one pair is (sum of all pair times - un-instrumented step time) / launches; it is taken off
     # every launch.  The rocprofv3 kernel trace under profiles/ measures the same durations directly.
-    n_timed = sum(v["launches"] for v in kt.values())
-    pair_cost_us = max(0.0, (sum(v["ms"] for v in kt.values()) * 1e3 - wall * 1e6) / max(n_timed, 1))
+    d = dominant_conv(kt, wall, args.steps)
+    pair_cost_us, convs, dom, conv = d["pair_cost_us"], d["convs"], d["kernel"], d["conv"]
     pair_us = {"empty_us": pair_cost_us}
-    convs = {k: v for k, v in kt.items() if k in ("k_conv_wave", "k_conv_igemm", "k_conv_seq", "k_conv_big", "k_conv_group", "k_stem_pool")}
-    dom = max(convs, key=lambda k: convs[k]["ms"]) if convs else "k_conv_wave"
-    conv = convs.get(dom, {"launches": 0, "ms": 0.0, "work": 0.0})
-    launches = max(conv["launches"], 1)
-    ops_per_launch = conv["work"] / launches
-    raw_avg_s = conv["ms"] / 1e3 / launches
-    avg_s = max(raw_avg_s - pair_us["empty_us"] * 1e-6, 1e-9)
+    ops_per_launch, raw_avg_s, avg_s = d["ops_per_launch"], d["raw_avg_s"], d["avg_s"]
     achieved = ops_per_launch / avg_s / 1e12
     all_ops = sum(v["work"] for v in convs.values())
     all_s = sum(v["ms"] / 1e3 - v["launches"] * pair_us["empty_us"] * 1e-6 for v in convs.values())
     step_s = wall / args.steps
-    traffic = TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dom, args.batch), (None, None))
+    traffic = TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dom, args.batch), (None, None, None))
+    source_hash = kernel_source_hash()
+    traffic_note = None
+    if traffic[0] is not None:
+        if traffic[2] == source_hash:
+            traffic_note = ("recorded from the FETCH_SIZE / WRITE_SIZE counter passes summarised in " + traffic[1] +
+                            " (kernel source " + str(source_hash) + "), not measured by this run")
+        else:
+            traffic_note = ("none reported: the kernels' source (" + str(source_hash) + ") has changed since the counter passes of " +
+                            traffic[1] + " (" + str(traffic[2]) + ")")
+            traffic = (None, traffic[1], traffic[2])
     line = {
         "metric": "images/sec int8 %s, one MI355X, input resident in HBM" % names[args.workload],
         "value": args.batch / step_s,
@@ -340,9 +419,8 @@ def main():
                    "output_checksum": int(np.bitwise_xor.reduce(out.view(np.uint32)))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_I8_TOPS, "unit": "TOP/s",
                      "frac": achieved / PEAK_I8_TOPS,
-                     "traffic": traffic[0], "traffic_unit": "bytes per launch",
-                     "traffic_source": ("recorded from the FETCH_SIZE / WRITE_SIZE counter passes summarised in "
-                                        + traffic[1] + ", not measured by this run") if traffic[0] else None,
+                     "traffic": traffic[0], "traffic_unit": "bytes per launch", "traffic_source": traffic_note,
+                     "kernel_source_sha256_16": source_hash,
                      "kernel": dom, "launches_per_step": conv["launches"] / args.steps,
                      "avg_launch_us": avg_s * 1e6, "avg_launch_us_with_event_pair": raw_avg_s * 1e6,
                      "event_pair_cost_us": pair_cost_us, "algorithmic_gop_per_launch": ops_per_launch / 1e9,
@@ -369,6 +447,11 @@ def main():
         m1.close()
         line["config"]["images_per_s_batch1"] = 1.0 / b1_s
         line["config"]["ms_per_step_batch1"] = b1_s * 1e3
+    if args.workload == "resnet50" and args.batch == 16 and not args.no_vgg:
+        line["config"]["vgg16_b16"] = side_workload(pkg, L, "vgg16", 16, max(args.steps // 2, 5), args.warmup, not args.no_cpu_baseline)
+        if line["config"]["vgg16_b16"].get("parity_checked") is False:
+            print(json.dumps(line))
+            sys.exit("bench.py: VGG-16 batch 16: the first image differs from the CPU runtime's result")
     # The CPU baseline leg runs the reference CPU runtime on the first image of the timed batch; its values also
     # check the timed configuration: the GPU's output for that image must equal them bit for bit.
     if not args.no_cpu_baseline:
