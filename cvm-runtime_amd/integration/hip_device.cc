@@ -287,6 +287,32 @@ CVM_REGISTER_GLOBAL("cvm.runtime.hip.non_max_suppression").set_body([](CVMArgs a
                                      p.force_suppress ? 1 : 0, Scratch(args), ScratchBytes(args), nullptr));
 });
 
+// ---- scratch memory.  The reference sizes an operator's ext_space with the operator's FOpExtraSpace attribute
+// (include/cvm/op_attr_types.h; called with the node's attributes, input shapes, precisions and the context in
+// src/runtime/graph_runtime.cc), in int32 elements.  For this device the sizes are this library's: the bodies of
+// FOpExtraSpace for conv2d, dense, get_valid_counts and non_max_suppression (src/top/nn/*.cc) return
+// HIPOpExtraSpace(attrs, shapes) when ctx.device_type is the HIP device.  Operators it does not name need none.
+int64_t HIPOpExtraSpace(const cvm::NodeAttrs& attrs, const std::vector<TShape>& in_shapes) {
+  const std::string& op = attrs.op->name;
+  size_t bytes = 0;
+  if (op == "conv2d" && in_shapes.size() >= 2 && in_shapes[0].ndim() == 4 && in_shapes[1].ndim() == 4) {
+    const auto& p = cvm::get<cvm::top::Conv2DParam>(attrs.parsed);
+    const TShape &x = in_shapes[0], &w = in_shapes[1];
+    bytes = cvmhip_conv2d_workspace_bytes(static_cast<int>(x[0]), static_cast<int>(x[1]), static_cast<int>(x[2]),
+                                          static_cast<int>(x[3]), static_cast<int>(w[0]), static_cast<int>(w[2]),
+                                          static_cast<int>(w[3]), p.groups);
+  } else if (op == "dense" && in_shapes.size() >= 2 && in_shapes[0].ndim() == 2 && in_shapes[1].ndim() == 2) {
+    bytes = cvmhip_dense_workspace_bytes(static_cast<int>(in_shapes[0][0]), static_cast<int>(in_shapes[0][1]),
+                                         static_cast<int>(in_shapes[1][0]));
+  } else if (op == "get_valid_counts" && in_shapes.size() >= 1 && in_shapes[0].ndim() == 3) {
+    bytes = cvmhip_get_valid_counts_workspace_bytes(static_cast<int>(in_shapes[0][0]), static_cast<int>(in_shapes[0][1]));
+  } else if (op == "non_max_suppression" && in_shapes.size() >= 1 && in_shapes[0].ndim() == 3) {
+    bytes = cvmhip_nms_workspace_bytes(static_cast<int>(in_shapes[0][0]), static_cast<int>(in_shapes[0][1]),
+                                       static_cast<int>(in_shapes[0][2]));
+  }
+  return static_cast<int64_t>((bytes + 3) / 4);
+}
+
 // ---- the device: memory and copies (cpu_device_api.cc:18-78 is the CPU counterpart).  The new device type takes
 // the next free value of DLDeviceType (include/cvm/dlpack.h:18-25).
 constexpr int kDLHIP = 5;
