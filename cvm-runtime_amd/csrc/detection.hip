@@ -173,6 +173,129 @@ k_nms_rank(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_coun
   if (i < vc && r) atomicAdd(&rank[(int64_t)b * n + i], r);
 }
 
+// ---- ranks by a stable sort, for many rows without a usable top_k.  Counting, for every row, the rows that sort
+// before it costs n^2 comparisons (hours at the 2^24 rows the operator accepts); a least-significant-digit radix
+// sort is the same stable order in four passes over the keys.  key = ~(score ^ 0x80000000) sorts ascending as the
+// score sorts descending, and equal keys keep their order of arrival, i.e. ascending row index -- the order
+// std::stable_sort gives (nms.cc:89-91).  A pass over one 8-bit digit is three launches:
+//   k_radix_hist     every workgroup counts the digits of its RADIX_CHUNK consecutive elements
+//   k_radix_scan     one workgroup per batch turns hist[digit][workgroup] into first positions (exclusive sum in
+//                    digit-major order)
+//   k_radix_scatter  every workgroup moves its elements, in their order, to first position + what came before
+// Everything is integer counts: no float, no order-dependent atomics, so the result is the same on every run.
+// Pass 0 reads the scores from the tensor (row i is element i); the last pass writes rank[row] = position.
+constexpr int RADIX_CHUNK = 2048, RADIX_THREADS = 256, RADIX_ROUNDS = RADIX_CHUNK / RADIX_THREADS;
+constexpr int RADIX_MIN_ROWS = 8192;   // below this the all-pairs count is faster
+
+__device__ __forceinline__ uint32_t radix_key(int32_t score) { return ~((uint32_t)score ^ 0x80000000u); }
+
+__global__ void __launch_bounds__(RADIX_THREADS)
+k_radix_hist(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, const uint32_t* __restrict__ keys_in,
+             int32_t* __restrict__ hist, int n, int k, int score_index, int pass, int nblocks, int64_t key_stride) {
+  __shared__ int s_hist[256];
+  const int b = blockIdx.y, blk = blockIdx.x, tid = threadIdx.x;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  s_hist[tid] = 0;
+  __syncthreads();
+  const int base = blk * RADIX_CHUNK;
+  const int32_t* xb = x + (int64_t)b * n * k;
+  const uint32_t* kin = keys_in + b * key_stride;
+  for (int r = 0; r < RADIX_ROUNDS; ++r) {
+    const int i = base + r * RADIX_THREADS + tid;
+    if (i < vc) {
+      const uint32_t key = pass == 0 ? radix_key(xb[(int64_t)i * k + score_index]) : kin[i];
+      atomicAdd(&s_hist[(key >> (8 * pass)) & 255u], 1);
+    }
+  }
+  __syncthreads();
+  hist[((int64_t)b * 256 + tid) * nblocks + blk] = s_hist[tid];
+}
+
+// exclusive prefix sum over the 256 * nblocks counts of a batch, in place
+__global__ void __launch_bounds__(1024)
+k_radix_scan(const int32_t* __restrict__ valid_count, int32_t* __restrict__ hist, int n, int nblocks) {
+  __shared__ int s_sum[1024];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  if (batch_state(valid_count, b, n) != 0) return;
+  int32_t* h = hist + (int64_t)b * 256 * nblocks;
+  const int total = 256 * nblocks;
+  const int per = (total + 1023) / 1024;
+  const int lo = tid * per < total ? tid * per : total, hi = lo + per < total ? lo + per : total;
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) sum += h[i];
+  s_sum[tid] = sum;
+  __syncthreads();
+  // inclusive scan of the 1024 partial sums
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int v = tid >= d ? s_sum[tid - d] : 0;
+    __syncthreads();
+    s_sum[tid] += v;
+    __syncthreads();
+  }
+  int run = s_sum[tid] - sum;
+  for (int i = lo; i < hi; ++i) {
+    const int c = h[i];
+    h[i] = run;
+    run += c;
+  }
+}
+
+__global__ void __launch_bounds__(RADIX_THREADS)
+k_radix_scatter(const int32_t* __restrict__ x, const int32_t* __restrict__ valid_count, const uint32_t* __restrict__ keys_in,
+                const int32_t* __restrict__ idx_in, uint32_t* __restrict__ keys_out, int32_t* __restrict__ idx_out,
+                const int32_t* __restrict__ hist, int32_t* __restrict__ rank, int n, int k, int score_index, int pass,
+                int nblocks, int64_t key_stride, int last) {
+  __shared__ int s_first[256];      // next free position of every digit for this workgroup
+  __shared__ int s_cnt[4][256];     // elements of the current round per wavefront and digit
+  const int b = blockIdx.y, blk = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (batch_state(valid_count, b, n) != 0) return;
+  const int vc = clamp_vc(valid_count[b], n);
+  const int base = blk * RADIX_CHUNK;
+  if (base >= vc) return;
+  s_first[tid] = hist[((int64_t)b * 256 + tid) * nblocks + blk];
+  const int32_t* xb = x + (int64_t)b * n * k;
+  const uint32_t* kin = keys_in + b * key_stride;
+  const int32_t* iin = idx_in + b * key_stride;
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int r = 0; r < RADIX_ROUNDS; ++r) {
+    for (int w = 0; w < 4; ++w) s_cnt[w][tid] = 0;
+    __syncthreads();
+    const int i = base + r * RADIX_THREADS + tid;
+    const bool live = i < vc;
+    uint32_t key = 0;
+    int row = 0;
+    if (live) {
+      key = pass == 0 ? radix_key(xb[(int64_t)i * k + score_index]) : kin[i];
+      row = pass == 0 ? i : iin[i];
+    }
+    const unsigned digit = (key >> (8 * pass)) & 255u;
+    // lanes of this wavefront that are live and hold the same digit
+    unsigned long long same = __ballot(live);
+#pragma unroll
+    for (int bit = 0; bit < 8; ++bit) {
+      const unsigned long long set = __ballot((digit >> bit) & 1u);
+      same &= ((digit >> bit) & 1u) ? set : ~set;
+    }
+    const int before = __popcll(same & lt);
+    if (live && before == 0) s_cnt[wave][digit] = __popcll(same);   // the first lane of every group of equal digits
+    __syncthreads();
+    if (live) {
+      int pos = s_first[digit] + before;
+      for (int w = 0; w < wave; ++w) pos += s_cnt[w][digit];
+      if (last) {
+        rank[(int64_t)b * n + row] = pos;
+      } else {
+        keys_out[b * key_stride + pos] = key;
+        idx_out[b * key_stride + pos] = row;
+      }
+    }
+    __syncthreads();
+    s_first[tid] += s_cnt[0][tid] + s_cnt[1][tid] + s_cnt[2][tid] + s_cnt[3][tid];
+    __syncthreads();
+  }
+}
+
 // With 0 < top_k <= TOPK_MAX_K only the top_k best rows are ever looked at again, so only they need a
 // rank.  One workgroup per batch keeps every score in registers (thread t owns rows t, t + 1024, ...),
 // finds the top_k-th largest score T by bisection on the bits in which scores differ (ballot counts, no
@@ -609,15 +732,20 @@ static int nms_static_scratch(void** ptr) {
 }
 
 static int nms_check_args(const int32_t* x, const int32_t* valid_count, const int32_t* y, int batches, int n, int k,
-                          int iou_threshold, int coord_start, int score_index, int id_index) {
+                          int iou_threshold, int coord_start, int score_index, int id_index, int topk) {
   if (!x || !valid_count || !y || x == y || batches < 1 || n < 1 || k < 2 || batches > 65535)
     return arg_error("non_max_suppression");
   if (iou_threshold <= 0) return arg_error("non_max_suppression.iou_threshold must be positive");
   if (coord_start < 0 || coord_start + 4 > k || score_index < 0 || score_index >= k || id_index >= k)
     return arg_error("non_max_suppression indices");
-  // 2^24 is the largest dimension the reference's shape check accepts (src/runtime/infer_attr.cc); without top_k
-  // the ranking compares all pairs of valid rows, as the reference's greedy walk does in its worst case
+  // 2^24 is the largest dimension the reference's shape check accepts (src/runtime/infer_attr.cc).  Ranking is a sort, but
+  // the greedy walk over the candidate rows (the first top_k in sorted order, or all valid rows) compares every kept
+  // row with every later one, as the reference's does: one workgroup needs about 0.8 s for 100 000 candidate rows of
+  // which most are kept, and the time grows with the square.  More than 2^18 candidates (about 5 s at worst) are
+  // refused rather than launched as a kernel that runs for minutes.
   if (n > (1 << 24)) return arg_error("non_max_suppression: more than 2^24 anchors per batch");
+  if (n > (1 << 18) && !(topk >= 0 && topk <= (1 << 18)))
+    return arg_error("non_max_suppression: more than 2^18 candidate rows per batch (set top_k to bound the greedy walk)");
   return CVMHIP_OK;
 }
 
@@ -637,6 +765,26 @@ static int nms_launch(int32_t* x, const int32_t* valid_count, int32_t* y,
   if (topk > 0 && topk <= TOPK_MAX_K && n <= TOPK_MAX_N) {
     k_nms_topk_rank<<<batches, TOPK_THREADS, 0, s>>>(x, valid_count, rank, n, k, score_index, topk);
     rc = check_launch("nms.topk_rank");
+  } else if (n >= RADIX_MIN_ROWS) {
+    // stable radix sort: two key and two index buffers and the digit counts, behind the bit matrix
+    const int nblocks = (n + RADIX_CHUNK - 1) / RADIX_CHUNK;
+    uint32_t* keys[2];
+    int32_t* idx[2];
+    keys[0] = mask + (size_t)batches * NMS_BM_ROWS * NMS_BM_WORDS;
+    keys[1] = keys[0] + (size_t)batches * n;
+    idx[0] = reinterpret_cast<int32_t*>(keys[1] + (size_t)batches * n);
+    idx[1] = idx[0] + (size_t)batches * n;
+    int32_t* hist = idx[1] + (size_t)batches * n;
+    rc = CVMHIP_OK;
+    for (int pass = 0; pass < 4 && !rc; ++pass) {
+      const int in = (pass + 1) & 1, out = pass & 1;   // pass 0 reads the tensor itself
+      dim3 grid(nblocks, batches);
+      k_radix_hist<<<grid, RADIX_THREADS, 0, s>>>(x, valid_count, keys[in], hist, n, k, score_index, pass, nblocks, (int64_t)n);
+      k_radix_scan<<<batches, 1024, 0, s>>>(valid_count, hist, n, nblocks);
+      k_radix_scatter<<<grid, RADIX_THREADS, 0, s>>>(x, valid_count, keys[in], idx[in], keys[out], idx[out], hist, rank, n, k,
+                                                     score_index, pass, nblocks, (int64_t)n, pass == 3 ? 1 : 0);
+      rc = check_launch("nms.radix_sort");
+    }
   } else {
     k_zero32<<<grid_for((int64_t)batches * n, 256), 256, 0, s>>>(rank, (int64_t)batches * n);
     dim3 rgrid((n + 255) / 256, (n + RANK_JT - 1) / RANK_JT, batches);
@@ -692,9 +840,12 @@ int cvmhip_get_valid_counts(const int32_t* x, int32_t* valid_count, int32_t* y,
   return check_launch("get_valid_counts.scatter");
 }
 
-// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix
+// per batch: order[n], nextneg[n+1], removed[n], sorted[n*k], rank[n], suppression bit matrix; from RADIX_MIN_ROWS rows on
+// also the radix sort's two key buffers, two index buffers and digit counts
 size_t cvmhip_nms_workspace_bytes(int batches, int n, int k) {
-  return (size_t)batches * ((size_t)n * (4 + (size_t)k) + 2 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS) * sizeof(int32_t);
+  size_t per = (size_t)n * (4 + (size_t)k) + 2 + (size_t)NMS_BM_ROWS * NMS_BM_WORDS;
+  if (n >= RADIX_MIN_ROWS) per += (size_t)n * 4 + (size_t)256 * ((n + RADIX_CHUNK - 1) / RADIX_CHUNK);
+  return (size_t)batches * per * sizeof(int32_t);
 }
 
 int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* y,
@@ -702,7 +853,7 @@ int cvmhip_non_max_suppression(int32_t* x, const int32_t* valid_count, int32_t* 
                                int iou_threshold, int topk, int coord_start,
                                int score_index, int id_index, int force_suppress,
                                void* workspace, size_t workspace_bytes, void* stream) {
-  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index);
+  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index, topk);
   if (rc) return rc;
   if (!workspace || workspace_bytes < cvmhip_nms_workspace_bytes(batches, n, k)) return arg_error("non_max_suppression workspace");
   return nms_launch(x, valid_count, y, batches, n, k, max_output_size, iou_threshold, topk, coord_start, score_index,
@@ -715,7 +866,7 @@ int cvmhip_non_max_suppression_static(int32_t* x, const int32_t* valid_count, in
                                       int batches, int n, int k, int max_output_size,
                                       int iou_threshold, int topk, int coord_start,
                                       int score_index, int id_index, int force_suppress, void* stream) {
-  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index);
+  const int rc = nms_check_args(x, valid_count, y, batches, n, k, iou_threshold, coord_start, score_index, id_index, topk);
   if (rc) return rc;
   const size_t need = cvmhip_nms_workspace_bytes(batches, n, k);
   if (need > cvmhip_nms_static_capacity_bytes()) {

@@ -344,6 +344,27 @@ def test_nms_top_k_selection(score, topk, n, dev):
     same(tx, x_after, "nms input after the call")
 
 
+@pytest.mark.parametrize("b,n,score,topk,extent", [
+    (1, 24564, (-127, 127), -1, 16),             # the detector's anchor count without top_k: long runs of equal scores
+    (2, 100000, (-1000, 1000), -1, 12),
+    (1, 20000, (-2 ** 31, 2 ** 31 - 1), 3000, 24),   # top_k above what the selection path takes; keys differ in every bit
+    (2, 8192, (0, 3), -1, 8),                     # the fewest rows that are sorted; four distinct scores
+    (2, 8191, (0, 3), -1, 8),                     # one fewer: ranked by counting
+    (1, 70000, (5, 5), 40000, 10),                # every score equal: the order is the row index alone
+])
+def test_nms_many_rows_without_usable_top_k_are_ranked_by_a_stable_sort(b, n, score, topk, extent, dev):
+    """From 8192 rows on, rows are ranked by a least-significant-digit radix sort on (score descending) that keeps rows
+    of equal score in index order -- the order of the reference's std::stable_sort (nms.cc:89-91)."""
+    x = _boxes("nms-sort-%d-%d-%s" % (b, n, score), b, n, -1, 3, score=score, extent=extent)
+    vc = np.array([n - 777 * i for i in range(b)], np.int32)
+    init = np.full_like(x, 5)
+    y_ref, x_after = oracle.non_max_suppression(x, vc, 45, False, topk, y_init=init)
+    tx, ty = T(x, dev), T(init, dev)
+    hipops.non_max_suppression(tx, T(vc, dev), ty, 45, False, topk)
+    same(ty, y_ref, "nms output")
+    same(tx, x_after, "nms input after the call")
+
+
 def test_nms_stops_at_first_batch_without_valid_rows(dev):
     x = _boxes("nms-early", 3, 40, 0, 3, extent=32)
     vc = np.array([12, 0, 30], np.int32)
@@ -370,3 +391,8 @@ def test_argument_errors_are_reported_not_launched(dev):
     x = T(np.zeros((1, 4, 6), np.int32), dev)
     with pytest.raises(CvmHipError):
         hipops.non_max_suppression(x, T(np.ones((1,), np.int32), dev), torch.empty_like(x), iou_threshold=0)
+    # more candidate rows than the greedy walk is allowed: refused unless top_k bounds them
+    big = torch.zeros((1, (1 << 18) + 1, 6), dtype=torch.int32, device=dev)
+    with pytest.raises(CvmHipError):
+        hipops.non_max_suppression(big, T(np.ones((1,), np.int32), dev), torch.empty_like(big), iou_threshold=45)
+    hipops.non_max_suppression(big, T(np.ones((1,), np.int32), dev), torch.empty_like(big), iou_threshold=45, top_k=100)
