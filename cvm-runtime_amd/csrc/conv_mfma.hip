@@ -414,6 +414,15 @@ __device__ __forceinline__ int4 fetch_act(const int8_t* __restrict__ xp, const C
   }
 }
 
+// XCD-aware tile order.  Workgroups are dealt round-robin to the 8 XCDs (workgroup w runs on XCD w % 8), and each XCD
+// has an L2 of its own, so the tiles are renumbered to give every XCD one contiguous run of them: neighbouring tiles
+// (the channel tiles of the same pixels, then the next pixels) share their operands in that XCD's L2.  Any grid size:
+// XCD x holds ceil((nb - x) / 8) workgroups, its run starts after those of the XCDs before it.
+__device__ __forceinline__ int xcd_tile_order(int pid, int nb) {
+  const int x = pid & 7, per = nb >> 3, extra = nb & 7;
+  return x * per + (x < extra ? x : extra) + (pid >> 3);
+}
+
 template <int WM, int WN, int G, int KS, int OUT>
 __global__ void __launch_bounds__(256)
 k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void* __restrict__ out,
@@ -435,12 +444,8 @@ k_conv_igemm(const int8_t* __restrict__ xp, const int8_t* __restrict__ wp, void*
   const int lrow = lane & 31;
   const int lgrp = lane >> 5;
 
-  // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so
-  // give each XCD a contiguous run of tiles (neighbouring tiles share the
-  // activation slab in that XCD's L2).
-  int pid = blockIdx.x;
   const int nb = gridDim.x;
-  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);
+  const int pid = xcd_tile_order(blockIdx.x, nb);
   const int oc_tiles = (g.OC + BM - 1) / BM;
   const int oc0 = (pid % oc_tiles) * BM;
   const int64_t px0 = (int64_t)(pid / oc_tiles) * BN;
@@ -1079,9 +1084,7 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
   constexpr int U = TM * TN * 4;
   __shared__ __attribute__((aligned(16))) int sPart[KSPLIT > 1 ? NW * U * 256 : 4];  // [wave][group][lane][4]
   __shared__ __attribute__((aligned(16))) int sBias[32 * TM * (KSPLIT == 1 ? NW : 1)];
-  int pid = blockIdx.x;
-  const int nb = gridDim.x;
-  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);  // contiguous tile runs per XCD
+  const int pid = xcd_tile_order(blockIdx.x, gridDim.x);
   conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT, MODE, SLICES, false, POOLR>(xp, wf, out, g, ep, pid, threadIdx.x, sPart, sBias);
 }
 
@@ -1148,9 +1151,7 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
   const int lrow = lane & 31, lgrp = lane >> 5;
-  int pid = blockIdx.x;
-  const int nb = gridDim.x;
-  if ((nb & 7) == 0) pid = (pid & 7) * (nb >> 3) + (pid >> 3);   // contiguous tile runs per XCD
+  const int pid = xcd_tile_order(blockIdx.x, gridDim.x);
   const int ptile = (int)fastdiv((unsigned)pid, g.div_octiles);
   const int oc0 = (pid - ptile * g.octiles) * BM;
   const int px0 = ptile * BN;
@@ -1595,13 +1596,15 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
       sLayer[(l + 1) & 1][tid] = next0;
       if (tid + 64 < LWORDS) sLayer[(l + 1) & 1][tid + 64] = next1;
     }
-    // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
+    // ---- done with the layer: every wavefront counts itself out as soon as its own stores are in the L2 (the counter
+    // counts wavefronts, 8 per workgroup), so a workgroup's slowest wavefront holds back only its own count; the barrier
+    // behind it is for the table entry in LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #ifdef CVM_SEQ_STAMPS
     if (tr && tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
 #endif
-    if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   // the last workgroup of a share to finish clears the share's counters for the next launch
   __syncthreads();
