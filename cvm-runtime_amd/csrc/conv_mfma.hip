@@ -1596,9 +1596,7 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
       sLayer[(l + 1) & 1][tid] = next0;
       if (tid + 64 < LWORDS) sLayer[(l + 1) & 1][tid + 64] = next1;
     }
-    // ---- done with the layer: every wavefront counts itself out as soon as its own stores are in the L2 (the counter
-    // counts wavefronts, 8 per workgroup), so a workgroup's slowest wavefront holds back only its own count; the barrier
-    // behind it is for the table entry in LDS
+    // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
