@@ -235,7 +235,7 @@ int conv_group_launch(const void* dev_table, int nlayers, int total_blocks, int 
 int conv_igemm_ws(const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep, void* ws, size_t ws_bytes,
                   hipStream_t s);
 
-// ---- a run of convolutions in one launch (k_conv_seq), for batches that are a multiple of 8: every XCD computes all
+// ---- a run of convolutions in one launch (k_conv_seq): every XCD (of the 8, 4, 2 or 1 that divide the batch) computes all
 // layers for its share of the images and layer boundaries are counters in that XCD's L2.  The caller builds a host
 // table with conv_seq_layer (one entry per convolution, in order; each must only read tensors that earlier entries
 // or earlier launches wrote), copies it to the device and launches it; `sync` is conv_seq_sync_bytes() of zeroed

@@ -1479,7 +1479,8 @@ struct SeqLayer {
   int kernel;          // configuration * 3 + mode (identity, no padding, padding)
   int px_per_share;    // output pixels of one share of the images
   int ptiles;          // pixel tiles that cover a share (its first block may begin before the share)
-  int reserved[3];     // keeps the entry a multiple of 16 bytes
+  int shares;          // XCDs that take part: the largest of 1, 2, 4, 8 that divides the batch; the others leave at once
+  int reserved[2];     // keeps the entry a multiple of 16 bytes
 };
 constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
 enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
@@ -1538,6 +1539,9 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   unsigned xcc;
   asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
   xcc &= 15u;
+  __syncthreads();   // the first table entry is in LDS
+  // a batch that does not divide over all 8 XCDs runs on the first `shares` of them; a workgroup elsewhere has nothing to do
+  if (xcc < SEQ_SHARES && (int)xcc >= reinterpret_cast<const SeqLayer*>(sLayer[0])->shares) return;
   unsigned* my = sync + (xcc < SEQ_SHARES ? xcc : 0) * SEQ_SYNC_WORDS;
   unsigned* error = sync + SEQ_SHARES * SEQ_SYNC_WORDS;
   if (tid == 0) {
@@ -2577,9 +2581,8 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   const int prc = conv_prepare(xp, wp, out, g, ep_in, ep);
   if (prc) return prc;
   const bool nopad = g.PH == 0 && g.PW == 0;
-  if (g.N % SEQ_SHARES != 0 || (g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT || ep.pool ||
-      !(nopad || (g.KH <= 32 && g.KW <= 32)))
-    return arg_error("conv_seq_layer: not eligible (batch not a multiple of 8, few-channel input, depthwise or int32 output)");
+  if ((g.Cp % 32) != 0 || g.row_bytes != 0 || g.dw || ep.out_mode != OUT_I8_ACT || ep.pool || !(nopad || (g.KH <= 32 && g.KW <= 32)))
+    return arg_error("conv_seq_layer: not eligible (few-channel input, depthwise or int32 output)");
   // results are stored through a buffer descriptor with 32-bit offsets
   if (act_bytes(g.P, ep.out_cp) > INT32_MAX) return arg_error("conv_seq_layer: not eligible (output tensor of 2 GiB or more)");
   const ConvTuning tune = t_conv_tuning;
@@ -2589,7 +2592,11 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
     return arg_error("conv_seq_layer: not eligible (a layer for the large-tile kernel)");
   SeqLayer& L = reinterpret_cast<SeqLayer*>(table)[index];
   memset(&L, 0, sizeof(L));
-  L.px_per_share = (int)(g.P / SEQ_SHARES);
+  // whole images per share: as many XCDs as divide the batch (8, 4, 2 or 1)
+  int shares = SEQ_SHARES;
+  while (g.N % shares != 0) shares >>= 1;
+  L.shares = shares;
+  L.px_per_share = (int)(g.P / shares);
   // the configuration is chosen for one share on the 32 compute units of its XCD
   ConvGeom share = g;
   share.P = L.px_per_share;
@@ -2606,7 +2613,7 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
   // a share begins at a multiple of px_per_share, which need not be a multiple of 32: its first pixel block
   // may start up to 31 pixels early (those pixels are computed and not stored)
   int ptiles = 0;
-  for (int x = 0; x < SEQ_SHARES; ++x) {
+  for (int x = 0; x < shares; ++x) {
     const int lead = (x * L.px_per_share) & 31;
     const int t = (lead + L.px_per_share + bn - 1) / bn;
     ptiles = t > ptiles ? t : ptiles;

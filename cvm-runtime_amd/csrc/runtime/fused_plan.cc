@@ -846,9 +846,9 @@ void HipGraphRuntime::BuildGroups() {
   if (!hooks_.head_group) { groups_.clear(); group_at_.assign(plan_.size(), -1); }
   // The same for consecutive convolutions with int8 output that do not read one another's results (at a small batch the
   // first 1x1 layer and the shortcut projection of a ResNet block, which the planner has put side by side), as long as
-  // all of them together are one round of workgroups (two per CU); only when no layer-sequence launch exists, which
-  // covers such layers at its batch sizes.
-  if (!hooks_.conv_group || !seqs_.empty()) return;
+  // all of them together are one round of workgroups (two per CU).  They are what runs when the model's sequence
+  // launches are not in use (Launch() takes a sequence launch first where both exist).
+  if (!hooks_.conv_group) return;
   i = 0;
   while (i < plan_.size()) {
     table.clear();

@@ -748,15 +748,15 @@ void HipGraphRuntime::Launch() {
   if (fused_) {
     const bool seq = seq_mode_;
     for (size_t i = 0; i < plan_.size();) {
-      if (!group_at_.empty() && group_at_[i] >= 0) {
-        const GroupRun& r = groups_[group_at_[i]];
-        if (r.i8) HipCheck(cvmhip_conv_group_launch_i8(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped convolutions");
-        else HipCheck(cvmhip_conv_group_launch(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped detection heads");
-        i = r.last + 1;
-      } else if (seq && seq_at_[i] >= 0) {
+      if (seq && seq_at_[i] >= 0) {   // (a sequence launch covers whatever grouped launches lie inside its run)
         const SeqRun& r = seqs_[seq_at_[i]];
         HipCheck(cvmhip_conv_seq_launch(r.table, r.nlayers, seq_sync_, r.ops, r.bytes, stream_), "layer-sequence launch");
         seq_ran_ = true;
+        i = r.last + 1;
+      } else if (!group_at_.empty() && group_at_[i] >= 0) {
+        const GroupRun& r = groups_[group_at_[i]];
+        if (r.i8) HipCheck(cvmhip_conv_group_launch_i8(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped convolutions");
+        else HipCheck(cvmhip_conv_group_launch(r.table, r.nlayers, r.blocks, r.ops, r.bytes, stream_), "grouped detection heads");
         i = r.last + 1;
       } else {
         RunStep(plan_[i++]);

@@ -164,8 +164,13 @@ class HipGraphRuntime {
     int seq = 0, lay = 0;
     if (SeqNow())
       for (const SeqRun& r : seqs_) { ++seq; lay += r.nlayers; }
-    int grouped = 0;
-    for (const GroupRun& r : groups_) grouped += r.nlayers - 1;
+    int grouped = 0;   // launches saved by grouped launches; a group inside a sequence launch that is in use saves none
+    for (const GroupRun& r : groups_) {
+      bool inside = false;
+      if (SeqNow())
+        for (const SeqRun& q : seqs_) inside = inside || (r.first >= q.first && r.last <= q.last);
+      if (!inside) grouped += r.nlayers - 1;
+    }
     if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq - (fused_ ? grouped : 0);
     if (sequences) *sequences = seq;
     if (layers) *layers = lay;

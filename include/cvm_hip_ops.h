@@ -323,8 +323,9 @@ int cvmhip_conv2d_pool2_i8_eligible(int n, int ic, int h, int wd, int oc, int kh
 int cvmhip_conv2d_pool2_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain, void* out,
                            int n, int ic, int h, int wd, int oc, int kh, int kw,
                            int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
-/* A run of convolutions in ONE launch, for a batch that is a multiple of cvmhip_conv_seq_shares() (8, the XCDs
- * of the chip).  No counterpart in the reference.  Images are independent, so every XCD computes all layers
+/* A run of convolutions in ONE launch.  No counterpart in the reference.  The images are dealt to
+ * cvmhip_conv_seq_shares() XCDs (8) when the batch is a multiple of it, else to the largest of 4, 2, 1 that divides
+ * the batch (the other XCDs' workgroups leave at once).  Images are independent, so every XCD computes all layers
  * of the run for its own share of the images; a layer boundary is then a counter in that XCD's L2 instead of a
  * kernel boundary (no L2 write-back, the next layer's operands are still in the L2).  Use: fill a host table of
  * n * cvmhip_conv_seq_layer_bytes() bytes with cvmhip_conv_seq_layer (entry i describes what

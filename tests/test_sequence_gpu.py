@@ -77,6 +77,15 @@ CHAINS = {
                                               (96, 1, 1, False, None)]),
     "b8_many_tiles_two_rounds": (8, 3, 40, [(64, 0, 0, 0, None), (256, 1, 1, True, None), (64, 1, 1, True, None), (64, 3, 1, True, None),
                                             (256, 1, 1, False, 1)]),
+    # batches that do not divide over the 8 XCDs run on 1, 2 or 4 of them
+    "b1_one_xcd": (1, 3, 28, [(64, 0, 0, 0, None), (256, 1, 1, True, None), (64, 1, 1, True, None), (64, 3, 1, True, None),
+                              (256, 1, 1, False, 1), (128, 3, 2, True, None)]),
+    "b2_two_xcds": (2, 3, 9, [(32, 0, 0, 0, None), (128, 1, 1, True, None), (128, 3, 1, True, None), (512, 1, 1, True, None),
+                              (96, 1, 1, False, None)]),
+    "b3_one_xcd_three_images": (3, 3, 10, [(32, 0, 0, 0, None), (64, 3, 1, True, None), (64, 1, 1, True, None), (64, 3, 2, True, None),
+                                           (160, 1, 1, False, None)]),
+    "b12_four_xcds": (12, 3, 8, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (64, 3, 1, True, None), (256, 1, 1, False, None),
+                                 (64, 1, 1, True, None)]),
 }
 
 
