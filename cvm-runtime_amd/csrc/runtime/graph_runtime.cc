@@ -561,8 +561,14 @@ void HipGraphRuntime::SetDataI8(const int8_t* host, const Shape& shape) {
     HipCheck(cvmhip_alloc(&in_stage_dev_, size), "input staging buffer");
   }
   HipCheck(cvmhip_stream_sync(stream_), "copy input to device");  // the previous copy out of the staging buffer is done
-  std::memcpy(in_stage_host_, host, size);
-  HipCheck(cvmhip_copy_h2d(in_stage_dev_, in_stage_host_, size, stream_), "copy input to device");
+  // The caller's bytes go through the pinned buffer in pieces: while the copy engine moves one piece to the device the
+  // host already copies the next into the buffer, so of the two copies only the longer one is on the call's clock.
+  const size_t piece = std::max<size_t>((size / 4 + 4095) & ~static_cast<size_t>(4095), 256 << 10);
+  for (size_t at = 0; at < size; at += piece) {
+    const size_t len = std::min(piece, size - at);
+    std::memcpy(static_cast<char*>(in_stage_host_) + at, reinterpret_cast<const char*>(host) + at, len);
+    HipCheck(cvmhip_copy_h2d(static_cast<char*>(in_stage_dev_) + at, static_cast<char*>(in_stage_host_) + at, len, stream_), "copy input to device");
+  }
   HipCheck(cvmhip_widen_clamp_i8(in_stage_dev_, entry_ptr_[eid], static_cast<int64_t>(size), range, stream_), "widen input");
 }
 
