@@ -82,6 +82,12 @@ def run(reps=20):
     rows[-1]["achieved_GBps"] = rows[-1]["algorithmic_bytes"] / rows[-1]["us_per_call"] / 1e3
     rows[-1]["frac_of_hbm_peak"] = rows[-1]["achieved_GBps"] / HBM_PEAK_GBS
 
+    # the same rows without top_k: ranked by the stable radix sort (12 launches), then every valid row is a candidate of the
+    # greedy walk, whose time grows with the square of their number -- a few repetitions are enough
+    def nms_all():
+        hipops.non_max_suppression(rows_sorted.clone(), vc, ny, 45, False, -1)
+    add("non_max_suppression iou 45 without top_k", "1x24564x6 int32, %d valid rows" % int(vc.item()), 4 * 2 * nb, nms_all, r=3)
+
     # ---- fused int8 forms (what the graph executor runs): one byte per element
     xa = hipops.pack_act_i8(_rand(act, -127, 127, dev))
     xb = hipops.pack_act_i8(_rand(act, -127, 127, dev))

@@ -112,6 +112,9 @@ def test_config4_vgg16_batch16_matches_per_image_runs(dev):
         o = np.frombuffer(m1.inference(x[i:i + 1].tobytes()), np.int32)
         assert np.array_equal(o, out16[i]), "image %d differs between batch 16 and batch 1" % i
     m1.close()
+    # and one image of the batch straight against the oracle's graph executor (the compiled reference where it is built)
+    ref = og.run_graph(js1, graphgen.load_params(pb1), x[9:10].astype(np.int32))
+    assert np.array_equal(ref[0].ravel(), out16[9])
 
 
 @pytest.mark.parametrize("neg_ids", [False, True])
