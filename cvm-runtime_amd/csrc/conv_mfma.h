@@ -84,7 +84,20 @@ struct Epilogue {
   int o32_ch_b, o32_px_b;
   int64_t o32_img_b;
   int32_t* out_b;
+  // which parts of which stages of chain / chain2 do anything (chain_flags_of), filled by conv_igemm: one scalar word a
+  // kernel branches on instead of comparing the stage parameters themselves (0: not filled, the kernel works them out)
+  unsigned chain_flags, chain2_flags;
 };
+// bit 31: valid; stage t (bits 5t .. 5t+4): exists, multiplies, shifts before the add, adds, shifts after it
+__host__ __device__ inline unsigned chain_flags_of(const DevChain& c) {
+  unsigned f = 0x80000000u;
+  for (int t = 0; t < 4; ++t) {
+    if (t >= c.count) break;
+    const DevStage& q = c.st[t];
+    f |= (1u | (q.mul != 1 ? 2u : 0u) | (q.s1 != 0 ? 4u : 0u) | (q.add != 0 ? 8u : 0u) | (q.s2 != 0 ? 16u : 0u)) << (5 * t);
+  }
+  return f;
+}
 
 // ---- int8 activation layout.  Channels are padded to Cp = 4, 8, 16 or a
 // multiple of 32.  Cp <= 16: plain NHWC.  Cp % 32 == 0: "pixel-blocked" -- the
@@ -178,6 +191,7 @@ struct ConvTuning {
   unsigned long long* seq_stamps;   // device memory for time stamps inside sequence launches (nullptr: none), see CVM_SEQ_STAMP
   int seq_stamp_layers;             // layers it has room for: 256 workgroups x layers x 8 words
   signed char seq_layer_cfg[64];    // configuration forced for entry i of the next sequence tables (-1: automatic)
+  int seq_chains;                   // 1: conv_seq_link may chain 1x1 layers behind the layer that feeds them
 };
 void set_conv_tuning(const ConvTuning& t);
 
@@ -246,6 +260,8 @@ size_t conv_seq_sync_bytes();
 int conv_seq_shares();
 int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep);
 int conv_seq_layer_config(const void* table, int index);   // configuration of the tile kernel chosen for an entry
+int conv_seq_layer_chain(const void* table, int index);    // entries chained behind this one (0, 1 or 2)
+int conv_seq_link(void* table, int count);                 // chains 1x1 layers behind the layer that feeds them; returns the chains found
 int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s);
 
 }  // namespace cvmhip

@@ -53,27 +53,36 @@ __device__ __forceinline__ int32_t clamp3(int32_t v, int32_t lo, int32_t hi) {
 // in place under a wave-uniform condition: a loop over the stages, or alternative forms of a stage
 // that meet at a join, make the compiler copy all N registers from one set to another at every edge
 // (measured: 40 % of the vector instructions of an epilogue were such copies).
-template <int N>
-__device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N]) {
+constexpr int SEQ_MAX_STAGES = 2;   // stages per chain of a layer inside a layer-sequence launch
+// `flags` (chain_flags_of, or 0: worked out here) says which parts exist, in one word that is made a scalar: the
+// conditions are then scalar bit tests whatever registers the stage parameters themselves arrive in (read from a table
+// in LDS they are vector registers, and a comparison of those is a vector compare, a wait for its result and a
+// branch -- twenty of them per chain).
+// MAXST, MUL: the caller knows that the chain has at most MAXST stages and (MUL false) none that multiplies -- the
+// layer-sequence kernel, whose host side admits no other layers: every layer of a sequence executes its epilogue code
+// once or twice, straight from memory, and code for stages that never occur is fetched like any other.
+template <int N, int MAXST = 4, bool MUL = true>
+__device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N], const unsigned flags = 0u) {
+  const unsigned f = (unsigned)__builtin_amdgcn_readfirstlane((int)((flags & 0x80000000u) ? flags : chain_flags_of(c)));
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    if (t < c.count) {
+  for (int t = 0; t < MAXST; ++t) {
+    if (f & (1u << (5 * t))) {
       const DevStage q = c.st[t];
 #pragma unroll
       for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], q.lo, q.hi);
-      if (q.mul != 1) {   // a multiplication stage (rare)
+      if (MUL && (f & (2u << (5 * t)))) {   // a multiplication stage (rare)
 #pragma unroll
         for (int e = 0; e < N; ++e) v[e] = wmul(v[e], q.mul);
       }
-      if (q.s1 != 0) {
+      if (f & (4u << (5 * t))) {
 #pragma unroll
         for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s1;
       }
-      if (q.add != 0) {
+      if (f & (8u << (5 * t))) {
 #pragma unroll
         for (int e = 0; e < N; ++e) v[e] = wadd(v[e], q.add);
       }
-      if (q.s2 != 0) {
+      if (f & (16u << (5 * t))) {
 #pragma unroll
         for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s2;
       }
@@ -121,14 +130,20 @@ __device__ __forceinline__ void mask_channels(uint32_t (&d)[N], int first, int O
 // outside every buffer (sizes stay below 2^31) and reads as zeros.
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 constexpr unsigned kOutsideBuffer = 0x80000000u;
+// The base address is the same in every lane and is put into scalar registers explicitly: read from a table in LDS it
+// arrives in vector registers, and a memory instruction whose descriptor is not known to be uniform is wrapped into a
+// loop over the distinct descriptor values of the lanes (a dozen instructions around every load and store).
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t act_rsrc(const void* base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+  const uintptr_t b = (uintptr_t)base;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uintptr_t)hi << 32) | lo), 0, 0x7fffffff, 0x00020000);
 }
 // `off` is the lane's own offset (the one the descriptor's range check sees), `uni` a wave-uniform one that the
 // instruction adds from a scalar register: it costs no vector instruction
 template <bool COH>
 __device__ __forceinline__ int4 ld16_buf(__amdgpu_buffer_rsrc_t rs, unsigned off, unsigned uni = 0) {
-  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)uni, COH ? 16 : 0);
+  // (said to be uniform explicitly, for the same reason as the descriptor's base address: computed from a table in LDS)
+  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, __builtin_amdgcn_readfirstlane((int)uni), COH ? 16 : 0);
   return make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
 }
 // Stores through a buffer descriptor: a 32-bit offset per lane instead of a 64-bit address, and the instruction is a
@@ -253,7 +268,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
           const int32_t ab = a > b ? a : b, cd = c > d ? c : d;
           red[qe] = ab > cd ? ab : cd;
         }
-        run_chain(ep.chain, red);
+        run_chain(ep.chain, red, ep.chain_flags);
         uint32_t a = pack_bytes(red[0], red[1], red[2], red[3]), b = pack_bytes(red[4], red[5], red[6], red[7]),
                  c = pack_bytes(red[8], red[9], red[10], red[11]), d = pack_bytes(red[12], red[13], red[14], red[15]);
         half_swap(a, c);
@@ -273,7 +288,8 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   }
   // one copy of each step, the residual part an update in place under a uniform condition (two
   // alternative paths that meet again cost a register-to-register copy of every value)
-  run_chain(ep.chain, val);
+  constexpr int MAXST = RANGE ? SEQ_MAX_STAGES : 4;   // RANGE: a layer of a sequence (conv_seq_layer admits short chains only)
+  run_chain<NG * 4, MAXST, !RANGE>(ep.chain, val, ep.chain_flags);
   if (ep.residual) {   // rp holds what load_residual fetched
     if (whole) {
 #pragma unroll
@@ -286,7 +302,7 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     }
 #pragma unroll
     for (int e = 0; e < NG * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
-    run_chain(ep.chain2, val);
+    run_chain<NG * 4, MAXST, !RANGE>(ep.chain2, val, ep.chain2_flags);
   }
 
   if (OUT == OUT_I32_NCHW) {
@@ -655,6 +671,22 @@ __device__ __forceinline__ unsigned tap_mask_dilated(int x0, int extent, int k, 
 //                    out-of-image granules are read from a zero granule
 enum { WAVE_IDENT = 0, WAVE_NOPAD = 1, WAVE_PAD = 2, WAVE_ROWS = 3 };
 
+struct alignas(16) SeqLayer {
+  const int8_t* xp;
+  const int8_t* wf;
+  void* out;
+  ConvGeom g;
+  Epilogue ep;
+  int kernel;          // configuration * 3 + mode (identity, no padding, padding)
+  int px_per_share;    // output pixels of one share of the images
+  int ptiles;          // pixel tiles that cover a share (its first block may begin before the share)
+  int shares;          // XCDs that take part: the largest of 1, 2, 4, 8 that divides the batch; the others leave at once
+  int chain;           // 1 or 2: the next one or two entries are 1x1 layers over this layer's output pixels, computed by the
+                       // same wavefront from registers (conv_chain_tail); they are then not layers of their own
+};
+constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
+enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
+
 // One tile set of the wavefront-private kernel: workgroup-level tile `pid` (channel tile fastest) of the
 // pixel range [p_begin, p_end) (COH only; otherwise the whole layer), computed by the NW wavefronts whose thread index is `tid`, with
 // sPart / sBias their LDS.  k_conv_wave is this function over a grid; the layer-sequence kernel calls it
@@ -670,6 +702,7 @@ struct LayerGate {
   unsigned* error;
   int spin_limit;
   unsigned* seen;      // LDS word of the workgroup (or of its half): the highest target its first wavefront has seen reached
+  int role;            // -1: the wavefront with index 0 in the tile polls the counter, the others watch `seen`; 0: this one polls; 1: watches
 };
 __device__ __forceinline__ void gate_poll(const LayerGate& gate) {
   if (!gate.counter) return;
@@ -723,12 +756,190 @@ __device__ __forceinline__ void gate_wait(const LayerGate& gate, const int wave)
 #else
 #define CVM_SEQ_STAMP(i, dep) do { } while (0)
 #endif
-template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH, bool POOLR = false>
+// One request: 16 bytes per lane from `gaddr` (any address per lane) to LDS byte lds_base + 16 * lane.  Written as
+// assembly on purpose: the compiler then neither counts these requests nor protects LDS reads against them (it would
+// wait for every outstanding one before the first ds_read of a step, which undoes the ring); the waits are wait_vm.
+
+typedef int8_t __attribute__((address_space(3))) * lptr_t;
+__device__ __forceinline__ void lds_dma16(const void* gaddr, uint32_t lds_base) {
+  // (the s_nop is the wait state an instruction that reads M0 needs after a scalar write to it; inside inline assembly
+  // nobody inserts it for us)
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(lds_base) : "memory");
+}
+
+// ---------------------------------------------------------------- 1x1 layers computed from registers
+// A 1x1 convolution with stride 1 needs, for a block of 32 pixels, nothing but the same 32 pixels of its input.  When
+// a wavefront holds a layer's result for a block of pixels with ALL its channels, the requantised int8 values of a
+// 32-channel tile, 16 consecutive channels per lane, are at once the KiB block that is stored and the operand an MFMA
+// of the next layer takes for those 32 channels of its K: the next layer can be computed right there, with no trip
+// through memory, no other wavefront and no layer boundary.  conv_chain_tail does that for one or two such layers
+// behind layer A (whose MT2 accumulator tiles the caller hands over): layer B (any number TB of 32-channel tiles,
+// optional residual) one tile at a time -- MT2 MFMAs, requantise, store -- and each finished tile is at once multiplied
+// into the MT1 accumulator tiles of layer C (MT1 = 0: no layer C), which are requantised and stored at the end.
+// Every result is the one the layers give on their own: the same integer sums, the same chains.
+//
+// One accumulator tile (32 channels x 32 pixels; element e of a lane: channel (e / 4) * 8 + (lane / 32) * 4 + e % 4 of
+// pixel lane % 32) -> v = chain(acc); if (residual) v = chain2(v + residual); int8, 16 consecutive channels per lane.
+// `res`: the lane's 16 bytes of the residual tensor's KiB block for the same pixels and channels.
+__device__ __forceinline__ v4i requant_tile(const v16i acc, const Epilogue& ep, const int4 res) {
+  int32_t val[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) val[e] = acc[e];
+  run_chain<16, SEQ_MAX_STAGES, false>(ep.chain, val, ep.chain_flags);
+  if (ep.residual) {
+    uint32_t a = (uint32_t)res.x, b = (uint32_t)res.y, c = (uint32_t)res.z, d = (uint32_t)res.w;
+    half_swap(a, b);
+    half_swap(c, d);
+    const uint32_t rp[4] = {a, c, b, d};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
+    run_chain<16, SEQ_MAX_STAGES, false>(ep.chain2, val, ep.chain2_flags);
+  }
+  uint32_t a = pack_bytes(val[0], val[1], val[2], val[3]), b = pack_bytes(val[4], val[5], val[6], val[7]),
+           c = pack_bytes(val[8], val[9], val[10], val[11]), d = pack_bytes(val[12], val[13], val[14], val[15]);
+  half_swap(a, c);   // lower half wave: channels 0..15 of the tile, upper: 16..31
+  half_swap(b, d);
+  return v4i{(int)a, (int)c, (int)b, (int)d};
+}
+// The filters and biases of a chain's layers are the same for every wavefront, and a wavefront's pixel block uses each of
+// their bytes once: fetched per wavefront they were most of its memory traffic (and four 16-byte loads per tile for
+// the bias alone).  The workgroup copies them to LDS once per step instead, memory -> LDS without passing registers,
+// requested BEFORE the wait at the layer boundary (they do not depend on the previous layer): filter of A at byte 0 of
+// the block, B's and C's behind it, as they lie in memory; the biases of B and C in `sBias`.
+struct ChainLds {
+  const char* w;      // LDS: A's packed filter; B's at w + off_b, C's at w + off_c
+  unsigned off_b, off_c;
+  const int* bias_b;  // LDS: OC_B words (zeros without a bias), C's OC_C words behind them
+  const int* bias_c;
+};
+__device__ __forceinline__ unsigned filter_bytes(const ConvGeom& g) {
+  return (unsigned)(g.OC >> 5) * (unsigned)((g.Kp >> 5) + 1) * 1024u;
+}
+// all 512 threads; the caller waits (vmcnt(0), barrier) before anyone reads
+__device__ __forceinline__ ChainLds chain_stage_operands(const SeqLayer& A, const SeqLayer& B, const SeqLayer* C, int* sPart, int* sBias,
+                                                         const int tid) {
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const uint32_t lds_w = (uint32_t)(uintptr_t)(lptr_t)reinterpret_cast<int8_t*>(sPart);
+  const uint32_t lds_b = (uint32_t)(uintptr_t)(lptr_t)reinterpret_cast<int8_t*>(sBias);
+  const unsigned sz_a = filter_bytes(A.g), sz_b = filter_bytes(B.g), sz_c = C ? filter_bytes(C->g) : 0u;
+  auto copy = [&](const int8_t* src_generic, const unsigned bytes, const uint32_t dst) __attribute__((always_inline)) {
+    const uintptr_t sb = (uintptr_t)src_generic;
+    const int8_t* src = reinterpret_cast<const int8_t*>(((uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(sb >> 32)) << 32) |
+                                                        (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)sb));
+    const int blocks = __builtin_amdgcn_readfirstlane((int)((bytes + 1023u) >> 10));
+    for (int k = wave; k < blocks; k += 8) {
+      if ((unsigned)k * 1024u + (unsigned)lane * 16u < bytes)
+        lds_dma16(src + (size_t)k * 1024 + lane * 16, (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + (unsigned)k * 1024u)));
+    }
+  };
+  copy(A.wf, sz_a, lds_w);
+  copy(B.wf, sz_b, lds_w + sz_a);
+  if (C) copy(C->wf, sz_c, lds_w + sz_a + sz_b);
+  const int ocb = B.g.OC, occ = C ? C->g.OC : 0;
+  if (B.ep.bias) copy(reinterpret_cast<const int8_t*>(B.ep.bias), (unsigned)ocb * 4u, lds_b);
+  else for (int k = tid; k < ocb; k += 512) sBias[k] = 0;
+  if (C) {
+    if (C->ep.bias) copy(reinterpret_cast<const int8_t*>(C->ep.bias), (unsigned)occ * 4u, lds_b + (unsigned)ocb * 4u);
+    else for (int k = tid; k < occ; k += 512) sBias[ocb + k] = 0;
+  }
+  return ChainLds{reinterpret_cast<const char*>(sPart), sz_a, sz_a + sz_b, sBias, sBias + ocb};
+}
+// the bias of 32 output channels as an accumulator tile holds them
+__device__ __forceinline__ v16i bias_tile(const int* sbias, const int first, const int lgrp) {
+  v16i r;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int4 bv = *reinterpret_cast<const int4*>(sbias + first + q * 8 + lgrp * 4);
+    r[q * 4] = bv.x; r[q * 4 + 1] = bv.y; r[q * 4 + 2] = bv.z; r[q * 4 + 3] = bv.w;
+  }
+  return r;
+}
+// The host has checked (conv_seq_link): A, B and C have whole 32-channel tiles and no padding channels, A has MT2 tiles,
+// C has MT1, B reads A's output and C reads B's, pixel for pixel; only B may have a residual; every bias is 16-byte
+// aligned; the filters fit the LDS block and the biases sBias; no output overlaps anything another wavefront may still
+// read in this layer.
+template <int MT2, int MT1>
+__device__ __forceinline__ void conv_chain_tail(const v16i (&accA)[MT2][1], const Epilogue& epA, void* outA, const SeqLayer& B,
+                                                const SeqLayer* C, const ChainLds& lds, const int px_wave, const int lane,
+                                                const int p_begin, const int p_end) {
+  if (px_wave >= p_end || px_wave + 32 <= p_begin) return;   // none of this wavefront's pixels belong to the share
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const int p = px_wave + lrow;
+  const bool mine = p >= p_begin && p < p_end;               // pixels of a neighbouring share are computed and not stored
+  const unsigned pblk = (unsigned)px_wave >> 5;
+  const unsigned lane16 = (unsigned)lane * 16u;
+
+  v4i b2[MT2];   // A's result: the K chunks of B
+  {
+    const __amdgpu_buffer_rsrc_t rs = act_rsrc(outA);
+#pragma unroll
+    for (int i = 0; i < MT2; ++i) {
+      b2[i] = requant_tile(accA[i][0], epA, zero4());
+      if (mine) st16_buf(rs, (pblk * MT2 + i) * 1024u + lane16, b2[i]);
+    }
+  }
+  const Epilogue& eB = B.ep;
+  const int TB = __builtin_amdgcn_readfirstlane(B.g.OC >> 5);
+  const unsigned strideB = (unsigned)__builtin_amdgcn_readfirstlane((B.g.Kp >> 5) + 1) * 1024u;   // from one 32-channel tile of the packed filter to the next
+  const __amdgpu_buffer_rsrc_t rs_oB = act_rsrc(B.out), rs_res = act_rsrc(eB.residual);
+  const bool has_res = eB.residual != nullptr;
+  const Epilogue& eC = MT1 > 0 ? C->ep : eB;
+  const unsigned strideC = MT1 > 0 ? (unsigned)__builtin_amdgcn_readfirstlane((C->g.Kp >> 5) + 1) * 1024u : 0u;
+  const char* wB = lds.w + lds.off_b + lane16;
+  const char* wC = lds.w + lds.off_c + lane16;
+  constexpr int NC = MT1 > 0 ? MT1 : 1;
+  v16i accC[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) accC[i] = bias_tile(lds.bias_c, MT1 > 0 ? i * 32 : 0, lgrp);
+
+  // the one thing tile t of B still needs from memory, requested a tile ahead: its block of the residual
+  auto request = [&](const int t) __attribute__((always_inline)) -> int4 {
+    return ld16_l2(rs_res, has_res ? (pblk * (unsigned)TB + (unsigned)t) * 1024u + lane16 : kOutsideBuffer);
+  };
+  auto tile = [&](const int4 res, const int t) __attribute__((always_inline)) {
+    v16i a = bias_tile(lds.bias_b, t * 32, lgrp);
+#pragma unroll
+    for (int c = 0; c < MT2; ++c) {
+      const int4 w = *reinterpret_cast<const int4*>(wB + (unsigned)t * strideB + (unsigned)c * 1024u);
+      a = __builtin_amdgcn_mfma_i32_32x32x32_i8(v4i{w.x, w.y, w.z, w.w}, b2[c], a, 0, 0, 0);
+    }
+    const v4i b3 = requant_tile(a, eB, res);
+    if (mine) st16_buf(rs_oB, (pblk * (unsigned)TB + (unsigned)t) * 1024u + lane16, b3);
+    if constexpr (MT1 > 0) {
+#pragma unroll
+      for (int i = 0; i < MT1; ++i) {
+        const int4 w = *reinterpret_cast<const int4*>(wC + (unsigned)i * strideC + (unsigned)t * 1024u);
+        accC[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(v4i{w.x, w.y, w.z, w.w}, b3, accC[i], 0, 0, 0);
+      }
+    }
+  };
+  // one copy of the tile's code (a second one would double what the instruction cache has to fetch): the block
+  // requested ahead changes hands in registers
+  int4 r0 = request(0);
+  for (int t = 0; t < TB; ++t) {
+    const int4 r1 = request(t + 1 < TB ? t + 1 : t);
+    tile(r0, t);
+    r0 = r1;
+  }
+  if constexpr (MT1 > 0) {
+    const __amdgpu_buffer_rsrc_t rs_oC = act_rsrc(C->out);
+#pragma unroll
+    for (int i = 0; i < MT1; ++i) {
+      const v4i y = requant_tile(accC[i], eC, zero4());
+      if (mine) st16_buf(rs_oC, (pblk * MT1 + i) * 1024u + lane16, y);
+    }
+  }
+}
+
+// TAIL >= 0 (layer-sequence kernel, unsplit K, one pixel block per wavefront, all of the layer's channels in the tile): the
+// accumulators go to conv_chain_tail<TM, TAIL> with the table entries tailB, tailC instead of the epilogue.
+template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLICES, bool COH, bool POOLR = false, int TAIL = -1>
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
-                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0, nullptr},
-                                               unsigned long long* tr = nullptr) {
+                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0, nullptr, -1},
+                                               unsigned long long* tr = nullptr, const SeqLayer* tailB = nullptr,
+                                               const SeqLayer* tailC = nullptr, const ChainLds* chain_lds = nullptr) {
   CVM_SEQ_STAMP(0, tid);
   constexpr int PS = NW / KSPLIT;         // wavefronts side by side along the pixel axis
   constexpr int BM = 32 * TM;             // output channels per workgroup
@@ -888,9 +1099,14 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // COH: called once, between the filter requests and the activation requests of the first batch
   auto pass_gate = [&]() __attribute__((always_inline)) {
     if constexpr (COH) {
-      gate_wait(gate, wave);
+      gate_wait(gate, gate.role < 0 ? wave : gate.role);
       CVM_SEQ_STAMP(1, tid);
     }
+  };
+  // a filter chunk of tile row i: from memory, or (a layer with a chain behind it) from the copy of the filter in LDS
+  auto load_w = [&](const int i, const unsigned chunk_bytes) __attribute__((always_inline)) -> int4 {
+    if constexpr (TAIL >= 0) return *reinterpret_cast<const int4*>(chain_lds->w + wa[i] + chunk_bytes);
+    else return ld16_buf<false>(rs_w, wa[i], chunk_bytes);
   };
   auto fetch = [&](const bool gated) __attribute__((always_inline)) -> regs_t {
     regs_t R;
@@ -910,7 +1126,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, ld16_buf<false>(rs_w, wa[i], (unsigned)ca[d] * 1024u));
+        for (int d = 0; d < D; ++d) put(R, (d * (TM + TN) + i) * 4, load_w(i, (unsigned)ca[d] * 1024u));
       if (gated) pass_gate();
 #pragma unroll
       for (int j = 0; j < TN; ++j)
@@ -927,7 +1143,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       // a chunk past the end multiplies the all-zero filter chunk with a valid activation address
       const int chunk = live ? cur : nch;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, ld16_buf<false>(rs_w, wa[i], (unsigned)chunk * 1024u));
+      for (int i = 0; i < TM; ++i) put(R, (d * (TM + TN) + i) * 4, load_w(i, (unsigned)chunk * 1024u));
       if (gated && d == 0) pass_gate();
       if (MODE == WAVE_ROWS) {
         // 16-byte unit k16 of K: filter row k16 / (row_bytes/16), part k16 % (row_bytes/16) of its window
@@ -1035,6 +1251,12 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     }
   }
   CVM_SEQ_STAMP(3, acc[0][0][0]);
+  if constexpr (TAIL >= 0) {
+    static_assert(TAIL < 0 || (KSPLIT == 1 && TN == 1 && COH && OUT == OUT_I8_ACT), "a chain starts from an unsplit tile of one pixel block");
+    conv_chain_tail<TM, TAIL>(acc, ep, out, *tailB, tailC, *chain_lds, px0 + pw_ * 32, lane, p_begin, p_end);
+    CVM_SEQ_STAMP(5, tid);
+    return;
+  }
 
   // ---- partial sums of the KSPLIT wavefronts that share a tile meet in LDS;
   // wavefront kw_ then finalises the groups kw_*NU .. kw_*NU + NU-1 of the tile set
@@ -1101,15 +1323,6 @@ k_conv_wave(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* 
 // s_barrier, request the step NST-1 ahead into the buffer everyone has just left, then 2 x (TM + TN)
 // ds_read_b128 and 2 x TM x TN MFMAs.  The barrier is the bare instruction and the waits are written by
 // hand: the fence that comes with __syncthreads would wait for every outstanding request, i.e. undo the ring.
-// One request: 16 bytes per lane from `gaddr` (any address per lane) to LDS byte lds_base + 16 * lane.  Written as
-// assembly on purpose: the compiler then neither counts these requests nor protects LDS reads against them (it would
-// wait for every outstanding one before the first ds_read of a step, which undoes the ring); the waits are wait_vm.
-__device__ __forceinline__ void lds_dma16(const void* gaddr, uint32_t lds_base) {
-  // (the s_nop is the wait state an instruction that reads M0 needs after a scalar write to it; inside inline assembly
-  // nobody inserts it for us)
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(lds_base) : "memory");
-}
-
 template <int N>
 __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -1185,7 +1398,6 @@ k_conv_big(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* _
     colmask[q] = cm;
   }
   const int8_t* zero = reinterpret_cast<const int8_t*>(g_zero_granule);
-  typedef int8_t __attribute__((address_space(3))) * lptr_t;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)smem;   // LDS byte address of the ring
 
   // ---- the request stream.  Stages are requested in order (the first NST - 1 before the loop, then one per step), so
@@ -1470,21 +1682,6 @@ k_stem_pool(const int8_t* __restrict__ xs, const int8_t* __restrict__ wf, int8_t
 // Every wait is bounded: when a counter does not arrive within spin_limit polls the workgroup raises
 // the error flag, which makes every workgroup leave at its next boundary; the host then falls back to one
 // launch per layer.
-struct SeqLayer {
-  const int8_t* xp;
-  const int8_t* wf;
-  void* out;
-  ConvGeom g;
-  Epilogue ep;
-  int kernel;          // configuration * 3 + mode (identity, no padding, padding)
-  int px_per_share;    // output pixels of one share of the images
-  int ptiles;          // pixel tiles that cover a share (its first block may begin before the share)
-  int shares;          // XCDs that take part: the largest of 1, 2, 4, 8 that divides the batch; the others leave at once
-  int reserved[2];     // keeps the entry a multiple of 16 bytes
-};
-constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
-enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
-
 template <int TM, int TN, int KSPLIT, int NW, int D, int MODE>
 __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                                 int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
@@ -1494,10 +1691,10 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
   const int htid = UNITS == 2 ? (tid & 255) : tid;
   for (int base = 0; base < ntiles; base += SEQ_WG_PER_SHARE * UNITS) {
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
-    conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid,
-                                                                         sPart + half * 16384, sBias + half * 256, p_begin, p_end,
-                                                                         base == 0 ? LayerGate{gate.counter, gate.target, gate.error, gate.spin_limit, gate.seen + half} : LayerGate{nullptr, 0, nullptr, 0, nullptr},
-                                                                         base == 0 ? tr : nullptr);
+    conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(
+        xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid, sPart + half * 16384, sBias + half * 256, p_begin, p_end,
+        base == 0 ? LayerGate{gate.counter, gate.target, gate.error, gate.spin_limit, gate.seen + half, -1} : LayerGate{nullptr, 0, nullptr, 0, nullptr, -1},
+        base == 0 ? tr : nullptr);
     if (KSPLIT > 1) __syncthreads();   // the next tile reuses the LDS of the partial sums
   }
 }
@@ -1517,6 +1714,39 @@ __device__ __forceinline__ void seq_layer_cfg(int cfg, const int8_t* xp, const i
   }
 }
 
+// A layer with a chain behind it: 64 output channels x 32 pixels per wavefront, unsplit.  Every wavefront is a tile of its
+// own, pixel block `wave * 32 + rank` of the share: up to 256 blocks run in one round, spread evenly over the 32
+// workgroups.  Before the tiles the workgroup as a whole requests the chain's filters and biases into LDS, waits at the
+// layer boundary (its first wavefront polls, the others watch its word in LDS) and meets at a barrier when the copies
+// have landed; from there on no wavefront needs another.  mt1: 32-channel tiles of the chain's second layer (0: none).
+template <int MODE, int TAIL>
+__device__ __forceinline__ void seq_chain_tiles(const SeqLayer& A, int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias,
+                                                int p_begin, int p_end, const LayerGate gate, unsigned long long* tr,
+                                                const SeqLayer* tailB, const SeqLayer* tailC) {
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const ChainLds lds = chain_stage_operands(A, *tailB, TAIL > 0 ? tailC : nullptr, sPart, sBias, tid);
+  gate_wait(gate, wave);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const LayerGate none = {nullptr, 0, nullptr, 0, nullptr, -1};
+  for (int base = 0; base < ntiles; base += 8 * SEQ_WG_PER_SHARE) {
+    const int t = base + wave * SEQ_WG_PER_SHARE + rank;
+    if (t >= ntiles) continue;
+    conv_wave_tile<2, 1, 1, 1, 4, OUT_I8_ACT, MODE, false, true, false, TAIL>(
+        A.xp, A.wf, A.out, A.g, A.ep, t, tid & 63, sPart, sBias, p_begin, p_end, none, base == 0 && wave == 0 ? tr : nullptr, tailB, tailC, &lds);
+  }
+}
+template <int MODE>
+__device__ __forceinline__ void seq_layer_chain(int mt1, const SeqLayer& A, int ntiles, int dead_tile, int rank, int tid, int* sPart,
+                                                int* sBias, int p_begin, int p_end, const LayerGate gate, unsigned long long* tr,
+                                                const SeqLayer* tailB, const SeqLayer* tailC) {
+  switch (mt1) {
+    case 0: seq_chain_tiles<MODE, 0>(A, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC); break;
+    case 2: seq_chain_tiles<MODE, 2>(A, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC); break;
+    default: seq_chain_tiles<MODE, 4>(A, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC); break;
+  }
+}
+
 __global__ void __launch_bounds__(512, 1)
 k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* __restrict__ sync, int spin_limit,
            unsigned long long* __restrict__ stamps, int stamp_layers) {
@@ -1524,22 +1754,25 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   __shared__ __attribute__((aligned(16))) int sBias[512];    // per half: one copy, or one per wavefront of an unsplit tile
   __shared__ int s_rank;
   __shared__ unsigned s_seen[2];   // per half of the workgroup: the highest layer boundary its first wavefront has seen reached
-  // The current layer's table entry lives in LDS, where any field is a short read away wherever the code needs
-  // it (a copy in registers would hold ~100 scalar registers for the whole layer, and reading it from memory
-  // would begin every layer with a trip there).  The first wavefront requests the next entry when a layer
-  // begins and stores it to the other LDS slot before the layer boundary.
+  // The table entries of the current layer (and of the one or two chained behind it) live in LDS, where any field is a
+  // short read away wherever the code needs it (a copy in registers would hold ~100 scalar registers for the whole
+  // layer, and reading it from memory would begin every layer with a trip there): a ring of eight slots, entry e in
+  // slot e % 8.  When a step over `cnt` entries begins, entries l .. l + 2 are in the ring; the first wavefront requests
+  // the entries l + 3 .. l + 2 + cnt, which arrive in their slots before the layer boundary.
   constexpr int LWORDS = (int)(sizeof(SeqLayer) / 4);
+  constexpr int RING = 8;
   static_assert(sizeof(SeqLayer) % 16 == 0 && LWORDS <= 128, "a table entry is copied by one wavefront, two words per lane");
-  __shared__ __attribute__((aligned(16))) uint32_t sLayer[2][LWORDS];
-  {
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(layers_generic);
-    if ((int)threadIdx.x < LWORDS) sLayer[0][threadIdx.x] = src[threadIdx.x];
+  __shared__ __attribute__((aligned(16))) uint32_t sLayer[RING][LWORDS];
+  const uint32_t* table_words = reinterpret_cast<const uint32_t*>(layers_generic);
+  for (int w = threadIdx.x; w < 3 * LWORDS; w += 512) {
+    const int e = w / LWORDS;
+    if (e < nlayers) sLayer[e][w - e * LWORDS] = table_words[w];
   }
   const int tid = threadIdx.x;
   unsigned xcc;
   asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
   xcc &= 15u;
-  __syncthreads();   // the first table entry is in LDS
+  __syncthreads();   // the first table entries are in LDS
   // a batch that does not divide over all 8 XCDs runs on the first `shares` of them; a workgroup elsewhere has nothing to do
   if (xcc < SEQ_SHARES && (int)xcc >= reinterpret_cast<const SeqLayer*>(sLayer[0])->shares) return;
   unsigned* my = sync + (xcc < SEQ_SHARES ? xcc : 0) * SEQ_SYNC_WORDS;
@@ -1555,14 +1788,21 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   __syncthreads();
   const int rank = s_rank;
   const bool stop = xcc >= SEQ_SHARES || rank >= SEQ_WG_PER_SHARE;
-  for (int l = 0; l < nlayers && !stop; ++l) {
-    const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer[l & 1]);
-    uint32_t next0 = 0, next1 = 0;
-    const bool fetch_next = tid < 64 && l + 1 < nlayers;
-    if (fetch_next) {
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(layers_generic + l + 1);
-      next0 = src[tid];
-      if (tid + 64 < LWORDS) next1 = src[tid + 64];
+  int step = 0;   // layer boundaries passed: a chain of layers is one step
+  for (int l = 0; l < nlayers && !stop; ++step) {
+    const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer[l & (RING - 1)]);
+    const int chain = __builtin_amdgcn_readfirstlane(L.chain);
+    const int cnt = chain + 1;   // table entries this step consumes (at most 3)
+    // (memory -> LDS without passing through registers: held in registers for the length of a layer, the entries cost
+    // every tile loop of the kernel, all of which use the whole register file, a spill)
+    if (tid < LWORDS / 4) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const int e = l + 3 + k;
+        if (k < cnt && e < nlayers)
+          lds_dma16(table_words + (size_t)e * LWORDS + tid * 4,
+                    (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lptr_t)&sLayer[e & (RING - 1)][0]));
+      }
     }
     const ConvGeom& g = L.g;
     const Epilogue& ep = L.ep;
@@ -1575,18 +1815,25 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int ntiles = g.octiles * L.ptiles;
     const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
-    // layer l may read what layer l - 1 wrote once all 32 workgroups of the XCD have counted themselves out of it
-    const LayerGate gate = {l > 0 ? my + SEQ_BAR : nullptr, (unsigned)l * SEQ_WG_PER_SHARE, error, spin_limit, s_seen};
+    // this step may read what the previous one wrote once all 32 workgroups of the XCD have counted themselves out of it
+    const LayerGate gate = {step > 0 ? my + SEQ_BAR : nullptr, (unsigned)step * SEQ_WG_PER_SHARE, error, spin_limit, s_seen, -1};
 #ifdef CVM_SEQ_STAMPS
     unsigned long long* tr = stamps && l < stamp_layers ? stamps + ((size_t)((int)xcc * SEQ_WG_PER_SHARE + rank) * stamp_layers + l) * 8 : nullptr;
     if (tr && tid == 0) tr[7] = __builtin_amdgcn_s_memtime();
 #else
     unsigned long long* tr = nullptr;
 #endif
-    if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
+    if (chain > 0) {
+      const SeqLayer* tailB = reinterpret_cast<const SeqLayer*>(sLayer[(l + 1) & (RING - 1)]);
+      const SeqLayer* tailC = reinterpret_cast<const SeqLayer*>(sLayer[(l + 2) & (RING - 1)]);
+      const int mt1 = chain > 1 ? __builtin_amdgcn_readfirstlane(tailC->g.OC) >> 5 : 0;
+      if (mode == 0) seq_layer_chain<WAVE_IDENT>(mt1, L, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC);
+      else if (mode == 1) seq_layer_chain<WAVE_NOPAD>(mt1, L, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC);
+      else seq_layer_chain<WAVE_PAD>(mt1, L, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr, tailB, tailC);
+    } else if (mode == 0) seq_layer_cfg<WAVE_IDENT>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
     else if (mode == 1) seq_layer_cfg<WAVE_NOPAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
     else seq_layer_cfg<WAVE_PAD>(cfg, xp, wf, out, g, ep, ntiles, dead_tile, rank, tid, sPart, sBias, p_begin, p_end, gate, tr);
-    if (l + 1 == nlayers) {
+    if (l + cnt >= nlayers) {
 #ifdef CVM_SEQ_STAMPS
       if (tr) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1596,17 +1843,15 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
 #endif
       break;
     }
-    if (fetch_next) {
-      sLayer[(l + 1) & 1][tid] = next0;
-      if (tid + 64 < LWORDS) sLayer[(l + 1) & 1][tid + 64] = next1;
-    }
-    // ---- this workgroup is done with the layer: every store of its wavefronts is in the L2, then it counts itself out
+    // ---- this workgroup is done with the step: every store of its wavefronts is in the L2 (and the table entries requested
+    // at its start are in LDS), then it counts itself out
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #ifdef CVM_SEQ_STAMPS
     if (tr && tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
 #endif
+    l += cnt;
   }
   // the last workgroup of a share to finish clears the share's counters for the next launch
   __syncthreads();
@@ -1923,7 +2168,7 @@ k_dense_i32(const int32_t* __restrict__ x, const int32_t* __restrict__ w, const 
 // ---------------------------------------------------------------- host side
 // Kernel choice forced by the calling thread (tests and tuning runs); automatic unless set.
 static ConvTuning default_tuning() {
-  ConvTuning t = {CONV_KERNEL_AUTO, -1, 0, 0, 2000000, nullptr, 0, {}};
+  ConvTuning t = {CONV_KERNEL_AUTO, -1, 0, 0, 2000000, nullptr, 0, {}, 1};
   memset(t.seq_layer_cfg, -1, sizeof(t.seq_layer_cfg));
   return t;
 }
@@ -2324,6 +2569,8 @@ static int conv_prepare(const int8_t* xp, const int8_t* wp, void* out, ConvGeom&
     return arg_error("conv tensor too large");
   ep = ep_in;
   ep.bias_vec = ep.bias != nullptr && ((uintptr_t)ep.bias & 15) == 0;
+  ep.chain_flags = chain_flags_of(ep.chain);
+  ep.chain2_flags = chain_flags_of(ep.chain2);
   if (ep.o32_img == 0 && ep.o32_ch == 0 && ep.o32_px == 0) {  // int32 output defaults to NCHW
     ep.o32_img = (int64_t)g.OC * g.OH * g.OW;
     ep.o32_ch = g.OH * g.OW;
@@ -2585,6 +2832,12 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
     return arg_error("conv_seq_layer: not eligible (few-channel input, depthwise or int32 output)");
   // results are stored through a buffer descriptor with 32-bit offsets
   if (act_bytes(g.P, ep.out_cp) > INT32_MAX) return arg_error("conv_seq_layer: not eligible (output tensor of 2 GiB or more)");
+  // the sequence kernel carries code for short chains without multiplications only
+  for (const DevChain* c : {&ep.chain, &ep.chain2}) {
+    if (c->count > SEQ_MAX_STAGES) return arg_error("conv_seq_layer: not eligible (a requantisation chain of more than two stages)");
+    for (int t = 0; t < c->count; ++t)
+      if (c->st[t].mul != 1) return arg_error("conv_seq_layer: not eligible (a requantisation chain that multiplies)");
+  }
   const ConvTuning tune = t_conv_tuning;
   // a layer that fills the chip several times over is faster as a launch of the large-tile kernel than as a layer of a
   // sequence (whose tile is the wavefront kernel's); a run of layers ends there
@@ -2630,6 +2883,80 @@ int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, v
 
 int conv_seq_layer_config(const void* table, int index) {
   return reinterpret_cast<const SeqLayer*>(table)[index].kernel / 3;
+}
+
+int conv_seq_layer_chain(const void* table, int index) {
+  return reinterpret_cast<const SeqLayer*>(table)[index].chain;
+}
+
+// ---- chains: 1x1 layers computed by the wavefront that holds their input (conv_chain_tail)
+static bool ranges_overlap(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes) {
+  const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+  return a0 < b0 + (uintptr_t)b_bytes && b0 < a0 + (uintptr_t)a_bytes;
+}
+// Layer `f` of the table can follow layer `prev` inside a chain that began with layer `a`: a 1x1 convolution with stride
+// 1 and no padding over prev's output, pixel for pixel, whole 32-channel tiles on both sides.
+static bool chain_follower(const SeqLayer& a, const SeqLayer& prev, const SeqLayer& f) {
+  if (f.kernel % 3 != 0 || f.xp != prev.out || f.g.P != a.g.P || f.shares != a.shares || f.px_per_share != a.px_per_share) return false;
+  if (f.g.Cp != prev.g.OC || prev.ep.out_cp != prev.g.OC || (f.g.OC & 31) != 0 || f.ep.out_cp != f.g.OC) return false;
+  if (f.g.Kp != ((f.g.Cp + 63) & ~63)) return false;   // the filter's chunks are the input's 32-channel tiles
+  if (f.ep.bias && !f.ep.bias_vec) return false;
+  return true;
+}
+static int chain_followers(const SeqLayer* L, int i, int count) {
+  const SeqLayer& a = L[i];
+  if (i + 1 >= count || a.g.OC != 64 || a.ep.out_cp != 64 || a.ep.residual || a.g.octiles < 1) return 0;
+  const SeqLayer& b = L[i + 1];
+  if (!chain_follower(a, a, b)) return 0;
+  const int64_t a_in = act_bytes((int64_t)a.g.N * a.g.H * a.g.W, a.g.Cp), a_out = act_bytes(a.g.P, 64), b_out = act_bytes(a.g.P, b.g.OC);
+  // While one wavefront stores its pixels of A, B and C, others still read A's input around theirs, and B's residual at
+  // theirs: no output may lie over either, nor over another output.  (The residual itself may be B's output tensor:
+  // a block of it is read and written by the same wavefront, in that order.)
+  if (ranges_overlap(a.out, a_out, a.xp, a_in) || ranges_overlap(b.out, b_out, a.xp, a_in) || ranges_overlap(a.out, a_out, b.out, b_out)) return 0;
+  if (b.ep.residual) {
+    if (b.ep.residual != b.out && ranges_overlap(b.out, b_out, b.ep.residual, b_out)) return 0;
+    if (ranges_overlap(a.out, a_out, b.ep.residual, b_out)) return 0;
+  }
+  // the filters are copied to the workgroup's 128 KiB LDS block and the biases to 512 words beside it
+  auto filter = [](const SeqLayer& l) { return (int64_t)(l.g.OC / 32) * (l.g.Kp / 32 + 1) * 1024; };
+  if (filter(a) + filter(b) > 131072 || b.g.OC > 512) return 0;
+  if (i + 2 >= count) return 1;
+  const SeqLayer& c = L[i + 2];
+  if (filter(a) + filter(b) + filter(c) > 131072 || b.g.OC + c.g.OC > 512) return 1;
+  if (!chain_follower(a, b, c) || c.ep.residual || (c.g.OC != 64 && c.g.OC != 128)) return 1;
+  const int64_t c_out = act_bytes(a.g.P, c.g.OC);
+  if (ranges_overlap(c.out, c_out, a.xp, a_in) || ranges_overlap(c.out, c_out, a.out, a_out) || ranges_overlap(c.out, c_out, b.out, b_out)) return 1;
+  if (b.ep.residual && ranges_overlap(c.out, c_out, b.ep.residual, b_out)) return 1;
+  return 2;
+}
+// Links the chains of a finished table of `count` entries (after every conv_seq_layer call, before it is copied to the
+// device); returns how many it found.  A layer whose configuration was forced is left as it is.
+int conv_seq_link(void* table, int count) {
+  const ConvTuning tune = t_conv_tuning;
+  if (!tune.seq_chains || tune.wave_cfg >= 0 || tune.kernel != CONV_KERNEL_AUTO) return 0;
+  SeqLayer* L = reinterpret_cast<SeqLayer*>(table);
+  int linked = 0;
+  for (int i = 0; i + 1 < count;) {
+    int n = chain_followers(L, i, count);
+    for (int k = 0; k <= n; ++k)
+      if (i + k < 64 && tune.seq_layer_cfg[i + k] >= 0) n = 0;
+    if (n == 0) { ++i; continue; }
+    SeqLayer& a = L[i];
+    a.chain = n;
+    a.kernel = 7 * 3 + a.kernel % 3;
+    a.g.octiles = 1;
+    a.g.div_octiles = make_fastdiv(1u);
+    int ptiles = 0;
+    for (int x = 0; x < a.shares; ++x) {
+      const int lead = (x * a.px_per_share) & 31;
+      const int t = (lead + a.px_per_share + 31) / 32;   // a pixel block per wavefront
+      ptiles = t > ptiles ? t : ptiles;
+    }
+    a.ptiles = ptiles;
+    ++linked;
+    i += n + 1;
+  }
+  return linked;
 }
 
 int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s) {
@@ -2683,6 +3010,13 @@ int cvmhip_set_seq_tuning(int spin_limit) {
   if (spin_limit < 0) return arg_error("set_seq_tuning");
   ConvTuning t = t_conv_tuning;
   t.seq_spin_limit = spin_limit;
+  set_conv_tuning(t);
+  return CVMHIP_OK;
+}
+
+int cvmhip_set_seq_chains(int on) {
+  ConvTuning t = t_conv_tuning;
+  t.seq_chains = on != 0;
   set_conv_tuning(t);
   return CVMHIP_OK;
 }

@@ -376,6 +376,16 @@ int cvmhip_conv_seq_layer_config(const void* table, int index) {
   return conv_seq_layer_config(table, index);
 }
 
+int cvmhip_conv_seq_layer_chain(const void* table, int index) {
+  if (!table || index < 0) return 0;
+  return conv_seq_layer_chain(table, index);
+}
+
+int cvmhip_conv_seq_link(void* table, int count) {
+  if (!table || count < 1) return 0;
+  return conv_seq_link(table, count);
+}
+
 int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream) {
   return conv_seq_launch(dev_table, nlayers, sync, ops, bytes, as_stream(stream));
 }

@@ -756,6 +756,7 @@ void HipGraphRuntime::BuildSequences() {
     }
     const size_t count = j - i;
     if (count >= 3) {
+      cvmhip_conv_seq_link(table.data(), static_cast<int>(count));
       auto buf = std::make_shared<DeviceBuffer>();
       Check(cvmhip_alloc(&buf->ptr, count * entry), "layer-sequence table");
       Check(cvmhip_copy_h2d(buf->ptr, table.data(), count * entry, stream_), "layer-sequence table");

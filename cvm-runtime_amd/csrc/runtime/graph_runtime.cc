@@ -450,6 +450,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.graph = env("CVM_HIP_GRAPH") != "0";
   hooks_.seq = env("CVM_HIP_SEQ") != "0";
   hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";
+  hooks_.seq_chains = env("CVM_HIP_SEQ_CHAIN") != "0";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   hooks_.pool_fuse = env("CVM_HIP_POOLFUSE") != "0";
   hooks_.head_pair = env("CVM_HIP_HEADPAIR") != "0";
@@ -481,6 +482,7 @@ void HipGraphRuntime::ReadHooks() {
 void HipGraphRuntime::ApplyTuning() {
   HipCheck(cvmhip_set_conv_tuning(hooks_.conv_kernel, hooks_.wave_cfg, hooks_.tile_wm, hooks_.tile_wn), "conv tuning");
   HipCheck(cvmhip_set_seq_tuning(hooks_.seq_spin), "sequence tuning");
+  HipCheck(cvmhip_set_seq_chains(hooks_.seq_chains ? 1 : 0), "sequence tuning");
   HipCheck(cvmhip_set_seq_layer_config(-1, -1), "sequence tuning");
   for (const auto& kv : hooks_.seq_layer_cfg) HipCheck(cvmhip_set_seq_layer_config(kv.first, kv.second), "sequence tuning");
 }

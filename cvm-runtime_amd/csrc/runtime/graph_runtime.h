@@ -231,6 +231,7 @@ class HipGraphRuntime {
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
     // layer-sequence launches: CVM_HIP_SEQ_SPIN=<polls> patience of a wait at a layer boundary (0: every wait gives up at once)
     int seq_spin = 2000000;
+    bool seq_chains = true;   // CVM_HIP_SEQ_CHAIN=0: no 1x1 layers chained behind the layer that feeds them (cvmhip_conv_seq_link)
     std::vector<std::pair<int, int>> seq_layer_cfg;   // CVM_HIP_SEQCFG: (layer of a sequence, configuration)
   };
   void ApplyTuning();   // hands the hooks to the kernels' per-thread tuning record

@@ -342,8 +342,23 @@ int cvmhip_conv_seq_layer(void* table, int index, const void* xp, const void* wp
                           const void* residual, const cvmhip_chain* chain2, void* out,
                           int n, int ic, int h, int wd, int oc, int kh, int kw,
                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w);
-/* configuration of the tile kernel that cvmhip_conv_seq_layer chose for entry `index` of a host table */
+/* configuration of the tile kernel that cvmhip_conv_seq_layer chose for entry `index` of a host table (7: the entry
+ * begins a chain, see cvmhip_conv_seq_link) */
 int cvmhip_conv_seq_layer_config(const void* table, int index);
+/* Optional, on a finished host table of `count` entries, before it is copied to the device.  A 1x1 convolution with
+ * stride 1 and no padding (conv2d: ops.cc:368-456) needs, for a block of 32 pixels, only the same 32 pixels of its
+ * input.  Where an entry with 64 output channels is followed by one or two such layers, each reading the one before it
+ * (the 3x3 -> 1x1 (+ residual) -> 1x1 run of a ResNet bottleneck), the wavefront that holds the first layer's result
+ * for a pixel block computes the followers there and then, from registers: one layer boundary instead of three, and
+ * the intermediate tensors are written (other layers may read them) but never read back.  Linked only when no output
+ * of the three lies over anything the run still reads (the first layer's input, the residual) and all channel
+ * counts are multiples of 32; results are bit for bit those of the unlinked table.  Returns the number of chains.
+ * cvmhip_set_seq_chains(0) switches linking off for the calling thread (on by default); a forced tile configuration
+ * (cvmhip_set_conv_tuning, cvmhip_set_seq_layer_config) leaves the layers concerned unlinked. */
+int cvmhip_conv_seq_link(void* table, int count);
+int cvmhip_set_seq_chains(int on);
+/* entries chained behind entry `index` of a host table (0, 1 or 2) */
+int cvmhip_conv_seq_layer_chain(const void* table, int index);
 /* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
 int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream);
 /* The same convolution with its int32 result written pixel-major (NHWC): image n's OH*OW*OC values

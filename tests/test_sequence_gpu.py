@@ -54,8 +54,10 @@ def _chain(cid, n, c, hw, layers):
     g = graphgen.GraphBuilder(cid)
     x = g.var("data", (n, c, hw, hw), 8)
     kept = [g.conv_relu_q(x, layers[0][0], 3, 1, 1)]          # the few-channel input layer stays outside the sequence
-    for oc, k, st, relu, res in layers[1:]:
-        y = g.conv_relu_q(kept[-1], oc, k, st, k // 2, relu=relu)
+    for layer in layers[1:]:
+        oc, k, st, relu, res = layer[:5]
+        pad = layer[5] if len(layer) > 5 else k // 2
+        y = g.conv_relu_q(kept[-1], oc, k, st, pad, relu=relu)
         if res is not None and g.shape(kept[res]) == g.shape(y):
             y = g.rshift(g.relu(g.add(y, kept[res])), 1)
         kept.append(y)
@@ -87,6 +89,68 @@ CHAINS = {
     "b12_four_xcds": (12, 3, 8, [(64, 0, 0, 0, None), (64, 1, 1, True, None), (64, 3, 1, True, None), (256, 1, 1, False, None),
                                  (64, 1, 1, True, None)]),
 }
+
+
+# Runs in which a layer with 64 output channels is followed by one or two 1x1 layers over the same pixels: the wavefront
+# that holds the first layer's result computes the followers from registers (cvmhip_conv_seq_link).  (name: expected
+# positions, among the sequence's layers, of the heads of chains -- the few-channel input layer is not part of the sequence)
+LINKED = {
+    # 3x3 (padding) -> 1x1 with residual -> 1x1 back to 64, twice; the second chain has no third layer of 64 or 128 channels
+    "b8_bottlenecks": (8, 3, 14, [(64, 0, 0, 0, None), (256, 1, 1, False, None), (64, 1, 1, True, None), (64, 3, 1, True, None),
+                                  (256, 1, 1, False, 1), (64, 1, 1, True, None), (64, 3, 1, True, None), (256, 1, 1, False, 4),
+                                  (96, 1, 1, True, None)], {2: 7, 5: 7}),
+    # the third layer has 128 channels; 7x7 maps at batch 16: shares of 98 pixels that begin inside a pixel block
+    "b16_third_layer_128_ragged_shares": (16, 3, 7, [(64, 0, 0, 0, None), (256, 1, 1, True, None), (64, 1, 1, True, None),
+                                                     (64, 3, 1, True, None), (256, 1, 1, False, 1), (128, 1, 1, True, None),
+                                                     (64, 1, 1, True, None)], {2: 7}),
+    # the head is a 3x3 layer without padding and stride 2, then one with 1x1 (identity addressing); 384 and 32 channels behind
+    "b8_heads_without_padding": (8, 3, 21, [(64, 0, 0, 0, None), (64, 3, 2, True, None, 0), (384, 1, 1, True, None), (64, 1, 1, True, None),
+                                            (64, 1, 1, True, None), (128, 1, 1, False, None), (32, 1, 1, True, None), (64, 3, 1, True, None)],
+                                 {0: 7, 3: 7}),
+    # batches on one and on four XCDs
+    "b3_one_xcd": (3, 3, 10, [(64, 0, 0, 0, None), (64, 3, 1, True, None), (256, 1, 1, True, None), (64, 1, 1, False, None),
+                              (64, 3, 1, True, None)], {0: 7}),
+    "b12_four_xcds": (12, 3, 9, [(32, 0, 0, 0, None), (64, 1, 1, True, None), (512, 1, 1, True, None), (128, 1, 1, True, None),
+                                 (128, 3, 1, True, None)], {0: 7}),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LINKED))
+def test_1x1_layers_chained_behind_the_layer_that_feeds_them(name, dev):
+    """The chains are found where expected (and nowhere with CVM_HIP_SEQ_CHAIN=0), and the model's output is the one of
+    one launch per layer and of the oracle either way."""
+    n, c, hw, layers, heads_at = LINKED[name]
+    cid = "seq-link-" + name
+    g, heads = _chain(cid, n, c, hw, layers)
+    js, pb = g.build(heads)
+    x = synth.tensor(cid, "data", g.shape((0, 0)), -127, 127).astype(np.int8)
+    os.environ["CVM_HIP_SEQ"] = "1"
+    try:
+        m = runtime.HipModel(js, pb)
+        linked = m.sequence_configs()
+        m.close()
+        os.environ["CVM_HIP_SEQ_CHAIN"] = "0"
+        m = runtime.HipModel(js, pb)
+        plain = m.sequence_configs()
+        m.close()
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+        os.environ.pop("CVM_HIP_SEQ_CHAIN", None)
+    assert 7 not in plain, plain
+    assert [i for i, cfg in enumerate(linked) if cfg == 7] == sorted(heads_at), (linked, plain)
+    with_chains = _run(js, pb, x, "1")
+    os.environ["CVM_HIP_SEQ_CHAIN"] = "0"
+    try:
+        without_chains = _run(js, pb, x, "1")
+    finally:
+        os.environ.pop("CVM_HIP_SEQ_CHAIN", None)
+    one_by_one = _run(js, pb, x, "0")
+    assert np.array_equal(with_chains, one_by_one), "%d of %d values differ from one launch per layer" % (
+        int((with_chains != one_by_one).sum()), one_by_one.size)
+    assert np.array_equal(without_chains, one_by_one)
+    ref = og.run_graph(js, graphgen.load_params(pb), x.astype(np.int32))
+    want = np.concatenate([r.ravel() for r in ref])
+    assert np.array_equal(with_chains, want), "%d of %d values differ from the oracle" % (int((with_chains != want).sum()), want.size)
 
 
 @pytest.mark.parametrize("name", sorted(CHAINS))
