@@ -260,7 +260,7 @@ size_t conv_seq_sync_bytes();
 int conv_seq_shares();
 int conv_seq_layer(void* table, int index, const int8_t* xp, const int8_t* wp, void* out, ConvGeom g, const Epilogue& ep);
 int conv_seq_layer_config(const void* table, int index);   // configuration of the tile kernel chosen for an entry
-int conv_seq_layer_chain(const void* table, int index);    // entries chained behind this one (0, 1 or 2)
+int conv_seq_layer_chain(const void* table, int index);    // entries chained behind this one (0, 1 or 2), + 16: no boundary behind it
 int conv_seq_link(void* table, int count);                 // chains 1x1 layers behind the layer that feeds them; returns the chains found
 int conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, hipStream_t s);
 

@@ -683,6 +683,8 @@ struct alignas(16) SeqLayer {
   int shares;          // XCDs that take part: the largest of 1, 2, 4, 8 that divides the batch; the others leave at once
   int chain;           // 1 or 2: the next one or two entries are 1x1 layers over this layer's output pixels, computed by the
                        // same wavefront from registers (conv_chain_tail); they are then not layers of their own
+  int join_next;       // 1: the layer behind this one (and its chain) reads nothing that this one writes and writes nothing
+                       // that this one touches: no layer boundary between the two
 };
 constexpr int SEQ_SHARES = 8, SEQ_WG_PER_SHARE = 32, SEQ_SYNC_WORDS = 64;   // counters of a share: one 256-byte line
 enum { SEQ_ARRIVE = 0, SEQ_BAR = 1, SEQ_DONE = 2 };
@@ -1788,8 +1790,9 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
   __syncthreads();
   const int rank = s_rank;
   const bool stop = xcc >= SEQ_SHARES || rank >= SEQ_WG_PER_SHARE;
-  int step = 0;   // layer boundaries passed: a chain of layers is one step
-  for (int l = 0; l < nlayers && !stop; ++step) {
+  int step = 0;          // layer boundaries passed: a chain of layers is one step, and so are two layers joined without a boundary
+  bool joined = false;   // no boundary behind the previous layer: this one does not wait
+  for (int l = 0; l < nlayers && !stop;) {
     const SeqLayer& L = *reinterpret_cast<const SeqLayer*>(sLayer[l & (RING - 1)]);
     const int chain = __builtin_amdgcn_readfirstlane(L.chain);
     const int cnt = chain + 1;   // table entries this step consumes (at most 3)
@@ -1816,7 +1819,7 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
     // this step may read what the previous one wrote once all 32 workgroups of the XCD have counted themselves out of it
-    const LayerGate gate = {step > 0 ? my + SEQ_BAR : nullptr, (unsigned)step * SEQ_WG_PER_SHARE, error, spin_limit, s_seen, -1};
+    const LayerGate gate = {step > 0 && !joined ? my + SEQ_BAR : nullptr, (unsigned)step * SEQ_WG_PER_SHARE, error, spin_limit, s_seen, -1};
 #ifdef CVM_SEQ_STAMPS
     unsigned long long* tr = stamps && l < stamp_layers ? stamps + ((size_t)((int)xcc * SEQ_WG_PER_SHARE + rank) * stamp_layers + l) * 8 : nullptr;
     if (tr && tid == 0) tr[7] = __builtin_amdgcn_s_memtime();
@@ -1843,11 +1846,19 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
 #endif
       break;
     }
-    // ---- this workgroup is done with the step: every store of its wavefronts is in the L2 (and the table entries requested
-    // at its start are in LDS), then it counts itself out
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    joined = __builtin_amdgcn_readfirstlane(L.join_next) != 0;
+    if (joined) {
+      // no boundary: only the table entries requested at the layer's start must be in LDS before anyone looks for them
+      if (tid < 64) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    } else {
+      // ---- this workgroup is done with the step: every store of its wavefronts is in the L2 (and the table entries
+      // requested at its start are in LDS), then it counts itself out
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) __hip_atomic_fetch_add(my + SEQ_BAR, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ++step;
+    }
 #ifdef CVM_SEQ_STAMPS
     if (tr && tid == 0) tr[6] = __builtin_amdgcn_s_memtime();
 #endif
@@ -2886,7 +2897,8 @@ int conv_seq_layer_config(const void* table, int index) {
 }
 
 int conv_seq_layer_chain(const void* table, int index) {
-  return reinterpret_cast<const SeqLayer*>(table)[index].chain;
+  const SeqLayer& l = reinterpret_cast<const SeqLayer*>(table)[index];
+  return l.chain + 16 * l.join_next;
 }
 
 // ---- chains: 1x1 layers computed by the wavefront that holds their input (conv_chain_tail)
@@ -2929,6 +2941,32 @@ static int chain_followers(const SeqLayer* L, int i, int count) {
   if (b.ep.residual && ranges_overlap(c.out, c_out, b.ep.residual, b_out)) return 1;
   return 2;
 }
+// What a layer (with the chain behind it, n followers) reads and writes, as address ranges.
+struct Footprint {
+  const void* r[2]; int64_t rb[2]; int nr;
+  const void* w[3]; int64_t wb[3]; int nw;
+};
+static Footprint footprint(const SeqLayer* L, int i) {
+  Footprint f{};
+  const SeqLayer& a = L[i];
+  f.r[f.nr] = a.xp; f.rb[f.nr++] = act_bytes((int64_t)a.g.N * a.g.H * a.g.W, a.g.Cp);
+  for (int k = 0; k <= a.chain; ++k) {
+    const SeqLayer& l = L[i + k];
+    f.w[f.nw] = l.out; f.wb[f.nw++] = act_bytes(l.g.P, l.ep.out_cp);
+    if (l.ep.residual && f.nr < 2) { f.r[f.nr] = l.ep.residual; f.rb[f.nr++] = act_bytes(l.g.P, l.ep.out_cp); }
+  }
+  return f;
+}
+static bool independent(const Footprint& p, const Footprint& q) {
+  for (int i = 0; i < p.nw; ++i) {
+    for (int j = 0; j < q.nr; ++j) if (ranges_overlap(p.w[i], p.wb[i], q.r[j], q.rb[j])) return false;
+    for (int j = 0; j < q.nw; ++j) if (ranges_overlap(p.w[i], p.wb[i], q.w[j], q.wb[j])) return false;
+  }
+  for (int i = 0; i < q.nw; ++i)
+    for (int j = 0; j < p.nr; ++j) if (ranges_overlap(q.w[i], q.wb[i], p.r[j], p.rb[j])) return false;
+  return true;
+}
+
 // Links the chains of a finished table of `count` entries (after every conv_seq_layer call, before it is copied to the
 // device); returns how many it found.  A layer whose configuration was forced is left as it is.
 int conv_seq_link(void* table, int count) {
@@ -2955,6 +2993,19 @@ int conv_seq_link(void* table, int count) {
     a.ptiles = ptiles;
     ++linked;
     i += n + 1;
+  }
+  // Two layers in a row of which the second neither reads what the first writes nor writes what the first touches (the
+  // first 1x1 layer and the shortcut projection of a ResNet block) need no boundary between them: a workgroup that is
+  // through with the first goes on to the second.  Pairs only -- a third layer would have to be independent of both.
+  for (int i = 0; i < count;) {
+    const int j = i + 1 + L[i].chain;
+    if (j < count && L[i].chain == 0 && L[i].shares == L[j].shares && independent(footprint(L, i), footprint(L, j))) {
+      L[i].join_next = 1;
+      ++linked;
+      i = j + 1 + L[j].chain;
+    } else {
+      i = j;
+    }
   }
   return linked;
 }

@@ -352,12 +352,15 @@ int cvmhip_conv_seq_layer_config(const void* table, int index);
  * for a pixel block computes the followers there and then, from registers: one layer boundary instead of three, and
  * the intermediate tensors are written (other layers may read them) but never read back.  Linked only when no output
  * of the three lies over anything the run still reads (the first layer's input, the residual) and all channel
- * counts are multiples of 32; results are bit for bit those of the unlinked table.  Returns the number of chains.
+ * counts are multiples of 32; results are bit for bit those of the unlinked table.  The call also marks pairs of
+ * consecutive layers that have nothing to do with one another (the second reads nothing the first writes and writes
+ * nothing the first reads or writes: the first 1x1 layer and the shortcut projection of a ResNet block): no layer
+ * boundary is kept between the two.  Returns the number of chains and pairs.
  * cvmhip_set_seq_chains(0) switches linking off for the calling thread (on by default); a forced tile configuration
  * (cvmhip_set_conv_tuning, cvmhip_set_seq_layer_config) leaves the layers concerned unlinked. */
 int cvmhip_conv_seq_link(void* table, int count);
 int cvmhip_set_seq_chains(int on);
-/* entries chained behind entry `index` of a host table (0, 1 or 2) */
+/* entries chained behind entry `index` of a host table (0, 1 or 2), plus 16 when no boundary follows the entry */
 int cvmhip_conv_seq_layer_chain(const void* table, int index);
 /* ops, bytes: algorithmic operations and HBM bytes of the layers, only reported by the kernel-timing session */
 int cvmhip_conv_seq_launch(const void* dev_table, int nlayers, void* sync, double ops, double bytes, void* stream);

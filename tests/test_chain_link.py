@@ -80,7 +80,7 @@ def test_an_output_over_something_the_layer_still_reads_breaks_the_chain(lib, ca
 def test_what_cannot_follow(lib):
     # the follower reads another tensor; has a stride; is a 3x3; the head has 128 channels; a third layer of 256 channels
     for layers, want, hw in [
-        ([(Y1, Y2, 0, 64, 64, 3, 1, 1), (X, XO, 0, 64, 256, 1, 1, 0)], [0, 0], 56),
+        ([(Y1, Y2, 0, 64, 64, 3, 1, 1), (X, XO, 0, 64, 256, 1, 1, 0)], [16, 0], 56),   # (no chain, but no boundary either: see below)
         ([(Y1, Y2, 0, 64, 64, 3, 1, 1), (Y2, XO, 0, 64, 256, 1, 2, 0)], [0, 0], 56),
         ([(Y1, Y2, 0, 64, 64, 3, 1, 1), (Y2, XO, 0, 64, 64, 3, 1, 1)], [0, 0], 56),
         ([(Y1, Y2, 0, 128, 128, 3, 1, 1), (Y2, XO, 0, 128, 512, 1, 1, 0)], [0, 0], 14),
@@ -90,6 +90,27 @@ def test_what_cannot_follow(lib):
         buf, n = _table(lib, layers, hw=hw)
         lib.cvmhip_conv_seq_link(buf, n)
         assert _chains(lib, buf, n) == want, layers
+
+
+def test_layers_that_have_nothing_to_do_with_one_another_share_a_step(lib):
+    """The first 1x1 layer and the shortcut projection of a ResNet block both read the block's input: no boundary between
+    them (16 = no boundary behind the entry).  The 3x3 layer behind them reads the first one's output and waits."""
+    buf, n = _table(lib, [(X, Y1, 0, 64, 64, 1, 1, 0), (X, XO, 0, 64, 256, 1, 1, 0), (Y1, Y2, 0, 64, 64, 3, 1, 1)])
+    assert lib.cvmhip_conv_seq_link(buf, n) == 1
+    assert _chains(lib, buf, n) == [16, 0, 0]
+    # the second layer writes over the first one's input, or over its output: a boundary stays
+    for second in [(Y2, X, 0, 64, 64, 1, 1, 0), (Y2, Y1, 0, 64, 64, 1, 1, 0), (Y2, Y1O, X + 4096, 64, 64, 1, 1, 0)]:
+        buf, n = _table(lib, [(X, Y1, 0, 64, 64, 1, 1, 0), second])
+        lib.cvmhip_conv_seq_link(buf, n)
+        assert _chains(lib, buf, n) == ([0, 0] if second[1] != Y1O else [16, 0]), second
+    # ... or reads, as residual, what the first one writes
+    buf, n = _table(lib, [(X, Y1, 0, 64, 64, 1, 1, 0), (Y2, Y1O, Y1, 64, 64, 1, 1, 0)])
+    lib.cvmhip_conv_seq_link(buf, n)
+    assert _chains(lib, buf, n) == [0, 0]
+    # a chain may be the second of the two
+    buf, n = _table(lib, [(X, XO, 0, 64, 256, 1, 1, 0), (Y1, Y2, 0, 64, 64, 3, 1, 1), (Y2, Y1O, 0, 64, 128, 1, 1, 0)])
+    assert lib.cvmhip_conv_seq_link(buf, n) == 2
+    assert _chains(lib, buf, n) == [16, 1, 0]
 
 
 def test_filters_must_fit_the_workgroups_lds(lib):
