@@ -248,6 +248,22 @@ k_pack_depthwise(const int32_t* __restrict__ w, int8_t* __restrict__ wp, int64_t
   }
 }
 
+// int8 act tensor of n images x hw pixels x cp channels (cp % 32 == 0) -> int8 act tensor of n "pixels" (one per image)
+// x hw * cp channels, channel p * cp + c of image i = channel c of the image's pixel p.  One 16-byte granule (16
+// channels of one pixel) per thread; rows n .. 31 of the destination's pixel block are not written.
+__global__ void __launch_bounds__(256)
+k_flatten_act(const int8_t* __restrict__ xp, int8_t* __restrict__ yp, unsigned granules, unsigned n, unsigned hw, unsigned cp) {
+  const unsigned gpp = cp >> 4;   // granules per pixel
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;   // (32-bit arithmetic throughout: the host bounds the sizes)
+  if (i >= granules) return;
+  const unsigned kg = i / n;             // granule of the flattened channel axis
+  const unsigned img = i - kg * n;       // consecutive threads: the rows of one destination block half
+  const unsigned p = kg / gpp;
+  const unsigned c = (kg - p * gpp) * 16u;
+  const int4 v = *reinterpret_cast<const int4*>(xp + act_offset((int64_t)(img * hw + p), (int)c, (int)cp));
+  *reinterpret_cast<int4*>(yp + act_offset((int64_t)img, (int)(kg * 16u), (int)(hw * cp))) = v;
+}
+
 }  // namespace cvmhip
 
 using namespace cvmhip;
@@ -255,6 +271,18 @@ using namespace cvmhip;
 extern "C" {
 
 int cvmhip_pad_channels(int channels) { return pad_channels(channels); }
+
+int cvmhip_flatten_act_i8(const void* xp, void* yp, int n, int c, int hw, void* stream) {
+  if (!xp || !yp || n < 1 || c < 32 || (c & 31) || hw < 1 || (int64_t)hw * c > (1 << 28) || (int64_t)n * hw * c > (1ll << 31) - 4096 ||
+      (((uintptr_t)xp | (uintptr_t)yp) & 15))
+    return arg_error("flatten_act_i8 (channels a multiple of 32, 16-byte aligned tensors, less than 2 GiB)");
+  hipStream_t s = as_stream(stream);
+  const unsigned granules = (unsigned)((int64_t)n * hw * (c >> 4));
+  KernelTimer timer("k_flatten_act", 2.0 * (double)granules * 16.0, s);   // bytes in + out
+  k_flatten_act<<<(granules + 255) / 256, 256, 0, s>>>(reinterpret_cast<const int8_t*>(xp), reinterpret_cast<int8_t*>(yp), granules,
+                                                      (unsigned)n, (unsigned)hw, (unsigned)c);
+  return check_launch("flatten_act_i8");
+}
 
 int cvmhip_pack_nhwc_i8(const int32_t* x, void* xp, int n, int c, int hw, void* stream) {
   if (!x || !xp || n < 1 || c < 1 || hw < 1 || ((uintptr_t)xp & 3)) return arg_error("pack_nhwc_i8");

@@ -451,6 +451,7 @@ void HipGraphRuntime::ReadHooks() {
   hooks_.seq = env("CVM_HIP_SEQ") != "0";
   hooks_.seq_forced = env("CVM_HIP_SEQ") == "1";
   hooks_.seq_chains = env("CVM_HIP_SEQ_CHAIN") != "0";
+  hooks_.flat_dense = env("CVM_HIP_FLATDENSE") != "0";
   hooks_.dw_on_mfma = env("CVM_HIP_DW").rfind("v", 0) != 0;
   hooks_.pool_fuse = env("CVM_HIP_POOLFUSE") != "0";
   hooks_.head_pair = env("CVM_HIP_HEADPAIR") != "0";

@@ -103,6 +103,8 @@ struct PlanStep {
   std::shared_ptr<void> ws;       // CONV: workspace of a K-sliced launch (cvmhip_conv2d_i8_ws), or empty
   size_t ws_bytes = 0;
   bool dw_mfma = false;           // DWCONV through the implicit-GEMM kernel (filter packed as diagonal blocks)
+  bool flat = false;              // CONV that is a dense layer over a whole map (kh x kw == h x w): the map is flattened into `aux`
+                                  // first (cvmhip_flatten_act_i8) and the layer runs as a 1x1 convolution over h * w * c channels
   bool pool2 = false;             // CONV also takes the 2x2 stride-2 max_pool2d that follows it (cvmhip_conv2d_pool2_i8); dst is the pooled tensor
   bool pool3 = false;             // CONV (stem) also takes the 3x3 stride-2 padding-1 max_pool2d that follows it (cvmhip_conv2d_stem_pool3_i8);
                                   // dst is the pooled tensor, oh x ow its extent
@@ -171,7 +173,10 @@ class HipGraphRuntime {
         for (const SeqRun& q : seqs_) inside = inside || (r.first >= q.first && r.last <= q.last);
       if (!inside) grouped += r.nlayers - 1;
     }
-    if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq - (fused_ ? grouped : 0);
+    int extra = 0;   // steps of two launches: a dense layer over a whole map behind the copy that flattens the map
+    if (fused_)
+      for (const PlanStep& st : plan_) extra += st.flat ? 1 : 0;
+    if (launches) *launches = static_cast<int>(NumSteps()) - lay + seq - (fused_ ? grouped : 0) + extra;
     if (sequences) *sequences = seq;
     if (layers) *layers = lay;
   }
@@ -231,6 +236,7 @@ class HipGraphRuntime {
     int conv_kernel = 0, wave_cfg = -1, tile_wm = 0, tile_wn = 0;
     // layer-sequence launches: CVM_HIP_SEQ_SPIN=<polls> patience of a wait at a layer boundary (0: every wait gives up at once)
     int seq_spin = 2000000;
+    bool flat_dense = true;   // CVM_HIP_FLATDENSE=0: a dense layer over a whole map gathers its operand from the map as it lies
     bool seq_chains = true;   // CVM_HIP_SEQ_CHAIN=0: no 1x1 layers chained behind the layer that feeds them (cvmhip_conv_seq_link)
     std::vector<std::pair<int, int>> seq_layer_cfg;   // CVM_HIP_SEQCFG: (layer of a sequence, configuration)
   };

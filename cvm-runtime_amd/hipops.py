@@ -376,6 +376,13 @@ def pack_act_i8(x):
     return xp
 
 
+def flatten_act_i8(xp, n, c, hw):
+    """int8 act tensor of n images x hw pixels x c channels -> act tensor of n pixels x hw * c channels (cvmhip_flatten_act_i8)"""
+    yp = _act_buffer(n, hw * c, xp.device)
+    check(lib().cvmhip_flatten_act_i8(_vp(xp), _vp(yp), n, c, hw, _stream()))
+    return yp
+
+
 def unpack_act_i8(xp, n, c, h, w):
     x = torch.empty((n, c, h, w), dtype=torch.int32, device=xp.device)
     check(lib().cvmhip_unpack_nhwc_i8(_vp(xp), _ptr(x), n, c, h * w, _stream()))

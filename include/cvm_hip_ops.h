@@ -448,6 +448,14 @@ int cvmhip_pack_depthwise_weights_mfma(const int32_t* w, void* wp, int c, int kh
 int cvmhip_depthwise_conv2d_mfma_i8(const void* xp, const void* wp, const int32_t* bias, const cvmhip_chain* chain,
                                     void* out, int out_is_i8, int n, int c, int h, int wd, int kh, int kw,
                                     int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void* stream);
+/* flatten (elemwise.cc:64-76: a copy, the rows of an image one behind the other) of an int8 act tensor of n images,
+ * hw pixels each, c channels (a multiple of 32), in the order a dense layer computed as a convolution over the whole
+ * map takes its K axis: yp is the act tensor of n pixels (one per image) x hw * c channels, channel p * c + ch = channel
+ * ch of pixel p (cvmhip_packed_act_bytes(n, hw * c) bytes, rows n .. 31 of its pixel block untouched).  With it that
+ * dense layer is a 1x1 convolution over hw * c channels whose operand blocks are contiguous KiB: cvmhip_conv2d_i8_ws
+ * with the filter packed for (ic = c, kh x kw = the map) and the geometry (ic = hw * c, 1 x 1 map, 1 x 1 filter) --
+ * the packed filter is byte for byte the same for both readings. */
+int cvmhip_flatten_act_i8(const void* xp, void* yp, int n, int c, int hw, void* stream);
 /* out = chain(a + b) on int8 act tensors of identical geometry */
 int cvmhip_add_i8(const void* a, const void* b, const cvmhip_chain* chain, void* out, int out_is_i8,
                   int n, int c, int hw, void* stream);

@@ -1060,3 +1060,50 @@ def test_dense_int32_kernel_blocks_of_rows(dev):
         y = hipops.dense(T(x, dev), T(w, dev), T(b, dev), operand_bits=32)
         torch.cuda.synchronize()
         eq(y.cpu().numpy(), ref, "dense int32 m=%d" % m)
+
+
+@pytest.mark.parametrize("case", [(8, 256, 6, 72), (5, 64, 12, 40), (16, 512, 7, 96)])
+def test_dense_over_a_whole_map_through_the_flattened_copy(case, dev):
+    """flatten -> dense over a 4-D tensor of 8192 or more values per image at a batch of four or more: the map is copied
+    once into a tensor whose K chunks are contiguous (cvmhip_flatten_act_i8) and the layer runs as a 1x1 convolution
+    over h * w * c channels.  Same bytes as with CVM_HIP_FLATDENSE=0 (the operand gathered from the map as it lies),
+    as node by node, and as the oracle; the run has one launch more."""
+    n, c, hw, units = case
+    g = graphgen.GraphBuilder("flat-dense-%dx%dx%d" % (n, c, hw))
+    x = g.var("data", (n, 3, hw, hw), 8)
+    y = g.conv_relu_q(x, c, 3, 1, 1)
+    y = g.conv_relu_q(y, c, 1)
+    d, k = g.dense(g.flatten(y), units)
+    d = g.rshift(g.relu(d), graphgen.shift_for(k))
+    e, _ = g.dense(d, 10)
+    js, pb = g.build([e])
+    xv = synth.tensor("flat-dense", "data", (n, 3, hw, hw), -127, 127)
+    ref = og.run_graph(js, graphgen.load_params(pb), xv)
+    want = np.concatenate([r.ravel() for r in ref])
+    launches = {}
+    for flat, fuse in (("1", "1"), ("0", "1"), ("1", "0")):
+        os.environ["CVM_HIP_FLATDENSE"] = flat
+        os.environ["CVM_HIP_FUSE"] = fuse
+        try:
+            m = runtime.HipModel(js, pb)
+            out = m.inference(xv.astype(np.int8).tobytes())
+            tsize = runtime.CVMAPIGetOutputTypeSize(m.net)
+            launches[(flat, fuse)] = m.launch_counts()[0]
+            m.close()
+        finally:
+            os.environ.pop("CVM_HIP_FLATDENSE", None)
+            os.environ.pop("CVM_HIP_FUSE", None)
+        got = np.frombuffer(out, np.int32 if tsize == 4 else np.int8).astype(np.int32)
+        assert np.array_equal(got, want), "flattened copy %s, planner %s" % (flat, fuse)
+    assert launches[("1", "1")] == launches[("0", "1")] + 1, launches
+
+
+def test_flatten_act_i8(dev):
+    """the copy itself: channel p * c + ch of image i in the result is channel ch of pixel p of image i"""
+    n, c, hw = 5, 96, 11
+    x = synth.tensor("flatten-act", "x", (n, c, hw, 1), -128, 127)
+    yp = hipops.flatten_act_i8(hipops.pack_act_i8(T(x, dev)), n, c, hw)
+    got = act_to_nchw(yp, n, hw * c, 1, 1).reshape(n, hw, c)          # (image, pixel, channel)
+    eq(got, x.reshape(n, c, hw).transpose(0, 2, 1), "flatten_act_i8")
+    with pytest.raises(CvmHipError):
+        hipops.flatten_act_i8(hipops.pack_act_i8(T(x[:, :40], dev)), n, 40, hw)   # channels not a multiple of 32
