@@ -26,8 +26,8 @@ PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 # The third field is the first 16 hex digits of the SHA-256 of the kernels' source file as it was when the counters were
 # read: a figure is only reported while that file is unchanged, otherwise `traffic` is null (measured figures go stale).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("resnet50", "k_conv_seq", 16): (548.6e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt", "unrecorded"),
-    ("vgg16", "k_conv_big", 16): (33.8e6, "profiles/k_conv_big_vgg16_b16_traffic.txt", "unrecorded"),
+    ("resnet50", "k_conv_seq", 16): (530.9e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt", "3b1aeeee3a8e8c86"),
+    ("vgg16", "k_conv_big", 16): (28.7e6, "profiles/k_conv_big_vgg16_b16_traffic.txt", "3b1aeeee3a8e8c86"),
 }
 KERNEL_SOURCE = os.path.join(ROOT, "cvm-runtime_amd", "csrc", "conv_mfma.hip")
 
@@ -251,6 +251,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vgg", action="store_true",
                     help="skip the VGG-16 batch-16 figures that the headline configuration reports beside its own")
+    ap.add_argument("--no-batch1", action="store_true",
+                    help="skip the batch-1 figures of the same graph (keeps a profiler's kernel statistics to the timed model)")
     ap.add_argument("--no-two-models", action="store_true",
                     help="skip the side measurement with two models in flight (keeps a profiler's kernel statistics to one model)")
     ap.add_argument("--suite", choices=("model", "ops"), default="model",
@@ -435,7 +437,7 @@ def main():
           "resnet20": lambda: graphgen.resnet20_cifar(1), "ssd512": graphgen.ssd_mobilenet}[args.workload]
     g1, h1 = b1()
     js1, pb1 = g1.build(h1)
-    if args.batch != 1:
+    if args.batch != 1 and not args.no_batch1:
         m1 = runtime.HipModel(js1, pb1)
         m1.set_input(x[:1].tobytes())
         m1.time_run(max(args.warmup, 1))

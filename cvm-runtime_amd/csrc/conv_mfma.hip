@@ -63,7 +63,9 @@ constexpr int SEQ_MAX_STAGES = 2;   // stages per chain of a layer inside a laye
 // once or twice, straight from memory, and code for stages that never occur is fetched like any other.
 template <int N, int MAXST = 4, bool MUL = true>
 __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N], const unsigned flags = 0u) {
-  const unsigned f = (unsigned)__builtin_amdgcn_readfirstlane((int)((flags & 0x80000000u) ? flags : chain_flags_of(c)));
+  unsigned f = flags;
+  if (!(__builtin_amdgcn_readfirstlane((int)flags) & 0x80000000u)) f = chain_flags_of(c);   // (a branch: the forty instructions are skipped)
+  f = (unsigned)__builtin_amdgcn_readfirstlane((int)f);
 #pragma unroll
   for (int t = 0; t < MAXST; ++t) {
     if (f & (1u << (5 * t))) {
@@ -704,7 +706,6 @@ struct LayerGate {
   unsigned* error;
   int spin_limit;
   unsigned* seen;      // LDS word of the workgroup (or of its half): the highest target its first wavefront has seen reached
-  int role;            // -1: the wavefront with index 0 in the tile polls the counter, the others watch `seen`; 0: this one polls; 1: watches
 };
 __device__ __forceinline__ void gate_poll(const LayerGate& gate) {
   if (!gate.counter) return;
@@ -939,7 +940,7 @@ template <int TM, int TN, int KSPLIT, int NW, int D, int OUT, int MODE, bool SLI
 __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, const int8_t* __restrict__ wf, void* __restrict__ out,
                                                const ConvGeom& g, const Epilogue& ep, int pid, const int tid,
                                                int* __restrict__ sPart, int* __restrict__ sBias, const int p_begin = 0,
-                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0, nullptr, -1},
+                                               const int p_end = 0, const LayerGate gate = LayerGate{nullptr, 0, nullptr, 0, nullptr},
                                                unsigned long long* tr = nullptr, const SeqLayer* tailB = nullptr,
                                                const SeqLayer* tailC = nullptr, const ChainLds* chain_lds = nullptr) {
   CVM_SEQ_STAMP(0, tid);
@@ -1101,7 +1102,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // COH: called once, between the filter requests and the activation requests of the first batch
   auto pass_gate = [&]() __attribute__((always_inline)) {
     if constexpr (COH) {
-      gate_wait(gate, gate.role < 0 ? wave : gate.role);
+      gate_wait(gate, wave);
       CVM_SEQ_STAMP(1, tid);
     }
   };
@@ -1669,7 +1670,8 @@ k_stem_pool(const int8_t* __restrict__ xs, const int8_t* __restrict__ wf, int8_t
 }
 
 // ---------------------------------------------------------------- layer-sequence kernel
-// A run of convolutions of one graph in ONE launch, for batches that divide over the chip's 8 XCDs.
+// A run of convolutions of one graph in ONE launch.  The images are dealt to 8, 4, 2 or 1 of the chip's 8 XCDs (the
+// largest of these that divides the batch; workgroups on the other XCDs leave at once).
 // Images are independent, so XCD x computes every layer for its own share of the images (pixel range
 // [x * px_per_share, (x + 1) * px_per_share) of every tensor) and never reads what another XCD wrote.  The
 // 32 compute units of an XCD share one L2, which makes a layer boundary cheap and local:
@@ -1684,6 +1686,8 @@ k_stem_pool(const int8_t* __restrict__ xs, const int8_t* __restrict__ wf, int8_t
 // Every wait is bounded: when a counter does not arrive within spin_limit polls the workgroup raises
 // the error flag, which makes every workgroup leave at its next boundary; the host then falls back to one
 // launch per layer.
+// A step between two boundaries is one layer, or a layer with the 1x1 layers chained behind it (SeqLayer::chain), or
+// two layers that have nothing to do with one another (SeqLayer::join_next); conv_seq_link decides on the host.
 template <int TM, int TN, int KSPLIT, int NW, int D, int MODE>
 __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* wf, void* out, const ConvGeom& g, const Epilogue& ep,
                                                 int ntiles, int dead_tile, int rank, int tid, int* sPart, int* sBias, int p_begin,
@@ -1695,7 +1699,7 @@ __device__ __forceinline__ void seq_layer_tiles(const int8_t* xp, const int8_t* 
     const int t = base + half * SEQ_WG_PER_SHARE + rank;   // the first 32 tiles go to 32 different compute units
     conv_wave_tile<TM, TN, KSPLIT, NW, D, OUT_I8_ACT, MODE, false, true>(
         xp, wf, out, g, ep, t < ntiles ? t : dead_tile, htid, sPart + half * 16384, sBias + half * 256, p_begin, p_end,
-        base == 0 ? LayerGate{gate.counter, gate.target, gate.error, gate.spin_limit, gate.seen + half, -1} : LayerGate{nullptr, 0, nullptr, 0, nullptr, -1},
+        base == 0 ? LayerGate{gate.counter, gate.target, gate.error, gate.spin_limit, gate.seen + half} : LayerGate{nullptr, 0, nullptr, 0, nullptr},
         base == 0 ? tr : nullptr);
     if (KSPLIT > 1) __syncthreads();   // the next tile reuses the LDS of the partial sums
   }
@@ -1730,7 +1734,7 @@ __device__ __forceinline__ void seq_chain_tiles(const SeqLayer& A, int ntiles, i
   gate_wait(gate, wave);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  const LayerGate none = {nullptr, 0, nullptr, 0, nullptr, -1};
+  const LayerGate none = {nullptr, 0, nullptr, 0, nullptr};
   for (int base = 0; base < ntiles; base += 8 * SEQ_WG_PER_SHARE) {
     const int t = base + wave * SEQ_WG_PER_SHARE + rank;
     if (t >= ntiles) continue;
@@ -1819,7 +1823,7 @@ k_conv_seq(const SeqLayer* __restrict__ layers_generic, int nlayers, unsigned* _
     const int dead_tile = g.octiles * (L.ptiles + 1);   // a tile past the share: computes, stores nothing
     const int cfg = kernel / 3, mode = kernel - cfg * 3;
     // this step may read what the previous one wrote once all 32 workgroups of the XCD have counted themselves out of it
-    const LayerGate gate = {step > 0 && !joined ? my + SEQ_BAR : nullptr, (unsigned)step * SEQ_WG_PER_SHARE, error, spin_limit, s_seen, -1};
+    const LayerGate gate = {step > 0 && !joined ? my + SEQ_BAR : nullptr, (unsigned)step * SEQ_WG_PER_SHARE, error, spin_limit, s_seen};
 #ifdef CVM_SEQ_STAMPS
     unsigned long long* tr = stamps && l < stamp_layers ? stamps + ((size_t)((int)xcc * SEQ_WG_PER_SHARE + rank) * stamp_layers + l) * 8 : nullptr;
     if (tr && tid == 0) tr[7] = __builtin_amdgcn_s_memtime();
