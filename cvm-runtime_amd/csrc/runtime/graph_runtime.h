@@ -298,6 +298,7 @@ class HipGraphRuntime {
   uint32_t* seq_error_host_ = nullptr;  // pinned copy of the error word
   bool use_seq_ = false;
   bool seq_counted_ = false;            // this model is counted among the models with sequence launches
+  bool seq_calibration_pending_ = false;   // loaded next to another such model: the two launch forms are compared at the first run alone
   bool seq_ran_ = false;                // a sequence launch was issued since the last check
 };
 

@@ -283,3 +283,36 @@ def test_two_models_with_sequences_on_two_threads(dev):
         assert len(results[i]) == 20
         for out in results[i]:
             assert np.array_equal(np.frombuffer(out, np.int32), want)
+
+
+def test_while_two_models_with_sequences_are_alive_both_use_one_launch_per_layer(dev):
+    """Sequence launches are for a model that has the chip to itself.  A model loaded next to one that uses them does not
+    compare the two launch forms then (both would be timed as one launch per layer) but stays counted, so that neither
+    of the two issues a sequence launch; when the other one is gone it makes the comparison at its next run.  Results
+    are the same bytes throughout."""
+    g, heads = graphgen.resnet50(8, width=16, size=64, classes=50, config_id="seq-policy")
+    js, pb = g.build(heads)
+    x = synth.tensor("seq-policy", "data", (8, 3, 64, 64), -127, 127).astype(np.int8)
+    want = _run(js, pb, x, "0")
+    os.environ["CVM_HIP_SEQ"] = "1"
+    try:
+        first = runtime.HipModel(js, pb)
+    finally:
+        os.environ.pop("CVM_HIP_SEQ", None)
+    try:
+        assert first.launch_counts()[1] >= 1
+        second = runtime.HipModel(js, pb)          # no switch: it would measure, were it alone
+        try:
+            assert first.launch_counts()[1] == 0 and second.launch_counts()[1] == 0
+            for m in (first, second, first, second):
+                assert np.array_equal(np.frombuffer(m.inference(x.tobytes()), np.int32), want)
+            assert first.launch_counts()[1] == 0 and second.launch_counts()[1] == 0
+        finally:
+            first.close()
+            first = None
+        for _ in range(3):                         # alone now: the comparison happens inside the first of these runs
+            assert np.array_equal(np.frombuffer(second.inference(x.tobytes()), np.int32), want)
+        second.close()
+    finally:
+        if first is not None:
+            first.close()
