@@ -92,6 +92,38 @@ __device__ __forceinline__ void run_chain(const DevChain& c, int32_t (&v)[N], co
   }
 }
 
+// The same chain read from the structure itself, for kernels that receive it as a kernel argument (one launch per
+// layer): every field is then a scalar already and the tests below are scalar branches as they stand, while the flag
+// word, its readfirstlane and its bit tests only add to such a kernel (ResNet-50 batch 1 0.2607 -> 0.2562 ms, batch
+// 16 with one launch per layer 0.421 -> 0.412 ms; with the bias added in the epilogue as well, 0.2485 and 0.393 ms).
+template <int N>
+__device__ __forceinline__ void run_chain_plain(const DevChain& c, int32_t (&v)[N]) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if (t < c.count) {
+      const DevStage q = c.st[t];
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = clamp3(v[e], q.lo, q.hi);
+      if (q.mul != 1) {   // a multiplication stage (rare)
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = wmul(v[e], q.mul);
+      }
+      if (q.s1 != 0) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s1;
+      }
+      if (q.add != 0) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = wadd(v[e], q.add);
+      }
+      if (q.s2 != 0) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = v[e] >> q.s2;
+      }
+    }
+  }
+}
+
 // low bytes of four values -> one dword
 __device__ __forceinline__ uint32_t pack_bytes(int32_t a, int32_t b, int32_t c, int32_t d) {
   const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
@@ -217,8 +249,9 @@ __device__ __forceinline__ void load_residual(uint32_t (&rp)[NG], int u0, int ch
 
 // RANGE: only the pixels [p_begin, p_end) are stored (one share of a layer inside the layer-sequence
 // kernel); the stores are then ordinary ones, because the next layer reads the tensor from this L2.
-// BIASED: the accumulators already hold the bias (the wavefront kernel starts them from it), sBias is not read.
-template <int TN, int NG, int OUT, bool RANGE = false, bool POOLR = false, bool BIASED = false>
+// BIASED: the accumulators already hold the bias (the layer-sequence kernel starts them from it), sBias is not read.
+// FLAGS: the chains are decoded from their flag words (run_chain) instead of from their fields (run_chain_plain).
+template <int TN, int NG, int OUT, bool RANGE = false, bool POOLR = false, bool BIASED = false, bool FLAGS = true>
 __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, const int* sBias, int ch_wave, int oc0,
                                               int px_wave, int lane, void* out, const ConvGeom& g, const Epilogue& ep,
                                               uint32_t (&rp)[NG], int p_begin = 0, int p_end = 0) {
@@ -270,7 +303,8 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
           const int32_t ab = a > b ? a : b, cd = c > d ? c : d;
           red[qe] = ab > cd ? ab : cd;
         }
-        run_chain(ep.chain, red, ep.chain_flags);
+        if constexpr (FLAGS) run_chain(ep.chain, red, ep.chain_flags);
+        else run_chain_plain(ep.chain, red);
         uint32_t a = pack_bytes(red[0], red[1], red[2], red[3]), b = pack_bytes(red[4], red[5], red[6], red[7]),
                  c = pack_bytes(red[8], red[9], red[10], red[11]), d = pack_bytes(red[12], red[13], red[14], red[15]);
         half_swap(a, c);
@@ -291,7 +325,8 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
   // one copy of each step, the residual part an update in place under a uniform condition (two
   // alternative paths that meet again cost a register-to-register copy of every value)
   constexpr int MAXST = RANGE ? SEQ_MAX_STAGES : 4;   // RANGE: a layer of a sequence (conv_seq_layer admits short chains only)
-  run_chain<NG * 4, MAXST, !RANGE>(ep.chain, val, ep.chain_flags);
+  if constexpr (FLAGS) run_chain<NG * 4, MAXST, !RANGE>(ep.chain, val, ep.chain_flags);
+  else run_chain_plain(ep.chain, val);
   if (ep.residual) {   // rp holds what load_residual fetched
     if (whole) {
 #pragma unroll
@@ -304,7 +339,8 @@ __device__ __forceinline__ void finish_groups(int32_t (&val)[NG * 4], int u0, co
     }
 #pragma unroll
     for (int e = 0; e < NG * 4; ++e) val[e] = wadd(val[e], (int32_t)(int8_t)(rp[e >> 2] >> (8 * (e & 3))));
-    run_chain<NG * 4, MAXST, !RANGE>(ep.chain2, val, ep.chain2_flags);
+    if constexpr (FLAGS) run_chain<NG * 4, MAXST, !RANGE>(ep.chain2, val, ep.chain2_flags);
+    else run_chain_plain(ep.chain2, val);
   }
 
   if (OUT == OUT_I32_NCHW) {
@@ -1055,9 +1091,11 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
 #pragma unroll
   for (int j = 0; j < TN; ++j) tapoff[j] = kOutsideBuffer;
 
-  // The accumulators start from the bias: the addend of a tile's first MFMA is the bias of its 32 output channels as the
+  // (COH) The accumulators start from the bias: the addend of a tile's first MFMA is the bias of its 32 output channels as the
   // accumulator holds them (element e of a lane: channel (e / 4) * 8 + (lane / 32) * 4 + e % 4 of the tile), so the
-  // epilogue neither reads nor adds it.  After a K split one wavefront of each tile set brings it in (the one whose
+  // epilogue neither reads nor adds it.  A launch of its own keeps the older form -- one word per lane requested
+  // behind the first operand batch, staged in LDS after the K loop, added in the epilogue: there the four 16-byte
+  // requests per 32 channels in front of the first operand request cost more than the epilogue's additions.  After a K split one wavefront of each tile set brings it in (the one whose
   // register groups are not permuted, kw_ == 0); the sums of the others start from zero.  The four 16-byte loads per
   // 32 channels are the first requests of the tile and hit two addresses per wavefront each.
   v16i binit[TM];
@@ -1065,7 +1103,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < TM; ++i) binit[i] = zero16;
-    if (ep.bias && (KSPLIT == 1 || kw_ == 0)) {
+    if (COH && ep.bias && (KSPLIT == 1 || kw_ == 0)) {
       const int OC = g.OC;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -1223,6 +1261,12 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   // front of the first operand request).
   if (!COH && ep.residual) load_residual<TN, NU, COH>(rp, kw_ * NU, 0, oc0, px0 + pw_ * TN * 32, lane, g, ep);
   regs_t R0 = fetch(COH);
+  int bias_mine = 0;   // (!COH) this lane's word of the bias: without a K split every wavefront stages a copy of its own
+  const int bias_lane = KSPLIT == 1 ? lane : tid;
+  int* bias_lds = KSPLIT == 1 ? sBias + wave * BM : sBias;
+  if constexpr (!COH) {
+    if (bias_lane < BM) bias_mine = (ep.bias && oc0 + bias_lane < g.OC) ? ep.bias[oc0 + bias_lane] : 0;
+  }
   // (Without a K split no wavefront needs anything from another one and the tile has no barrier at all: the
   // wavefronts of a workgroup drift apart, and one's epilogue runs under another's operand requests.)
 
@@ -1254,6 +1298,9 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
     }
   }
   CVM_SEQ_STAMP(3, acc[0][0][0]);
+  if constexpr (!COH) {
+    if (bias_lane < BM) bias_lds[bias_lane] = bias_mine;
+  }
   if constexpr (TAIL >= 0) {
     static_assert(TAIL < 0 || (KSPLIT == 1 && TN == 1 && COH && OUT == OUT_I8_ACT), "a chain starts from an unsplit tile of one pixel block");
     conv_chain_tail<TM, TAIL>(acc, ep, out, *tailB, tailC, *chain_lds, px0 + pw_ * 32, lane, p_begin, p_end);
@@ -1288,6 +1335,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
       val[m * 4] = sum.x; val[m * 4 + 1] = sum.y; val[m * 4 + 2] = sum.z; val[m * 4 + 3] = sum.w;
     }
   } else {
+    if constexpr (!COH) __builtin_amdgcn_wave_barrier();   // bias staged: written and read by this wavefront only, and LDS serves a wavefront in order
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1298,7 +1346,7 @@ __device__ __forceinline__ void conv_wave_tile(const int8_t* __restrict__ xp, co
   CVM_SEQ_STAMP(4, val[0]);
   void* dst = out;
   if (SLICES && g.kslices > 1) dst = reinterpret_cast<int32_t*>(out) + (int64_t)kslice * g.slice_stride;   // int32 output only (host)
-  finish_groups<TN, NU, OUT, COH, POOLR, true>(val, kw_ * NU, nullptr, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
+  finish_groups<TN, NU, OUT, COH, POOLR, COH, COH>(val, kw_ * NU, COH ? nullptr : bias_lds, 0, oc0, px0 + pw_ * TN * 32, lane, dst, g, ep, rp, p_begin, p_end);
   CVM_SEQ_STAMP(5, tid);
 }
 
