@@ -872,9 +872,10 @@ void HipGraphRuntime::CopyOutputTo(int index, int32_t* host) {
   CVM_VERIFY(index >= 0 && static_cast<size_t>(index) < outputs_.size());
   const uint32_t eid = entry_id(outputs_[index]);
   HipCheck(cvmhip_copy_d2h(host, entry_ptr_[eid], static_cast<size_t>(shape_size(shape_[eid])) * 4, stream_), "copy output");
+  const bool status = RequestSequenceStatus();
   HipCheck(cvmhip_stream_sync(stream_), "copy output");
   if (seq_ran_) {
-    CheckSequences();
+    CheckSequences(status);
     if (!use_seq_) CopyOutputTo(index, host);   // the run was repeated with one launch per layer
   }
 }
@@ -882,12 +883,23 @@ void HipGraphRuntime::CopyOutputTo(int index, int32_t* host) {
 // A layer-sequence launch whose bounded waits ran out (its workgroups were not all resident at once) leaves its error
 // word set and its results undefined.  Seen after a synchronisation: sequences are switched off for this model for
 // good and the run is repeated with one launch per layer.
-void HipGraphRuntime::CheckSequences() {
+// The status word travels behind whatever the caller copies back, so that one synchronisation serves both (a second
+// copy and wait of its own cost every CVMAPIInference call a round trip to the device).
+bool HipGraphRuntime::RequestSequenceStatus() {
+  if (!seq_ran_ || !use_seq_ || !seq_sync_) return false;
+  const size_t words = cvmhip_conv_seq_sync_bytes() / 4;
+  HipCheck(cvmhip_copy_d2h(seq_error_host_, static_cast<uint32_t*>(seq_sync_) + (words - 64), 4, stream_), "sequence status");
+  return true;
+}
+
+void HipGraphRuntime::CheckSequences(bool requested) {
   seq_ran_ = false;
   if (!use_seq_ || !seq_sync_) return;
   const size_t words = cvmhip_conv_seq_sync_bytes() / 4;
-  HipCheck(cvmhip_copy_d2h(seq_error_host_, static_cast<uint32_t*>(seq_sync_) + (words - 64), 4, stream_), "sequence status");
-  HipCheck(cvmhip_stream_sync(stream_), "sequence status");
+  if (!requested) {
+    HipCheck(cvmhip_copy_d2h(seq_error_host_, static_cast<uint32_t*>(seq_sync_) + (words - 64), 4, stream_), "sequence status");
+    HipCheck(cvmhip_stream_sync(stream_), "sequence status");
+  }
   if (*seq_error_host_ == 0) return;
   std::cerr << "cvm hip: a layer-sequence launch could not keep all its workgroups resident; using one launch per layer\n";
   DropSequences();
@@ -914,9 +926,10 @@ const std::vector<const int32_t*>& HipGraphRuntime::FetchOutputs() {
     HipCheck(cvmhip_copy_d2h(const_cast<int32_t*>(out_host_[k]), entry_ptr_[eid], static_cast<size_t>(shape_size(shape_[eid])) * 4,
                              stream_), "copy output");
   }
+  const bool status = RequestSequenceStatus();
   HipCheck(cvmhip_stream_sync(stream_), "copy output");
   if (seq_ran_) {
-    CheckSequences();
+    CheckSequences(status);
     if (!use_seq_) return FetchOutputs();   // the run was repeated with one launch per layer
   }
   return out_host_;
@@ -928,8 +941,9 @@ int32_t* HipGraphRuntime::DataDevicePtr() {
 }
 
 void HipGraphRuntime::SyncStream() {
+  const bool status = RequestSequenceStatus();
   HipCheck(cvmhip_stream_sync(stream_), "synchronise");
-  if (seq_ran_) CheckSequences();
+  if (seq_ran_) CheckSequences(status);
 }
 
 const Shape& HipGraphRuntime::InputShape() const {

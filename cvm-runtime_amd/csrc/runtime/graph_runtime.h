@@ -291,7 +291,8 @@ class HipGraphRuntime {
   bool SeqNow() const;                  // does the next run use sequence launches?
   bool seq_mode_ = false;               // what the launches being issued (and the captured graph) use
   void DropSequences();                 // sequence launches are off for good for this model
-  void CheckSequences();                // after a synchronisation: did a sequence launch give up?
+  bool RequestSequenceStatus();         // before a synchronisation: the status word of the sequence launches rides along (true when requested)
+  void CheckSequences(bool requested);  // after a synchronisation: did a sequence launch give up?  (fetches the word itself unless requested)
   std::vector<SeqRun> seqs_;
   std::vector<int> seq_at_;             // per plan_ index: the run that starts there, or -1
   void* seq_sync_ = nullptr;            // counters and error word of the sequence launches (device)
