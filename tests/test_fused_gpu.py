@@ -190,6 +190,8 @@ KSLICE_CASES = [
     # n, ic, h, w, oc, k   (output 1x1: a dense layer over the flattened map, or a plain dense layer)
     (16, 512, 7, 7, 256, 7),      # the shape of VGG-16's first dense layer, fewer units
     (5, 8192, 1, 1, 100, 1),      # plain dense, ragged unit count, K exactly at the threshold
+    (32, 8192, 1, 1, 96, 1),      # 32 rows: the one-pixel-block tile (at most 32 pixels, 1x1) completely full
+    (16, 12544, 1, 1, 520, 1),    # 392 chunks of K over four slices and four wavefronts each, 17 channel tiles
     (33, 1024, 3, 3, 64, 3),      # 33 rows: second half of the pixel tile partly empty
     (1, 9216, 1, 1, 8192, 1),     # more than 256 tiles: not sliced, same answer
     (2, 4096, 1, 1, 64, 1),       # K below the threshold: no workspace
